@@ -1,0 +1,152 @@
+/*
+ * tqamd -- C ABI of the MI355X (gfx950) TurboQuant V3 KV-cache codec.
+ *
+ * Plain pointers and sizes only.  Every entry point returns an int status:
+ *   0            success
+ *   < 0          argument error (TQ_ERR_*), nothing was launched
+ *   > 0          a hipError_t reported by the HIP runtime
+ * No entry point allocates or frees device memory, synchronises the device or
+ * keeps state between calls; work is enqueued on the caller's stream.
+ *
+ * Each declaration cites the line range of the upstream Python reference
+ * (tonbistudio/turboquant-pytorch, turboquant/...) whose behaviour it replaces.
+ */
+#ifndef TQAMD_H
+#define TQAMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TQ_ABI_VERSION 1
+
+/* element types of K/V tensors */
+enum { TQ_F32 = 0, TQ_F16 = 1, TQ_BF16 = 2 };
+
+enum {
+    TQ_OK = 0,
+    TQ_ERR_NULL = -1,        /* a required pointer is NULL */
+    TQ_ERR_BITS = -2,        /* bits outside 1..8 */
+    TQ_ERR_HEAD_DIM = -3,    /* head_dim the kernels do not support (only 128) */
+    TQ_ERR_DTYPE = -4,       /* unknown element type */
+    TQ_ERR_SIZE = -5,        /* negative / inconsistent size, stride or buffer too small */
+    TQ_ERR_CODEBOOK = -6,    /* centroids not finite and strictly ascending */
+    TQ_ERR_TABLE = -7,       /* table blob malformed (bad magic / version) */
+    TQ_ERR_ALIGN = -8,       /* pointer or stride not aligned as required */
+    TQ_ERR_NO_DEVICE = -9    /* no usable HIP device */
+};
+
+int tq_abi_version(void);
+const char *tq_status_string(int status);
+
+/* Number of HIP devices visible (0 when there is none); never fails. */
+int tq_device_count(void);
+
+/*
+ * Packed bytes per vector: ceil(head_dim / floor(8 / bits)).
+ * Replaces the size arithmetic of MSECompressor.compress / memory_bytes,
+ * compressors_v3.py:64-69 and :111-112.  Returns TQ_ERR_BITS for bits outside 1..8.
+ */
+int tq_bytes_per_vector(int head_dim, int bits);
+
+/*
+ * Decision thresholds of the nearest-centroid rule.  thresholds[i] (i < levels-1) is the
+ * smallest float32 r for which |r - c[i+1]| < |r - c[i]| in float32 arithmetic, so that
+ *     argmin_j |r - c[j]|  (first minimum on ties)  ==  #{ i : r >= thresholds[i] }
+ * for every finite r.  Replaces the [N,D,L] broadcast + abs + argmin of
+ * compressors_v3.py:60-61.  Host only.
+ */
+int tq_decision_thresholds(const float *centroids, int levels, float *thresholds);
+
+/*
+ * Codec table: everything a compressor instance keeps on the device, baked on the host
+ * into one blob (rotation split into 16-bit MFMA operand tiles for both directions,
+ * quantiser lookup grid, decode tables).  Replaces the device state built by
+ * MSECompressor.__init__ (self.Pi, self.centroids), compressors_v3.py:37-43.
+ *
+ *   tq_table_bytes  size of the blob for (head_dim, bits); < 0 on error
+ *   tq_table_build  fill `table_host` (host memory, tq_table_bytes long) from
+ *                   Pi [head_dim*head_dim] row-major float32 (rotated = x @ Pi^T, as
+ *                   turboquant.py:18-33 returns it) and centroids [2^bits] ascending.
+ * The caller copies the blob to device memory (256-byte aligned) and passes that pointer
+ * to the compress / decompress entry points.
+ */
+long long tq_table_bytes(int head_dim, int bits);
+int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bits,
+                   void *table_host, size_t table_bytes);
+
+/*
+ * Host emulation of the kernels' quantiser lookup, bit for bit (same fused multiply-add,
+ * same grid): idx[i] = code chosen for unit-sphere coordinate r[i].  For tests of the
+ * table contents; the product path never calls it.
+ */
+int tq_table_quantize_host(const void *table_host, const float *r, long long n, uint8_t *idx);
+
+/*
+ * compress: K or V vectors -> packed codes + fp16 norms.
+ * Replaces MSECompressor.compress, compressors_v3.py:46-81.
+ *
+ *   states      device pointer, `dtype` elements; vector n (0 <= n < rows*tokens) starts at
+ *               element  (n / tokens) * row_stride + (n % tokens) * token_stride
+ *               and its head_dim (=128) elements are contiguous.  A contiguous
+ *               [B,H,S,D] tensor is rows=1, tokens=B*H*S, token_stride=128; a slice
+ *               [:, :, :s, :] of one is rows=B*H, tokens=s, row_stride=S*128.
+ *               Base address and strides must keep every vector 16-byte aligned.
+ *   table_dev   device copy of the blob from tq_table_build
+ *   idx_bytes   device, [rows*tokens, bytes_per_vector] uint8, contiguous
+ *   vec_norms   device, [rows*tokens] IEEE fp16 bit patterns (norm of the fp32-widened vector)
+ *   stream      hipStream_t (NULL = the default stream)
+ */
+int tq_compress(const void *states, int dtype, long long rows, long long tokens,
+                long long row_stride, long long token_stride,
+                const void *table_dev, int head_dim, int bits,
+                uint8_t *idx_bytes, uint16_t *vec_norms, void *stream);
+
+/*
+ * decompress: packed codes + fp16 norms -> vectors of `out_dtype`.
+ * Replaces MSECompressor.decompress, compressors_v3.py:84-105 (out_dtype = TQ_F32), and with
+ * TQ_F16 / TQ_BF16 the fused `.to(dtype)` + torch.cat into the full-length K/V buffer of
+ * TurboQuantV3.decompress_kv, compressors_v3.py:226-232: vector n is written at element
+ *   (n / tokens) * row_stride + (n % tokens) * token_stride   of `out`.
+ */
+int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms,
+                  long long rows, long long tokens,
+                  const void *table_dev, int head_dim, int bits,
+                  void *out, int out_dtype, long long row_stride, long long token_stride,
+                  void *stream);
+
+/*
+ * Batched forms: one launch for many (layer, tensor) jobs, each with its own table.
+ * Replaces the per-layer Python loop over TurboQuantV3.compress_kv / decompress_kv calls
+ * (callers: generation_test_v2.py:65-78,109,121,135; validate_v3.py:71-84).
+ * All jobs of one call share `bits` and `dtype` (group by width and launch once per group).
+ * `jobs_host` is read for validation and launch sizing; `jobs_dev` is a device copy of the
+ * same n_jobs records that the kernel reads -- the caller uploads it once and may reuse it
+ * for every call with the same buffers (nothing is allocated here).
+ */
+typedef struct tq_job {
+    const void *states;        /* compress: input vectors;   decompress: output vectors   */
+    uint8_t *idx_bytes;        /* compress: output;          decompress: input            */
+    uint16_t *vec_norms;       /* compress: output;          decompress: input            */
+    const void *table_dev;     /* this job's codec table                                 */
+    long long rows, tokens;    /* vector n = (n / tokens, n % tokens)                     */
+    long long row_stride;      /* elements, for `states`                                  */
+    long long token_stride;    /* elements, for `states`                                  */
+    int bits;                  /* 1..8, must match the table                              */
+    int dtype;                 /* element type of `states`                                */
+} tq_job;
+
+#define TQ_MAX_JOBS 4096
+
+int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
+                        int head_dim, void *stream);
+int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
+                          int head_dim, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TQAMD_H */

@@ -1,0 +1,280 @@
+"""
+TEST INFRASTRUCTURE ONLY -- not part of the product.
+
+CPU oracle for the TurboQuant V3 KV codec.  Two independent restatements of the
+upstream algorithm live here and check each other:
+
+  * `NumpyOracle`  -- the reference's op sequence in numpy float32, vectorised
+    the same way (norm, divide, [N,D]x[D,D] product, [N,D,L] |diff| argmin,
+    integer pack; unpack, gather, product, scale), chunked over N.
+    Follows turboquant/compressors_v3.py:46-81 (compress) and :84-105 (decompress).
+  * `COracle`      -- ctypes front end of oracle/tq_oracle.c (scalar loops, OpenMP
+    over vectors): fast enough for the large parity tests and the timed CPU
+    baseline of the benchmark.
+
+Only tests/, the repository's smoke check and the benchmark's cpu_baseline leg
+may import this module; the shipped package never does.
+
+What pins it: tests/golden/*.npz hold outputs of the real reference on seeded
+inputs (tests/golden/make_fixtures.py wrote them); tests/test_oracle.py checks
+both restatements against those, against each other, against exhaustive
+pack/unpack enumeration and brute-force nearest-centroid search.  Open at the
+last-bit level ("parity unpinned"): the summation order inside torch.norm and
+the BLAS sgemm the reference calls -- compared through the 1e-5 decision-boundary
+window, never bit for bit.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_BUILD = os.path.join(_HERE, "_build")
+_LIB = os.path.join(_BUILD, "libtq_oracle.so")
+
+
+# --------------------------------------------------------------------------
+# dtype helpers: fp16 / bf16 travel as uint16 bit patterns
+# --------------------------------------------------------------------------
+def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """Round-to-nearest-even float32 -> bfloat16 bit pattern (NaN kept quiet)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = np.isnan(x)
+    if nan.any():
+        rounded = np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), rounded)
+    return rounded
+
+
+def widen(x: np.ndarray, dtype: str) -> np.ndarray:
+    """Exact conversion of a tensor given as 'f32' array or 'f16'/'bf16' bit patterns to float32."""
+    if dtype == "f32":
+        return np.ascontiguousarray(x, dtype=np.float32)
+    if dtype == "f16":
+        return np.ascontiguousarray(x).view(np.float16).astype(np.float32)
+    if dtype == "bf16":
+        return bf16_bits_to_f32(np.ascontiguousarray(x))
+    raise ValueError(dtype)
+
+
+def indices_per_byte(bits: int) -> int:
+    return 8 // bits  # compressors_v3.py:64 (ZeroDivisionError above 8 bits, like the reference)
+
+
+def bytes_per_vector(D: int, bits: int) -> int:
+    ipb = indices_per_byte(bits)
+    return -(-D // ipb)
+
+
+# --------------------------------------------------------------------------
+# numpy restatement
+# --------------------------------------------------------------------------
+class NumpyOracle:
+    """The reference op sequence in float32 numpy.  `chunk` bounds the [n,D,L] temporary."""
+
+    def __init__(self, Pi: np.ndarray, centroids: np.ndarray, bits: int, chunk: int = 2048):
+        self.Pi = np.ascontiguousarray(Pi, dtype=np.float32)
+        self.centroids = np.ascontiguousarray(centroids, dtype=np.float32)
+        self.bits = int(bits)
+        self.D = self.Pi.shape[0]
+        self.chunk = chunk
+
+    def rotate(self, x: np.ndarray):
+        """-> (norms fp32 [N], rotated unit coordinates fp32 [N,D])   (:52-59)"""
+        flat = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.D)
+        norms = np.sqrt(np.sum(flat * flat, axis=-1, dtype=np.float32)).astype(np.float32)
+        unit = flat / (norms[:, None] + np.float32(1e-8))
+        return norms, unit @ self.Pi.T
+
+    def nearest(self, rotated: np.ndarray) -> np.ndarray:
+        """argmin_j |r - c_j|, first minimum wins  (:60-61)"""
+        out = np.empty(rotated.shape, dtype=np.uint8)
+        flat_r = rotated.reshape(-1)
+        flat_o = out.reshape(-1)
+        step = max(1, (self.chunk * self.D))
+        for s in range(0, flat_r.size, step):
+            d = np.abs(flat_r[s:s + step, None] - self.centroids[None, :])
+            flat_o[s:s + step] = np.argmin(d, axis=-1).astype(np.uint8)
+        return out
+
+    def pack(self, idx: np.ndarray) -> np.ndarray:
+        """[N,D] codes -> [N,G] bytes, MSB first, zero padded  (:64-74)"""
+        ipb = indices_per_byte(self.bits)
+        N, D = idx.shape
+        pad = (ipb - D % ipb) % ipb
+        wide = idx.astype(np.int64)
+        if pad:
+            wide = np.pad(wide, ((0, 0), (0, pad)))
+        weights = np.array([2 ** (self.bits * i) for i in range(ipb - 1, -1, -1)], dtype=np.int64)
+        return (wide.reshape(N, -1, ipb) * weights).sum(-1).astype(np.uint8)
+
+    def unpack(self, idx_bytes: np.ndarray) -> np.ndarray:
+        """[N,G] bytes -> [N,D] codes  (:93-101)"""
+        ipb = indices_per_byte(self.bits)
+        mask = (1 << self.bits) - 1
+        shifts = np.array([self.bits * i for i in range(ipb - 1, -1, -1)], dtype=np.int64)
+        idx = (idx_bytes.astype(np.int64)[:, :, None] >> shifts) & mask
+        return idx.reshape(idx_bytes.shape[0], -1)[:, :self.D].astype(np.uint8)
+
+    def compress(self, x: np.ndarray):
+        """x [..., D] float32 -> dict(idx_bytes [N,G] u8, vec_norms [N] fp16 bits, rotated [N,D])"""
+        norms, rotated = self.rotate(x)
+        idx = self.nearest(rotated)
+        return {
+            "idx_bytes": self.pack(idx),
+            "vec_norms": norms.astype(np.float16).view(np.uint16),
+            "rotated": rotated,
+            "norms_f32": norms,
+        }
+
+    def decompress(self, idx_bytes: np.ndarray, vec_norms_bits: np.ndarray) -> np.ndarray:
+        idx = self.unpack(idx_bytes.reshape(-1, idx_bytes.shape[-1]))
+        y = self.centroids[idx]
+        n = vec_norms_bits.reshape(-1, 1).view(np.float16).astype(np.float32)
+        with np.errstate(invalid="ignore", over="ignore"):
+            return (y @ self.Pi) * n
+
+
+# --------------------------------------------------------------------------
+# C restatement
+# --------------------------------------------------------------------------
+def build_c_oracle(force: bool = False) -> str:
+    """Compile oracle/tq_oracle.c with gcc into oracle/_build/ and return the library path."""
+    src = os.path.join(_HERE, "tq_oracle.c")
+    if (not force and os.path.exists(_LIB)
+            and os.path.getmtime(_LIB) >= os.path.getmtime(src)):
+        return _LIB
+    os.makedirs(_BUILD, exist_ok=True)
+    cmd = ["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-shared", "-fPIC", src, "-o", _LIB, "-lm"]
+    subprocess.run(cmd, check=True)
+    return _LIB
+
+
+_lib = None
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        path = _LIB if os.path.exists(_LIB) else build_c_oracle()
+        lib = ctypes.CDLL(path)
+        f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+        u8p = np.ctypeslib.ndpointer(np.uint8, flags="C_CONTIGUOUS")
+        u16p = np.ctypeslib.ndpointer(np.uint16, flags="C_CONTIGUOUS")
+        lib.tqo_compress.argtypes = [f32p, ctypes.c_longlong, ctypes.c_int, f32p, f32p, ctypes.c_int,
+                                     ctypes.c_int, u8p, u16p, ctypes.c_void_p]
+        lib.tqo_compress.restype = ctypes.c_int
+        lib.tqo_decompress.argtypes = [u8p, u16p, ctypes.c_longlong, ctypes.c_int, f32p, f32p,
+                                       ctypes.c_int, ctypes.c_int, f32p]
+        lib.tqo_decompress.restype = ctypes.c_int
+        lib.tqo_nearest.argtypes = [f32p, ctypes.c_longlong, f32p, ctypes.c_int, u8p]
+        lib.tqo_pack.argtypes = [u8p, ctypes.c_int, ctypes.c_int, u8p]
+        lib.tqo_unpack.argtypes = [u8p, ctypes.c_int, ctypes.c_int, u8p]
+        lib.tqo_f32_to_f16.argtypes = [f32p, u16p, ctypes.c_longlong]
+        lib.tqo_f16_to_f32.argtypes = [u16p, f32p, ctypes.c_longlong]
+        lib.tqo_max_threads.restype = ctypes.c_int
+        lib.tqo_set_threads.argtypes = [ctypes.c_int]
+        _lib = lib
+    return _lib
+
+
+class COracle:
+    """ctypes front end of tq_oracle.c."""
+
+    def __init__(self, Pi: np.ndarray, centroids: np.ndarray, bits: int, accum_double: bool = False):
+        self.lib = _load()
+        self.Pi = np.ascontiguousarray(Pi, dtype=np.float32)
+        self.centroids = np.ascontiguousarray(centroids, dtype=np.float32)
+        self.bits = int(bits)
+        self.D = self.Pi.shape[0]
+        self.accum_double = int(bool(accum_double))
+        assert self.centroids.size == 1 << self.bits
+
+    def compress(self, x: np.ndarray, want_rotated: bool = True):
+        flat = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.D)
+        N = flat.shape[0]
+        G = bytes_per_vector(self.D, self.bits)
+        idx_bytes = np.empty((N, G), dtype=np.uint8)
+        norms = np.empty(N, dtype=np.uint16)
+        rotated = np.empty((N, self.D), dtype=np.float32) if want_rotated else None
+        rc = self.lib.tqo_compress(flat, N, self.D, self.Pi, self.centroids, self.bits, self.accum_double,
+                                   idx_bytes, norms,
+                                   rotated.ctypes.data_as(ctypes.c_void_p) if want_rotated else None)
+        if rc:
+            raise RuntimeError(f"tqo_compress failed: {rc}")
+        return {"idx_bytes": idx_bytes, "vec_norms": norms, "rotated": rotated}
+
+    def decompress(self, idx_bytes: np.ndarray, vec_norms_bits: np.ndarray) -> np.ndarray:
+        G = bytes_per_vector(self.D, self.bits)
+        b = np.ascontiguousarray(idx_bytes, dtype=np.uint8).reshape(-1, G)
+        n = np.ascontiguousarray(vec_norms_bits, dtype=np.uint16).reshape(-1)
+        out = np.empty((b.shape[0], self.D), dtype=np.float32)
+        rc = self.lib.tqo_decompress(b, n, b.shape[0], self.D, self.Pi, self.centroids, self.bits,
+                                     self.accum_double, out)
+        if rc:
+            raise RuntimeError(f"tqo_decompress failed: {rc}")
+        return out
+
+    @staticmethod
+    def threads() -> int:
+        return _load().tqo_max_threads()
+
+    @staticmethod
+    def set_threads(n: int) -> None:
+        _load().tqo_set_threads(n)
+
+
+# --------------------------------------------------------------------------
+# comparison helpers shared by the parity tests
+# --------------------------------------------------------------------------
+def unpack_codes(idx_bytes: np.ndarray, D: int, bits: int) -> np.ndarray:
+    ipb = indices_per_byte(bits)
+    mask = (1 << bits) - 1
+    shifts = np.array([bits * i for i in range(ipb - 1, -1, -1)], dtype=np.int64)
+    flat = idx_bytes.reshape(-1, idx_bytes.shape[-1]).astype(np.int64)
+    return ((flat[:, :, None] >> shifts) & mask).reshape(flat.shape[0], -1)[:, :D].astype(np.int16)
+
+
+def code_mismatch_report(test_bytes: np.ndarray, oracle_bytes: np.ndarray, rotated: np.ndarray,
+                         centroids: np.ndarray, bits: int, window: float = 1e-5) -> dict:
+    """Compare packed codes.  A differing coordinate is excused only if the oracle's rotated
+    coordinate lies within `window` of the decision boundary (midpoint) between the two codes
+    and the codes are neighbours.  Returns counts; `outside` must be zero for parity."""
+    D = rotated.shape[-1]
+    a = unpack_codes(test_bytes, D, bits)
+    b = unpack_codes(oracle_bytes, D, bits)
+    diff = a != b
+    n_diff = int(diff.sum())
+    outside = 0
+    worst = 0.0
+    if n_diff:
+        r = rotated.reshape(-1, D)[diff].astype(np.float64)
+        ia = a[diff].astype(np.int64)
+        ib = b[diff].astype(np.int64)
+        c = centroids.astype(np.float64)
+        neighbours = np.abs(ia - ib) == 1
+        lo = np.minimum(ia, ib)
+        hi = np.minimum(lo + 1, len(c) - 1)
+        boundary = 0.5 * (c[lo] + c[hi])
+        dist = np.abs(r - boundary)
+        ok = neighbours & (dist <= window)
+        outside = int((~ok).sum())
+        worst = float(dist.max())
+    return {"coords": int(a.size), "differ": n_diff, "outside_window": outside,
+            "worst_boundary_distance": worst,
+            "padding_equal": bool(np.array_equal(test_bytes.shape, oracle_bytes.shape))}
+
+
+def fp16_ulp_distance(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
+    """Distance in fp16 units-in-the-last-place between two bit-pattern arrays (same sign assumed ok)."""
+    def key(u):
+        u = u.astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u & 0x7FFF)
+    return np.abs(key(a_bits) - key(b_bits))

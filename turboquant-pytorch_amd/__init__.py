@@ -1,0 +1,17 @@
+"""
+MI355X-native TurboQuant V3 KV-cache compress / decompress path.
+
+The directory name contains a hyphen, so import it through the `turboquant_amd`
+alias module at the repository root (or `importlib.import_module("turboquant-pytorch_amd")`):
+
+    from turboquant_amd import TurboQuantV3, MSECompressor
+"""
+from .lloyd_max import LloydMaxCodebook, solve_lloyd_max
+from .rotation import generate_rotation_matrix
+from .compressors_v3 import MSECompressor, TurboQuantV3
+from . import _native
+
+__all__ = [
+    "MSECompressor", "TurboQuantV3", "LloydMaxCodebook", "solve_lloyd_max",
+    "generate_rotation_matrix", "_native",
+]

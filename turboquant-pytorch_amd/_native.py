@@ -1,0 +1,335 @@
+"""
+Loader, builder and Python bindings of the C-ABI library `csrc/libtqamd.so`
+(declared in include/tqamd.h), plus the `torch.library` custom ops that put the
+HIP kernels behind ordinary tensor calls.
+
+There is no CPU implementation and no fallback: if the library is missing, or a
+tensor is not on a HIP device, the calls raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import shutil
+import subprocess
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_HERE, "csrc")
+LIB_PATH = os.path.join(CSRC, "libtqamd.so")
+SOURCES = ("tq_host.cpp", "tq_compress.hip", "tq_decompress.hip")
+HEADERS = ("tq_table.h", "tq_device.h", os.path.join("..", "..", "include", "tqamd.h"))
+GPU_ARCH = "gfx950"
+
+TQ_F32, TQ_F16, TQ_BF16 = 0, 1, 2
+_DTYPE_CODE = {torch.float32: TQ_F32, torch.float16: TQ_F16, torch.bfloat16: TQ_BF16}
+HEAD_DIM = 128
+
+
+class TqError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+
+# ------------------------------------------------------------------------------------
+# build
+# ------------------------------------------------------------------------------------
+def hipcc_command(out_path: str = LIB_PATH) -> List[str]:
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    return [
+        hipcc, "-shared", "-fPIC", "-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        "-Wno-unused-command-line-argument",
+        *[os.path.join(CSRC, s) for s in SOURCES],
+        "-o", out_path,
+    ]
+
+
+def build(force: bool = True, verbose: bool = False) -> str:
+    """Compile the HIP/C++ sources into csrc/libtqamd.so (cross-compiles without a GPU)."""
+    if not force and os.path.exists(LIB_PATH):
+        newest = max(os.path.getmtime(os.path.join(CSRC, f)) for f in SOURCES + HEADERS)
+        if os.path.getmtime(LIB_PATH) >= newest:
+            return LIB_PATH
+    tmp = LIB_PATH + ".tmp"
+    cmd = hipcc_command(tmp)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    if verbose and res.stderr:
+        print(res.stderr)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+# ------------------------------------------------------------------------------------
+# ctypes view of include/tqamd.h
+# ------------------------------------------------------------------------------------
+class TqJob(ctypes.Structure):
+    _fields_ = [
+        ("states", ctypes.c_void_p),
+        ("idx_bytes", ctypes.c_void_p),
+        ("vec_norms", ctypes.c_void_p),
+        ("table_dev", ctypes.c_void_p),
+        ("rows", ctypes.c_longlong),
+        ("tokens", ctypes.c_longlong),
+        ("row_stride", ctypes.c_longlong),
+        ("token_stride", ctypes.c_longlong),
+        ("bits", ctypes.c_int),
+        ("dtype", ctypes.c_int),
+    ]
+
+
+EXPORTS = (
+    "tq_abi_version", "tq_status_string", "tq_device_count", "tq_bytes_per_vector",
+    "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_quantize_host",
+    "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched",
+)
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise TqError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(hipcc --offload-arch=gfx950). There is no fallback implementation.")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, ll, ci = ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int
+    L.tq_abi_version.restype = ci
+    L.tq_status_string.restype = ctypes.c_char_p
+    L.tq_status_string.argtypes = [ci]
+    L.tq_device_count.restype = ci
+    L.tq_bytes_per_vector.argtypes = [ci, ci]
+    L.tq_decision_thresholds.argtypes = [vp, ci, vp]
+    L.tq_table_bytes.restype = ll
+    L.tq_table_bytes.argtypes = [ci, ci]
+    L.tq_table_build.argtypes = [vp, vp, ci, ci, vp, ctypes.c_size_t]
+    L.tq_table_quantize_host.argtypes = [vp, vp, ll, vp]
+    L.tq_compress.argtypes = [vp, ci, ll, ll, ll, ll, vp, ci, ci, vp, vp, vp]
+    L.tq_decompress.argtypes = [vp, vp, ll, ll, vp, ci, ci, vp, ci, ll, ll, vp]
+    L.tq_compress_batched.argtypes = [vp, vp, ci, ci, vp]
+    L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp]
+    for name in EXPORTS:
+        if name not in ("tq_status_string", "tq_table_bytes"):
+            getattr(L, name).restype = ci
+    _lib = L
+    return L
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = lib().tq_status_string(status).decode()
+        raise TqError(f"{what}: {msg} (status {status})")
+
+
+# ------------------------------------------------------------------------------------
+# host-side table construction
+# ------------------------------------------------------------------------------------
+def decision_thresholds(centroids: np.ndarray) -> np.ndarray:
+    c = np.ascontiguousarray(centroids, dtype=np.float32)
+    out = np.empty(max(c.size - 1, 0), dtype=np.float32)
+    check(lib().tq_decision_thresholds(c.ctypes.data, c.size, out.ctypes.data), "tq_decision_thresholds")
+    return out
+
+
+def build_table(Pi: torch.Tensor, centroids: torch.Tensor, bits: int) -> np.ndarray:
+    """Bake rotation + codebook into the codec-table blob (host, uint8 array)."""
+    pi = np.ascontiguousarray(Pi.detach().cpu().to(torch.float32).numpy())
+    cent = np.ascontiguousarray(centroids.detach().cpu().to(torch.float32).numpy())
+    d = pi.shape[0]
+    if pi.shape != (d, d):
+        raise ValueError("Pi must be square")
+    if cent.size != 1 << bits:
+        raise ValueError(f"expected {1 << bits} centroids, got {cent.size}")
+    nbytes = lib().tq_table_bytes(d, bits)
+    if nbytes < 0:
+        check(int(nbytes), "tq_table_bytes")
+    blob = np.zeros(nbytes, dtype=np.uint8)
+    check(lib().tq_table_build(pi.ctypes.data, cent.ctypes.data, d, bits, blob.ctypes.data, blob.size), "tq_table_build")
+    return blob
+
+
+def quantize_host(table: np.ndarray, r: np.ndarray) -> np.ndarray:
+    """Table self-check used by the tests: the kernels' code search, emulated on the host."""
+    rr = np.ascontiguousarray(r, dtype=np.float32).reshape(-1)
+    out = np.empty(rr.size, dtype=np.uint8)
+    check(lib().tq_table_quantize_host(table.ctypes.data, rr.ctypes.data, rr.size, out.ctypes.data), "tq_table_quantize_host")
+    return out.reshape(np.shape(r))
+
+
+# ------------------------------------------------------------------------------------
+# tensor plumbing
+# ------------------------------------------------------------------------------------
+def _require_gpu(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise TqError(f"{what} must live on a HIP device (got {t.device}); this package has no CPU path")
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dt]
+    except KeyError:
+        raise TqError(f"unsupported element type {dt}; float32, float16 and bfloat16 are supported") from None
+
+
+def vector_layout(t: torch.Tensor) -> Optional[Tuple[int, int, int, int]]:
+    """(rows, tokens, row_stride, token_stride) in elements for a [B,H,S,D] tensor whose last
+    dimension is dense, or None if its strides do not reduce to the two-level form."""
+    B, H, S, D = t.shape
+    sb, sh, ss, sd = t.stride()
+    if D != 1 and sd != 1:
+        return None
+    esz = t.element_size()
+    if (t.data_ptr() % 16) or any((s * esz) % 16 for s in (sb, sh, ss)):
+        return None
+    n = B * H * S
+    if n == 0:
+        return (0, 0, 0, D)
+    # drop dimensions of extent 1, then try to merge (b,h,s) left to right
+    dims = [(e, s) for e, s in ((B, sb), (H, sh), (S, ss)) if e != 1]
+    if not dims:
+        return (1, 1, 0, D)
+    merged = [dims[0]]
+    for e, s in dims[1:]:
+        pe, ps = merged[-1]
+        if ps == e * s:
+            merged[-1] = (pe * e, s)
+        else:
+            merged.append((e, s))
+    if len(merged) == 1:
+        return (1, merged[0][0], 0, merged[0][1])
+    if len(merged) == 2:
+        return (merged[0][0], merged[1][0], merged[0][1], merged[1][1])
+    return None
+
+
+def _stream_handle(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def compress_into(states: torch.Tensor, table: torch.Tensor, bits: int,
+                  idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> None:
+    """Launch tq_compress on `states` ([B,H,S,128], any supported float type, last dim dense)."""
+    _require_gpu(states, "states")
+    _require_gpu(table, "codec table")
+    lay = vector_layout(states)
+    if lay is None:
+        states = states.contiguous()
+        lay = vector_layout(states)
+    rows, tokens, row_stride, token_stride = lay
+    with torch.cuda.device(states.device):
+        rc = lib().tq_compress(states.data_ptr(), dtype_code(states.dtype), rows, tokens, row_stride, token_stride,
+                               table.data_ptr(), states.shape[-1], bits,
+                               idx_bytes.data_ptr(), vec_norms.data_ptr(), _stream_handle(states.device))
+    check(rc, "tq_compress")
+
+
+def decompress_into(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
+                    out: torch.Tensor) -> None:
+    """Launch tq_decompress, writing vector n of the packed stream to `out` ([B,H,S,128] view)."""
+    _require_gpu(idx_bytes, "idx_bytes")
+    _require_gpu(out, "output")
+    lay = vector_layout(out)
+    if lay is None:
+        raise TqError("decompress output must have a dense last dimension, 16-byte aligned rows and at most "
+                      "two stride levels")
+    rows, tokens, row_stride, token_stride = lay
+    with torch.cuda.device(out.device):
+        rc = lib().tq_decompress(idx_bytes.data_ptr(), vec_norms.data_ptr(), rows, tokens, table.data_ptr(),
+                                 out.shape[-1], bits, out.data_ptr(), dtype_code(out.dtype), row_stride,
+                                 token_stride, _stream_handle(out.device))
+    check(rc, "tq_decompress")
+
+
+# ------------------------------------------------------------------------------------
+# torch.library custom ops (so the kernels compose with the dispatcher, autocast guards,
+# fake tensors and graph capture like any other operator)
+# ------------------------------------------------------------------------------------
+def _packed_width(head_dim: int, bits: int) -> int:
+    ipb = 8 // bits
+    return -(-head_dim // ipb)
+
+
+@torch.library.custom_op("tqamd::compress", mutates_args=(), device_types="cuda")
+def compress_op(states: torch.Tensor, table: torch.Tensor, bits: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    B, H, S, D = states.shape
+    idx_bytes = torch.empty((B, H, S, _packed_width(D, bits)), dtype=torch.uint8, device=states.device)
+    vec_norms = torch.empty((B, H, S), dtype=torch.float16, device=states.device)
+    compress_into(states, table, bits, idx_bytes, vec_norms)
+    return idx_bytes, vec_norms
+
+
+@compress_op.register_fake
+def _(states, table, bits):
+    B, H, S, D = states.shape
+    return (states.new_empty((B, H, S, _packed_width(D, bits)), dtype=torch.uint8),
+            states.new_empty((B, H, S), dtype=torch.float16))
+
+
+@torch.library.custom_op("tqamd::decompress", mutates_args=(), device_types="cuda")
+def decompress_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
+                  head_dim: int, out_dtype: torch.dtype) -> torch.Tensor:
+    B, H, S, _ = idx_bytes.shape
+    out = torch.empty((B, H, S, head_dim), dtype=out_dtype, device=idx_bytes.device)
+    decompress_into(idx_bytes.contiguous(), vec_norms.contiguous(), table, bits, out)
+    return out
+
+
+@decompress_op.register_fake
+def _(idx_bytes, vec_norms, table, bits, head_dim, out_dtype):
+    B, H, S, _ = idx_bytes.shape
+    return idx_bytes.new_empty((B, H, S, head_dim), dtype=out_dtype)
+
+
+@torch.library.custom_op("tqamd::decompress_into", mutates_args=("out",), device_types="cuda")
+def decompress_into_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
+                       out: torch.Tensor) -> None:
+    decompress_into(idx_bytes.contiguous(), vec_norms.contiguous(), table, bits, out)
+
+
+# ------------------------------------------------------------------------------------
+# batched jobs
+# ------------------------------------------------------------------------------------
+class JobList:
+    """A fixed list of (tensor, packed buffers, table) jobs of one bit width and element type,
+    uploaded once and launched as a single kernel per direction."""
+
+    def __init__(self, jobs: Sequence[dict], device: torch.device):
+        if not jobs:
+            raise ValueError("empty job list")
+        self.n = len(jobs)
+        self.device = torch.device(device)
+        self.host = (TqJob * self.n)()
+        self._keep = []
+        for i, j in enumerate(jobs):
+            t = j["states"]
+            _require_gpu(t, "states")
+            lay = vector_layout(t)
+            if lay is None:
+                raise TqError("batched jobs need tensors with a dense last dimension and at most two stride levels")
+            rows, tokens, row_stride, token_stride = lay
+            self.host[i] = TqJob(t.data_ptr(), j["idx_bytes"].data_ptr(), j["vec_norms"].data_ptr(),
+                                 j["table"].data_ptr(), rows, tokens, row_stride, token_stride,
+                                 int(j["bits"]), dtype_code(t.dtype))
+            self._keep.append((t, j["idx_bytes"], j["vec_norms"], j["table"]))
+        raw = np.frombuffer(bytes(self.host), dtype=np.uint8).copy()
+        self.dev = torch.from_numpy(raw).to(self.device)
+
+    def compress(self) -> None:
+        with torch.cuda.device(self.device):
+            rc = lib().tq_compress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, HEAD_DIM,
+                                           _stream_handle(self.device))
+        check(rc, "tq_compress_batched")
+
+    def decompress(self) -> None:
+        with torch.cuda.device(self.device):
+            rc = lib().tq_decompress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, HEAD_DIM,
+                                             _stream_handle(self.device))
+        check(rc, "tq_decompress_batched")

@@ -1,0 +1,219 @@
+"""
+TurboQuant V3 KV-cache compressors on MI355X.
+
+Same classes, constructor arguments, method names, dictionary schemas and byte accounting as
+the reference's turboquant/compressors_v3.py (MSECompressor :28-120, TurboQuantV3 :123-265);
+the arithmetic runs in two fused gfx950 kernels (csrc/tq_compress.hip, csrc/tq_decompress.hip)
+reached through the C ABI in include/tqamd.h.  There is no CPU path: tensors must live on a
+HIP device.
+
+Differences a caller can observe, all deliberate:
+  * `device` defaults to "cuda" (the reference defaults to "cpu").
+  * Codebooks and rotations are cached per (head_dim, bits) / (head_dim, seed); the reference
+    re-solves them for every instance.  Values are identical.
+  * `TurboQuantV3.decompress_kv` writes the de-quantised tokens straight into the
+    full-length output in the window's dtype (one rounding from the fp32 accumulator) instead
+    of materialising an fp32 tensor, casting and concatenating.
+"""
+from __future__ import annotations
+
+import functools
+import math
+from typing import Tuple
+
+import torch
+
+from . import _native
+from .lloyd_max import LloydMaxCodebook
+from .rotation import generate_rotation_matrix
+
+
+@functools.lru_cache(maxsize=None)
+def _cached_rotation(head_dim: int, seed: int) -> torch.Tensor:
+    return generate_rotation_matrix(head_dim, seed=seed, device="cpu")
+
+
+@functools.lru_cache(maxsize=None)
+def _cached_centroids(head_dim: int, bits: int) -> torch.Tensor:
+    return LloydMaxCodebook(head_dim, bits).centroids
+
+
+class MSECompressor:
+    """
+    Single-stage MSE-optimal compressor for keys or values: unit-normalise, rotate, pick the
+    nearest Lloyd-Max centroid per coordinate, store bit-packed codes and fp16 norms.
+    Interface of compressors_v3.py:28-120.
+    """
+
+    def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cuda"):
+        self.head_dim = head_dim
+        self.bits = bits
+        self.device = device
+
+        pi_host = _cached_rotation(head_dim, seed)
+        cent_host = _cached_centroids(head_dim, bits)
+        self.Pi = pi_host.to(device)
+        self.centroids = cent_host.to(device)
+        # Everything the kernels read, baked once: split rotation tiles, quantiser grid, decode tables.
+        self._table_host = _native.build_table(pi_host, cent_host, bits)
+        self._table = None
+
+    @classmethod
+    def from_tensors(cls, Pi: torch.Tensor, centroids: torch.Tensor, bits: int, device: str = "cuda"):
+        """Build a compressor from an explicit rotation and codebook (parity tests pass the
+        reference's own matrices through here)."""
+        self = cls.__new__(cls)
+        self.head_dim = Pi.shape[0]
+        self.bits = bits
+        self.device = device
+        self.Pi = Pi.to(device=device, dtype=torch.float32)
+        self.centroids = centroids.to(device=device, dtype=torch.float32)
+        self._table_host = _native.build_table(Pi, centroids, bits)
+        self._table = None
+        return self
+
+    def table(self) -> torch.Tensor:
+        """Device copy of the codec table (uploaded on first use)."""
+        if self._table is None:
+            dev = torch.device(self.device)
+            if dev.type != "cuda":
+                raise _native.TqError(f"MSECompressor(device={self.device!r}): the codec runs on HIP devices only")
+            self._table = torch.from_numpy(self._table_host).to(dev)
+        return self._table
+
+    @torch.no_grad()
+    def compress(self, states: torch.Tensor) -> dict:
+        """(B, H, S, D) -> {"idx_bytes" u8 [B,H,S,G], "vec_norms" f16 [B,H,S], "shape", "idx_pad"}."""
+        B, H, S, D = states.shape
+        indices_per_byte = 8 // self.bits
+        idx_pad = (indices_per_byte - D % indices_per_byte) % indices_per_byte
+        idx_bytes, vec_norms = torch.ops.tqamd.compress(states, self.table(), self.bits)
+        return {
+            "idx_bytes": idx_bytes,
+            "vec_norms": vec_norms,
+            "shape": (B, H, S, D),
+            "idx_pad": idx_pad,
+        }
+
+    @torch.no_grad()
+    def decompress(self, compressed: dict) -> torch.Tensor:
+        """Back to a float32 (B, H, S, D) tensor."""
+        B, H, S, D = compressed["shape"]
+        idx_bytes = compressed["idx_bytes"].reshape(B, H, S, -1)
+        vec_norms = compressed["vec_norms"].reshape(B, H, S)
+        return torch.ops.tqamd.decompress(idx_bytes, vec_norms, self.table(), self.bits, D, torch.float32)
+
+    @torch.no_grad()
+    def decompress_into(self, compressed: dict, out: torch.Tensor) -> torch.Tensor:
+        """De-quantise into `out` (a [B,H,S,D] tensor or strided view of any supported float type)."""
+        B, H, S, D = compressed["shape"]
+        if tuple(out.shape) != (B, H, S, D):
+            raise ValueError(f"output shape {tuple(out.shape)} does not match compressed shape {(B, H, S, D)}")
+        torch.ops.tqamd.decompress_into(compressed["idx_bytes"].reshape(B, H, S, -1),
+                                        compressed["vec_norms"].reshape(B, H, S), self.table(), self.bits, out)
+        return out
+
+    def memory_bytes(self, B: int, H: int, S: int) -> dict:
+        """Bytes actually stored for B*H*S vectors (compressors_v3.py:107-120)."""
+        n_vec = B * H * S
+        indices_per_byte = 8 // self.bits
+        compressed = n_vec * math.ceil(self.head_dim / indices_per_byte) + n_vec * 2
+        fp16 = n_vec * self.head_dim * 2
+        return {
+            "compressed_bytes": compressed,
+            "fp16_bytes": fp16,
+            "compression_ratio": fp16 / compressed if compressed > 0 else 0,
+        }
+
+
+class TurboQuantV3:
+    """
+    KV-cache compressor: asymmetric key/value widths, an uncompressed window of recent tokens,
+    wider codes for the first and last `protected_layers` layers.  Interface of
+    compressors_v3.py:123-265.
+    """
+
+    def __init__(
+        self,
+        head_dim: int,
+        key_bits: int = 4,
+        value_bits: int = 2,
+        residual_window: int = 128,
+        layer_idx: int = 0,
+        n_layers: int = 36,
+        protected_layers: int = 4,
+        protected_bits: int = 8,
+        seed: int = 42,
+        device: str = "cuda",
+    ):
+        self.head_dim = head_dim
+        self.residual_window = residual_window
+        self.device = device
+
+        protected = layer_idx < protected_layers or layer_idx >= (n_layers - protected_layers)
+        self.key_bits = min(protected_bits if protected else key_bits, 8)
+        self.value_bits = min(protected_bits if protected else value_bits, 8)
+
+        seed_base = seed + layer_idx * 1000
+        self.key_compressor = MSECompressor(head_dim, self.key_bits, seed=seed_base, device=device)
+        self.val_compressor = MSECompressor(head_dim, self.value_bits, seed=seed_base + 500, device=device)
+
+    @torch.no_grad()
+    def compress_kv(self, keys: torch.Tensor, values: torch.Tensor) -> Tuple[dict, dict]:
+        """keys, values (B, H, S, D) -> two dicts with "compressed", "fp16", "shape", "split_at"."""
+        B, H, S, D = keys.shape
+        rw = self.residual_window
+        if S <= rw:
+            return (
+                {"fp16": keys, "compressed": None, "shape": (B, H, S, D), "split_at": S},
+                {"fp16": values, "compressed": None, "shape": (B, H, S, D), "split_at": S},
+            )
+        split_at = S - rw
+        out = []
+        for tensor, comp in ((keys, self.key_compressor), (values, self.val_compressor)):
+            out.append({
+                # the kernel reads the strided slice in place: no contiguous copy of the old tokens
+                "compressed": comp.compress(tensor[:, :, :split_at, :]),
+                "fp16": tensor[:, :, split_at:, :],
+                "shape": (B, H, S, D),
+                "split_at": split_at,
+            })
+        return out[0], out[1]
+
+    @torch.no_grad()
+    def decompress_kv(self, compressed_k: dict, compressed_v: dict) -> Tuple[torch.Tensor, torch.Tensor]:
+        """-> keys, values (B, H, S, D) in the dtype of the uncompressed window."""
+        if compressed_k["compressed"] is None:
+            return compressed_k["fp16"], compressed_v["fp16"]
+        out = []
+        for c, comp in ((compressed_k, self.key_compressor), (compressed_v, self.val_compressor)):
+            B, H, S, D = c["shape"]
+            split_at = c["split_at"]
+            window = c["fp16"]
+            full = torch.empty((B, H, S, D), dtype=window.dtype, device=window.device)
+            comp.decompress_into(c["compressed"], full[:, :, :split_at, :])
+            if S > split_at:
+                full[:, :, split_at:, :].copy_(window)
+            out.append(full)
+        return out[0], out[1]
+
+    def memory_bytes(self, B: int, H: int, S: int) -> dict:
+        """Bytes stored including the uncompressed window (compressors_v3.py:235-265)."""
+        fp16_tokens = min(self.residual_window, S)
+        compressed_tokens = max(S - fp16_tokens, 0)
+        compressed_bytes = 0
+        if compressed_tokens > 0:
+            compressed_bytes = (self.key_compressor.memory_bytes(B, H, compressed_tokens)["compressed_bytes"]
+                                + self.val_compressor.memory_bytes(B, H, compressed_tokens)["compressed_bytes"])
+        window_bytes = B * H * fp16_tokens * self.head_dim * 2 * 2
+        total = compressed_bytes + window_bytes
+        baseline = B * H * S * self.head_dim * 2 * 2
+        return {
+            "compressed_bytes": total,
+            "fp16_bytes": baseline,
+            "compression_ratio": baseline / total if total > 0 else 0,
+            "compressed_tokens": compressed_tokens,
+            "fp16_tokens": fp16_tokens,
+            "key_bits": self.key_bits,
+            "value_bits": self.value_bits,
+        }

@@ -1,0 +1,391 @@
+// compress: per-vector L2 norm, rotation on the matrix cores, Lloyd-Max code search, bit packing.
+// Replaces MSECompressor.compress (upstream turboquant/compressors_v3.py:46-81) with one kernel.
+//
+// Work decomposition (gfx950, wave64):
+//   * a wave owns a tile of 32 consecutive vectors; waves never synchronise with each other
+//     after the block-wide table load;
+//   * the tile is fetched with fully coalesced 16-byte loads (one instruction = 1 KiB of
+//     consecutive memory), parked in a wave-private LDS buffer with an XOR swizzle, and read
+//     back as the B operand of v_mfma_f32_32x32x16 (vector n on MFMA column n);
+//   * the A operand is the rotation, pre-split on the host into 16-bit terms whose sum is Pi
+//     to ~2^-22 (fp16 path) / 2^-17 or 2^-25 (bf16 path, 2 or 3 terms); inputs are exact in
+//     the MFMA input type (fp32 inputs are split into three exact bf16 terms), accumulation is
+//     fp32, so the rotated coordinates agree with an fp32 GEMM to ~1e-7 or better;
+//   * the rotation is applied to the raw vector and divided by (norm + 1e-8) afterwards
+//     (linearity), so the norm reduction overlaps the MFMAs;
+//   * every lane ends up with 64 consecutive rotated coordinates of one vector: the code search
+//     is one fused multiply-add, one 8-byte LDS lookup and one compare per coordinate, and the
+//     packed bytes of a lane are contiguous in memory.
+#include "tq_device.h"
+
+namespace {
+
+template <int DTYPE> struct InTraits;
+template <> struct InTraits<TQ_F16> {
+    static constexpr int ELEM = 2, WAVES = 8, TERMS = 2;
+};
+template <> struct InTraits<TQ_BF16> {
+    static constexpr int ELEM = 2, WAVES = 8, TERMS = 2;
+};
+template <> struct InTraits<TQ_F32> {
+    static constexpr int ELEM = 4, WAVES = 2, TERMS = 3;
+};
+
+template <int DTYPE>
+constexpr size_t compress_lds_bytes() {
+    using T = InTraits<DTYPE>;
+    return (size_t)T::TERMS * TQ_OPERAND_BYTES + TQ_GRID_LDS_BYTES + (size_t)T::WAVES * 32 * TQ_HEAD_DIM * T::ELEM;
+}
+
+__device__ __forceinline__ tq_f16v mfma_f16(tq_u4 a, tq_u4 b, tq_f16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, a), __builtin_bit_cast(tq_half8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ tq_f16v mfma_bf16(tq_u4 a, tq_u4 b, tq_f16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(tq_bf8, a), __builtin_bit_cast(tq_bf8, b), c, 0, 0, 0);
+}
+
+// sum of squares of the eight 16-bit values in v, added to acc (fp32)
+template <int DTYPE>
+__device__ __forceinline__ float sumsq8(tq_u4 v, float acc) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        if (DTYPE == TQ_F16) {
+            const tq_half2 h = __builtin_bit_cast(tq_half2, v[d]);
+            acc = __builtin_amdgcn_fdot2(h, h, acc, false);
+        } else {
+            const float lo = __uint_as_float(v[d] << 16), hi = __uint_as_float(v[d] & 0xffff0000u);
+            acc = fmaf(lo, lo, acc);
+            acc = fmaf(hi, hi, acc);
+        }
+    }
+    return acc;
+}
+
+// Exact split of eight floats into three bf16 terms each (x = t0 + t1 + t2, every term a
+// truncation, every remainder exact in fp32).  Output: packed bf16 operands.
+__device__ __forceinline__ void split_f32x8(const float (&x)[8], tq_u4 &t0, tq_u4 &t1, tq_u4 &t2) {
+    uint32_t a[8], b[8], c[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t xa = __float_as_uint(x[i]) & 0xffff0000u;
+        const float r1 = x[i] - __uint_as_float(xa);
+        const uint32_t xb = __float_as_uint(r1) & 0xffff0000u;
+        const float r2 = r1 - __uint_as_float(xb);
+        a[i] = xa; b[i] = xb; c[i] = __float_as_uint(r2) & 0xffff0000u;
+    }
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        t0[d] = (a[2 * d] >> 16) | a[2 * d + 1];
+        t1[d] = (b[2 * d] >> 16) | b[2 * d + 1];
+        t2[d] = (c[2 * d] >> 16) | c[2 * d + 1];
+    }
+}
+
+template <int DTYPE, int BITS>
+__global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_kernel(TqDevJob job0, const tq_job *jobs) {
+    using T = InTraits<DTYPE>;
+    constexpr int ELEM = T::ELEM;
+    constexpr int VEC_BYTES = TQ_HEAD_DIM * ELEM;      // 256 or 512
+    constexpr int STAGE = 32 * VEC_BYTES;              // wave-private tile buffer
+    constexpr int NLOAD = STAGE / 1024;                // 16-byte loads per lane per tile
+    constexpr int PIECES = VEC_BYTES / 16;             // 16-byte pieces per vector
+    constexpr int VEC_PER_LOAD = 64 / PIECES;          // vectors covered by one load instruction
+    constexpr int IPB = 8 / BITS;                      // codes per byte
+    constexpr int NB = 64 / IPB;                       // packed bytes per lane (half a vector)
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    TqDevJob job = job0;
+    if (jobs) {
+        const tq_job &j = jobs[blockIdx.y];
+        job.states = static_cast<const uint8_t *>(j.states);
+        job.idx_bytes = j.idx_bytes;
+        job.vec_norms = j.vec_norms;
+        job.table = static_cast<const uint8_t *>(j.table_dev);
+        job.n_vec = (uint32_t)(j.rows * j.tokens);
+        job.tokens = (uint32_t)j.tokens;
+        job.row_stride = j.row_stride;
+        job.token_stride = j.token_stride;
+    }
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t n_tiles = (job.n_vec + 31u) / 32u;
+    if (blockIdx.x * T::WAVES >= n_tiles) return;  // whole block idle (uniform)
+
+    const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
+    uint8_t *lds_a = lds;
+    uint8_t *lds_grid = lds + T::TERMS * TQ_OPERAND_BYTES;
+    uint8_t *stage = lds_grid + TQ_GRID_LDS_BYTES + wave * STAGE;
+
+    tq_copy_to_lds(lds_a, job.table + (DTYPE == TQ_F16 ? hd->off_a_f16 : hd->off_a_bf16),
+                   T::TERMS * TQ_OPERAND_BYTES, tid, T::WAVES * TQ_WAVE);
+    tq_copy_to_lds(lds_grid, job.table + hd->off_grid, (hd->grid_cells * 8u + 15u) & ~15u, tid, T::WAVES * TQ_WAVE);
+    const float grid_scale = hd->grid_scale, grid_bias = hd->grid_bias;
+    __syncthreads();
+
+    const uint32_t tile_stride = gridDim.x * T::WAVES;
+    uint32_t tile = blockIdx.x * T::WAVES + wave;
+
+    const uint32_t ld_vec = lane / PIECES, ld_piece = lane % PIECES;  // role in the coalesced loads
+    const uint32_t n = lane & 31u, hk = lane >> 5;                    // role in the MFMA: column, half
+
+    tq_u4 pre[NLOAD];
+    auto issue_loads = [&](uint32_t tl) {
+#pragma unroll
+        for (int j = 0; j < NLOAD; ++j) {
+            const uint32_t v = tl * 32u + j * VEC_PER_LOAD + ld_vec;
+            tq_u4 val = {0u, 0u, 0u, 0u};
+            if (v < job.n_vec)
+                val = *reinterpret_cast<const tq_u4 *>(job.states + tq_vec_offset<ELEM>(job, v) + ld_piece * 16u);
+            pre[j] = val;
+        }
+    };
+    if (tile < n_tiles) issue_loads(tile);
+
+    while (tile < n_tiles) {
+        // ---- park the tile in LDS (swizzled so that the operand reads below are conflict free)
+#pragma unroll
+        for (int j = 0; j < NLOAD; ++j) {
+            const uint32_t vl = j * VEC_PER_LOAD + ld_vec;
+            const uint32_t swz = (ELEM == 2) ? (vl & 15u) : ((vl & 15u) << 1);
+            *reinterpret_cast<tq_u4 *>(stage + vl * VEC_BYTES + ((ld_piece ^ swz) << 4)) = pre[j];
+        }
+        const uint32_t next = tile + tile_stride;
+        if (next < n_tiles) issue_loads(next);
+
+        // ---- rotation: acc[t][r] = sum_k Pi[64h + 16t + r][k] * x_n[k]  (raw, unnormalised)
+        tq_f16v acc[TQ_TILES];
+#pragma unroll
+        for (int t = 0; t < TQ_TILES; ++t) acc[t] = tq_zero16();
+        float ss0 = 0.f, ss1 = 0.f;
+
+#pragma unroll
+        for (int s = 0; s < TQ_STEPS; ++s) {
+            const tq_u4 *a_base = reinterpret_cast<const tq_u4 *>(lds_a) + (size_t)s * 64 + lane;
+            constexpr int TILE_STRIDE = TQ_STEPS * 64;          // tq_u4 units between tiles
+            constexpr int TERM_STRIDE = TQ_OPERAND_BYTES / 16;  // tq_u4 units between terms
+            if constexpr (ELEM == 2) {
+                const uint32_t piece = 2u * s + hk;
+                const tq_u4 b = *reinterpret_cast<const tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4));
+                if (s & 1) ss1 = sumsq8<DTYPE>(b, ss1); else ss0 = sumsq8<DTYPE>(b, ss0);
+#pragma unroll
+                for (int term = 0; term < T::TERMS; ++term)
+#pragma unroll
+                    for (int t = 0; t < TQ_TILES; ++t) {
+                        const tq_u4 a = a_base[term * TERM_STRIDE + t * TILE_STRIDE];
+                        acc[t] = (DTYPE == TQ_F16) ? mfma_f16(a, b, acc[t]) : mfma_bf16(a, b, acc[t]);
+                    }
+            } else {
+                const uint32_t piece = 2u * (2u * s + hk);
+                const uint32_t swz = (n & 15u) << 1;
+                const uint8_t *row = stage + n * VEC_BYTES;
+                const tq_u4 q0 = *reinterpret_cast<const tq_u4 *>(row + ((piece ^ swz) << 4));
+                const tq_u4 q1 = *reinterpret_cast<const tq_u4 *>(row + (((piece + 1u) ^ swz) << 4));
+                float x[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { x[i] = __uint_as_float(q0[i]); x[4 + i] = __uint_as_float(q1[i]); }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) { if (i & 1) ss1 = fmaf(x[i], x[i], ss1); else ss0 = fmaf(x[i], x[i], ss0); }
+                tq_u4 xt[3];
+                split_f32x8(x, xt[0], xt[1], xt[2]);
+                // all products whose weight is >= 2^-24 of the leading one: (x term i, Pi term j), i + j <= 2
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+#pragma unroll
+                    for (int term = 0; term + i < 3; ++term)
+#pragma unroll
+                        for (int t = 0; t < TQ_TILES; ++t) {
+                            const tq_u4 a = a_base[term * TERM_STRIDE + t * TILE_STRIDE];
+                            acc[t] = mfma_bf16(a, xt[i], acc[t]);
+                        }
+            }
+        }
+
+        // ---- norm: both lanes of a vector hold half of the squares
+        float ss = ss0 + ss1;
+        ss += __shfl_xor(ss, 32);
+        const float nrm = sqrtf(ss);
+        float inv = 1.0f / (nrm + 1e-8f);
+        if (DTYPE == TQ_F16) inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
+
+        // ---- code search + packing.  Lane (n, hk) holds coordinates 64*hk + 16*t + r.
+        uint32_t words[NB / 4];
+#pragma unroll
+        for (int w = 0; w < NB / 4; ++w) words[w] = 0u;
+#pragma unroll
+        for (int t = 0; t < TQ_TILES; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float rot = acc[t][r] * inv;
+                const uint32_t addr = __float_as_uint(fmaf(rot, grid_scale, grid_bias)) & TQ_GRID_ADDR_MASK;
+                const TqGridCell cell = *reinterpret_cast<const TqGridCell *>(lds_grid + addr);
+                const uint32_t code = cell.base + (rot >= cell.threshold ? 1u : 0u);
+                const int c = 16 * t + r;            // local coordinate 0..63
+                const int byte = c / IPB;            // local byte
+                const int k = c % IPB;               // position inside the byte, MSB first
+                const int shift = 8 * (byte % 4) + BITS * (IPB - 1 - k);
+                words[byte / 4] |= code << shift;
+            }
+
+        const uint32_t v = tile * 32u + n;
+        if (v < job.n_vec) {
+            uint8_t *dst = job.idx_bytes + (size_t)v * (2 * NB) + hk * NB;
+            if (NB == 8) {
+                tq_u2 o = {words[0], words[1]};
+                *reinterpret_cast<tq_u2 *>(dst) = o;
+            } else {
+#pragma unroll
+                for (int q = 0; q < NB / 16; ++q) {
+                    tq_u4 o = {words[4 * q], words[4 * q + 1], words[4 * q + 2], words[4 * q + 3]};
+                    *reinterpret_cast<tq_u4 *>(dst + 16 * q) = o;
+                }
+            }
+            if (hk == 0) {
+                const _Float16 hn = (_Float16)nrm;
+                job.vec_norms[v] = __builtin_bit_cast(uint16_t, hn);
+            }
+        }
+        tile = next;
+    }
+}
+
+// ---- host side --------------------------------------------------------------------------
+
+struct DeviceInfo {
+    int cus = 0;
+    int lds_optin = 0;
+};
+int query_device(DeviceInfo &info) {
+    static DeviceInfo cache[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return TQ_ERR_NO_DEVICE;
+    if (cache[dev].cus == 0) {
+        int cus = 0, lds = 0;
+        e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return (int)e;
+        e = hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev);
+        if (e != hipSuccess) return (int)e;
+        cache[dev].lds_optin = lds;
+        cache[dev].cus = cus > 0 ? cus : 1;
+    }
+    info = cache[dev];
+    return 0;
+}
+
+template <int DTYPE, int BITS>
+int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t stream) {
+    using T = InTraits<DTYPE>;
+    DeviceInfo info;
+    int rc = query_device(info);
+    if (rc) return rc;
+    constexpr size_t lds = compress_lds_bytes<DTYPE>();
+    static bool configured[64] = {};
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (!configured[dev]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&tq_compress_kernel<DTYPE, BITS>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        configured[dev] = true;
+    }
+    const uint32_t want = (max_tiles + T::WAVES - 1) / T::WAVES;
+    uint32_t per_job = (uint32_t)((info.cus * 2 + n_jobs - 1) / n_jobs);
+    if (n_jobs == 1) per_job = (uint32_t)info.cus;
+    uint32_t bx = want < per_job ? want : per_job;
+    if (bx == 0) bx = 1;
+    dim3 grid(bx, (unsigned)n_jobs, 1), block(T::WAVES * TQ_WAVE, 1, 1);
+    hipLaunchKernelGGL((tq_compress_kernel<DTYPE, BITS>), grid, block, lds, stream, job, jobs_dev);
+    return (int)hipGetLastError();
+}
+
+template <int DTYPE>
+int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t s) {
+    switch (bits) {
+        case 1: return launch_compress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, s);
+        case 2: return launch_compress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, s);
+        case 3: return launch_compress<DTYPE, 3>(job, jobs_dev, n_jobs, max_tiles, s);
+        case 4: return launch_compress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, s);
+        case 5: case 6: case 7: case 8:  // one code per byte: identical packing
+            return launch_compress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, s);
+        default: return TQ_ERR_BITS;
+    }
+}
+
+int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t s) {
+    switch (dtype) {
+        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, s);
+        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, s);
+        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, s);
+        default: return TQ_ERR_DTYPE;
+    }
+}
+
+int elem_bytes(int dtype) { return dtype == TQ_F32 ? 4 : (dtype == TQ_F16 || dtype == TQ_BF16) ? 2 : 0; }
+
+// Shared argument checks of one job; fills n_vec.
+int check_job(const void *states, int dtype, long long rows, long long tokens, long long row_stride,
+              long long token_stride, const void *table, int head_dim, int bits, const void *idx_bytes,
+              const void *vec_norms, long long *n_vec) {
+    if (bits < 1 || bits > 8) return TQ_ERR_BITS;
+    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
+    const int eb = elem_bytes(dtype);
+    if (!eb) return TQ_ERR_DTYPE;
+    if (rows < 0 || tokens < 0) return TQ_ERR_SIZE;
+    if (rows != 0 && tokens > (long long)0x7fffffff / rows) return TQ_ERR_SIZE;
+    *n_vec = rows * tokens;
+    if (*n_vec == 0) return TQ_OK;
+    if (!states || !table || !idx_bytes || !vec_norms) return TQ_ERR_NULL;
+    if (token_stride < TQ_HEAD_DIM && tokens > 1) return TQ_ERR_SIZE;
+    if (rows > 1 && row_stride < 0) return TQ_ERR_SIZE;
+    if (((uintptr_t)states & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & 15u) || ((uintptr_t)vec_norms & 1u))
+        return TQ_ERR_ALIGN;
+    if (((token_stride * eb) & 15) || (rows > 1 && ((row_stride * eb) & 15))) return TQ_ERR_ALIGN;
+    return TQ_OK;
+}
+
+}  // namespace
+
+extern "C" int tq_compress(const void *states, int dtype, long long rows, long long tokens,
+                           long long row_stride, long long token_stride, const void *table_dev,
+                           int head_dim, int bits, uint8_t *idx_bytes, uint16_t *vec_norms, void *stream) {
+    long long n_vec = 0;
+    const int rc = check_job(states, dtype, rows, tokens, row_stride, token_stride, table_dev, head_dim, bits,
+                             idx_bytes, vec_norms, &n_vec);
+    if (rc || n_vec == 0) return rc;
+    TqDevJob job;
+    job.states = static_cast<const uint8_t *>(states);
+    job.idx_bytes = idx_bytes;
+    job.vec_norms = vec_norms;
+    job.table = static_cast<const uint8_t *>(table_dev);
+    job.n_vec = (uint32_t)n_vec;
+    job.tokens = (uint32_t)tokens;
+    job.row_stride = row_stride;
+    job.token_stride = token_stride;
+    return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
+                                   int head_dim, void *stream) {
+    if (n_jobs == 0) return TQ_OK;
+    if (!jobs_host || !jobs_dev) return TQ_ERR_NULL;
+    if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
+    long long max_vec = 0;
+    for (int i = 0; i < n_jobs; ++i) {
+        const tq_job &j = jobs_host[i];
+        if (j.bits != jobs_host[0].bits) return TQ_ERR_BITS;
+        if (j.dtype != jobs_host[0].dtype) return TQ_ERR_DTYPE;
+        long long n_vec = 0;
+        const int rc = check_job(j.states, j.dtype, j.rows, j.tokens, j.row_stride, j.token_stride, j.table_dev,
+                                 head_dim, j.bits, j.idx_bytes, j.vec_norms, &n_vec);
+        if (rc) return rc;
+        if (n_vec > max_vec) max_vec = n_vec;
+    }
+    if (max_vec == 0) return TQ_OK;
+    TqDevJob none{};
+    return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec + 31) / 32),
+                    static_cast<hipStream_t>(stream));
+}

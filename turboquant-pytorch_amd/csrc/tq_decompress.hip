@@ -1,0 +1,339 @@
+// decompress: unpack codes, centroid lookup, inverse rotation on the matrix cores, norm rescale,
+// cast to the output type, coalesced store (optionally straight into a strided slice of the
+// full-length K/V buffer).  Replaces MSECompressor.decompress (upstream
+// turboquant/compressors_v3.py:84-105) and the cast + concatenation of
+// TurboQuantV3.decompress_kv (:226-232) with one kernel.
+//
+// A wave owns 32 consecutive vectors.  Lane (n, hk) reads the packed bytes of codes
+// [64*hk, 64*hk+64) of vector n, turns every byte into the fp16 centroids it holds with one
+// LDS table lookup (the table is indexed by the whole byte, so 2-, 4- and 8-per-byte widths
+// cost 1/2, 1/4, 1/8 lookup per code) and feeds them as the B operand of
+// v_mfma_f32_32x32x16_f16; the A operand is Pi^T in fp16, fp32 accumulate.  The 32x128 result
+// tile is transposed through a wave-private, XOR-swizzled LDS buffer so that every store
+// instruction writes 1 KiB of consecutive memory.
+#include "tq_device.h"
+
+namespace {
+
+template <int DTYPE> struct OutTraits;
+template <> struct OutTraits<TQ_F16> { static constexpr int ELEM = 2, WAVES = 8; };
+template <> struct OutTraits<TQ_BF16> { static constexpr int ELEM = 2, WAVES = 8; };
+template <> struct OutTraits<TQ_F32> { static constexpr int ELEM = 4, WAVES = 4; };
+
+constexpr int LUT_LDS_BYTES = 4096;
+
+template <int DTYPE>
+constexpr size_t decompress_lds_bytes() {
+    using T = OutTraits<DTYPE>;
+    return (size_t)TQ_OPERAND_BYTES + LUT_LDS_BYTES + (size_t)T::WAVES * 32 * TQ_HEAD_DIM * T::ELEM;
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint16_t h) {
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+
+// Decode the eight codes of MFMA step s held by this lane into a packed fp16x8 operand.
+// raw[] holds the lane's 64/IPB packed bytes, little-endian dwords.
+template <int IPB, int NW>
+__device__ __forceinline__ tq_u4 decode_step(const uint32_t (&raw)[NW], int s, const uint8_t *lut) {
+    tq_u4 out;
+    if constexpr (IPB == 1) {  // 8 bytes, one code each -> 8 two-byte lookups
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const uint32_t b0 = (raw[2 * s + (2 * d) / 4] >> (8 * ((2 * d) % 4))) & 0xffu;
+            const uint32_t b1 = (raw[2 * s + (2 * d + 1) / 4] >> (8 * ((2 * d + 1) % 4))) & 0xffu;
+            const uint32_t lo = *reinterpret_cast<const uint16_t *>(lut + b0 * 2u);
+            const uint32_t hi = *reinterpret_cast<const uint16_t *>(lut + b1 * 2u);
+            out[d] = lo | (hi << 16);
+        }
+    } else if constexpr (IPB == 2) {  // 4 bytes, two codes each -> 4 four-byte lookups
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const uint32_t b = (raw[s] >> (8 * d)) & 0xffu;
+            out[d] = *reinterpret_cast<const uint32_t *>(lut + b * 4u);
+        }
+    } else if constexpr (IPB == 4) {  // 2 bytes, four codes each -> 2 eight-byte lookups
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t b = (raw[s / 2] >> (16 * (s % 2) + 8 * q)) & 0xffu;
+            const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lut + b * 8u);
+            out[2 * q] = v[0];
+            out[2 * q + 1] = v[1];
+        }
+    } else {  // IPB == 8: 1 byte, eight codes -> 1 sixteen-byte lookup
+        const uint32_t b = (raw[s / 4] >> (8 * (s % 4))) & 0xffu;
+        out = *reinterpret_cast<const tq_u4 *>(lut + b * 16u);
+    }
+    return out;
+}
+
+template <int DTYPE, int IPB>
+__global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompress_kernel(TqDevJob job0, const tq_job *jobs) {
+    using T = OutTraits<DTYPE>;
+    constexpr int ELEM = T::ELEM;
+    constexpr int VEC_BYTES = TQ_HEAD_DIM * ELEM;   // 256 or 512
+    constexpr int STAGE = 32 * VEC_BYTES;
+    constexpr int NSTORE = STAGE / 1024;            // 16-byte stores per lane per tile
+    constexpr int PIECES = VEC_BYTES / 16;          // 16-byte pieces per vector: 16 or 32
+    constexpr int VEC_PER_STORE = 64 / PIECES;
+    constexpr int NB = 64 / IPB;                    // packed bytes per lane
+    constexpr int NW = NB / 4;                      // dwords per lane: 2, 4, 8, 16
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    TqDevJob job = job0;
+    if (jobs) {
+        const tq_job &j = jobs[blockIdx.y];
+        job.states = static_cast<const uint8_t *>(j.states);
+        job.idx_bytes = j.idx_bytes;
+        job.vec_norms = j.vec_norms;
+        job.table = static_cast<const uint8_t *>(j.table_dev);
+        job.n_vec = (uint32_t)(j.rows * j.tokens);
+        job.tokens = (uint32_t)j.tokens;
+        job.row_stride = j.row_stride;
+        job.token_stride = j.token_stride;
+    }
+    uint8_t *out_base = const_cast<uint8_t *>(job.states);
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t n_tiles = (job.n_vec + 31u) / 32u;
+    if (blockIdx.x * T::WAVES >= n_tiles) return;
+
+    const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
+    uint8_t *lds_a = lds;
+    uint8_t *lds_lut = lds + TQ_OPERAND_BYTES;
+    uint8_t *stage = lds_lut + LUT_LDS_BYTES + wave * STAGE;
+
+    tq_copy_to_lds(lds_a, job.table + hd->off_at_f16, TQ_OPERAND_BYTES, tid, T::WAVES * TQ_WAVE);
+    tq_copy_to_lds(lds_lut, job.table + hd->off_lut, 256u * 2u * IPB, tid, T::WAVES * TQ_WAVE);
+    __syncthreads();
+
+    const uint32_t tile_stride = gridDim.x * T::WAVES;
+    uint32_t tile = blockIdx.x * T::WAVES + wave;
+    const uint32_t n = lane & 31u, hk = lane >> 5;
+    const uint32_t st_vec = lane / PIECES, st_piece = lane % PIECES;
+
+    uint32_t raw[NW];
+    uint16_t norm_bits = 0;
+    auto issue_loads = [&](uint32_t tl) {
+        const uint32_t v = tl * 32u + n;
+        const bool ok = v < job.n_vec;
+        const uint8_t *src = job.idx_bytes + (size_t)(ok ? v : 0u) * (2 * NB) + hk * NB;
+        if constexpr (NW == 2) {
+            tq_u2 t = {0u, 0u};
+            if (ok) t = *reinterpret_cast<const tq_u2 *>(src);
+            raw[0] = t[0]; raw[1] = t[1];
+        } else {
+#pragma unroll
+            for (int q = 0; q < NW / 4; ++q) {
+                tq_u4 t = {0u, 0u, 0u, 0u};
+                if (ok) t = *reinterpret_cast<const tq_u4 *>(src + 16 * q);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) raw[4 * q + i] = t[i];
+            }
+        }
+        norm_bits = ok ? job.vec_norms[v] : (uint16_t)0;
+    };
+    if (tile < n_tiles) issue_loads(tile);
+
+    while (tile < n_tiles) {
+        uint32_t cur[NW];
+#pragma unroll
+        for (int i = 0; i < NW; ++i) cur[i] = raw[i];
+        const float nrm = half_bits_to_float(norm_bits);
+        const uint32_t next = tile + tile_stride;
+        if (next < n_tiles) issue_loads(next);
+
+        // ---- x_hat[64h + 16t + r] = sum_j y[j] * Pi[j][.]   (un-scaled)
+        tq_f16v acc[TQ_TILES];
+#pragma unroll
+        for (int t = 0; t < TQ_TILES; ++t) acc[t] = tq_zero16();
+#pragma unroll
+        for (int s = 0; s < TQ_STEPS; ++s) {
+            const tq_u4 b = decode_step<IPB, NW>(cur, s, lds_lut);
+            const tq_u4 *a_base = reinterpret_cast<const tq_u4 *>(lds_a) + (size_t)s * 64 + lane;
+#pragma unroll
+            for (int t = 0; t < TQ_TILES; ++t) {
+                const tq_u4 a = a_base[t * TQ_STEPS * 64];
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, a),
+                                                                __builtin_bit_cast(tq_half8, b), acc[t], 0, 0, 0);
+            }
+        }
+
+        // ---- scale, cast, transpose through LDS.  Lane (n, hk) holds elements 64*hk + 16*t + r.
+        if constexpr (ELEM == 2) {
+#pragma unroll
+            for (int t = 0; t < TQ_TILES; ++t)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {  // two 16-byte pieces of 8 elements per MFMA tile
+                    tq_u4 o;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const float x0 = acc[t][8 * c + 2 * d] * nrm, x1 = acc[t][8 * c + 2 * d + 1] * nrm;
+                        if constexpr (DTYPE == TQ_F16) {
+                            const tq_half2 h = {(_Float16)x0, (_Float16)x1};
+                            o[d] = __builtin_bit_cast(uint32_t, h);
+                        } else {
+                            const tq_bf2 h = {(__bf16)x0, (__bf16)x1};
+                            o[d] = __builtin_bit_cast(uint32_t, h);
+                        }
+                    }
+                    const uint32_t piece = 8u * hk + 2u * t + c;
+                    *reinterpret_cast<tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4)) = o;
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < TQ_TILES; ++t)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {  // four 16-byte pieces of 4 floats per MFMA tile
+                    tq_u4 o;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) o[d] = __float_as_uint(acc[t][4 * c + d] * nrm);
+                    const uint32_t piece = 16u * hk + 4u * t + c;
+                    *reinterpret_cast<tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ n) << 4)) = o;
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < NSTORE; ++j) {
+            const uint32_t vl = j * VEC_PER_STORE + st_vec;
+            const uint32_t swz = (ELEM == 2) ? (vl & 15u) : vl;
+            const tq_u4 o = *reinterpret_cast<const tq_u4 *>(stage + vl * VEC_BYTES + ((st_piece ^ swz) << 4));
+            const uint32_t v = tile * 32u + vl;
+            if (v < job.n_vec)
+                *reinterpret_cast<tq_u4 *>(out_base + tq_vec_offset<ELEM>(job, v) + st_piece * 16u) = o;
+        }
+        tile = next;
+    }
+}
+
+// ---- host side --------------------------------------------------------------------------
+
+int device_cus(int &cus) {
+    static int cache[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return TQ_ERR_NO_DEVICE;
+    if (cache[dev] == 0) {
+        int c = 0;
+        e = hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return (int)e;
+        cache[dev] = c > 0 ? c : 1;
+    }
+    cus = cache[dev];
+    return 0;
+}
+
+template <int DTYPE, int IPB>
+int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t stream) {
+    using T = OutTraits<DTYPE>;
+    int cus = 0;
+    int rc = device_cus(cus);
+    if (rc) return rc;
+    constexpr size_t lds = decompress_lds_bytes<DTYPE>();
+    static bool configured[64] = {};
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (!configured[dev]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&tq_decompress_kernel<DTYPE, IPB>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        configured[dev] = true;
+    }
+    const uint32_t want = (max_tiles + T::WAVES - 1) / T::WAVES;
+    uint32_t per_job = (uint32_t)((cus * 2 + n_jobs - 1) / n_jobs);
+    if (n_jobs == 1) per_job = (uint32_t)cus;
+    uint32_t bx = want < per_job ? want : per_job;
+    if (bx == 0) bx = 1;
+    dim3 grid(bx, (unsigned)n_jobs, 1), block(T::WAVES * TQ_WAVE, 1, 1);
+    hipLaunchKernelGGL((tq_decompress_kernel<DTYPE, IPB>), grid, block, lds, stream, job, jobs_dev);
+    return (int)hipGetLastError();
+}
+
+template <int DTYPE>
+int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t s) {
+    switch (8 / bits) {
+        case 8: return launch_decompress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, s);
+        case 4: return launch_decompress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, s);
+        case 2: return launch_decompress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, s);
+        case 1: return launch_decompress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, s);
+        default: return TQ_ERR_BITS;
+    }
+}
+
+int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t s) {
+    switch (dtype) {
+        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, s);
+        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, s);
+        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, s);
+        default: return TQ_ERR_DTYPE;
+    }
+}
+
+int elem_bytes(int dtype) { return dtype == TQ_F32 ? 4 : (dtype == TQ_F16 || dtype == TQ_BF16) ? 2 : 0; }
+
+int check_job(const void *out, int dtype, long long rows, long long tokens, long long row_stride,
+              long long token_stride, const void *table, int head_dim, int bits, const void *idx_bytes,
+              const void *vec_norms, long long *n_vec) {
+    if (bits < 1 || bits > 8) return TQ_ERR_BITS;
+    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
+    const int eb = elem_bytes(dtype);
+    if (!eb) return TQ_ERR_DTYPE;
+    if (rows < 0 || tokens < 0) return TQ_ERR_SIZE;
+    if (rows != 0 && tokens > (long long)0x7fffffff / rows) return TQ_ERR_SIZE;
+    *n_vec = rows * tokens;
+    if (*n_vec == 0) return TQ_OK;
+    if (!out || !table || !idx_bytes || !vec_norms) return TQ_ERR_NULL;
+    if (token_stride < TQ_HEAD_DIM && tokens > 1) return TQ_ERR_SIZE;
+    if (rows > 1 && row_stride < 0) return TQ_ERR_SIZE;
+    if (((uintptr_t)out & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & 15u) || ((uintptr_t)vec_norms & 1u))
+        return TQ_ERR_ALIGN;
+    if (((token_stride * eb) & 15) || (rows > 1 && ((row_stride * eb) & 15))) return TQ_ERR_ALIGN;
+    return TQ_OK;
+}
+
+}  // namespace
+
+extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long rows, long long tokens,
+                             const void *table_dev, int head_dim, int bits, void *out, int out_dtype,
+                             long long row_stride, long long token_stride, void *stream) {
+    long long n_vec = 0;
+    const int rc = check_job(out, out_dtype, rows, tokens, row_stride, token_stride, table_dev, head_dim, bits,
+                             idx_bytes, vec_norms, &n_vec);
+    if (rc || n_vec == 0) return rc;
+    TqDevJob job;
+    job.states = static_cast<const uint8_t *>(out);
+    job.idx_bytes = const_cast<uint8_t *>(idx_bytes);
+    job.vec_norms = const_cast<uint16_t *>(vec_norms);
+    job.table = static_cast<const uint8_t *>(table_dev);
+    job.n_vec = (uint32_t)n_vec;
+    job.tokens = (uint32_t)tokens;
+    job.row_stride = row_stride;
+    job.token_stride = token_stride;
+    return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
+                                     int head_dim, void *stream) {
+    if (n_jobs == 0) return TQ_OK;
+    if (!jobs_host || !jobs_dev) return TQ_ERR_NULL;
+    if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
+    long long max_vec = 0;
+    for (int i = 0; i < n_jobs; ++i) {
+        const tq_job &j = jobs_host[i];
+        if (8 / (j.bits < 1 || j.bits > 8 ? 1 : j.bits) != 8 / (jobs_host[0].bits < 1 || jobs_host[0].bits > 8 ? 1 : jobs_host[0].bits))
+            return TQ_ERR_BITS;
+        if (j.dtype != jobs_host[0].dtype) return TQ_ERR_DTYPE;
+        long long n_vec = 0;
+        const int rc = check_job(j.states, j.dtype, j.rows, j.tokens, j.row_stride, j.token_stride, j.table_dev,
+                                 head_dim, j.bits, j.idx_bytes, j.vec_norms, &n_vec);
+        if (rc) return rc;
+        if (n_vec > max_vec) max_vec = n_vec;
+    }
+    if (max_vec == 0) return TQ_OK;
+    TqDevJob none{};
+    return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec + 31) / 32),
+                    static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,53 @@
+// Device-side helpers shared by the compress and decompress kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tqamd.h"
+#include "tq_table.h"
+
+typedef _Float16 tq_half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 tq_half2 __attribute__((ext_vector_type(2)));
+typedef __bf16 tq_bf8 __attribute__((ext_vector_type(8)));
+typedef __bf16 tq_bf2 __attribute__((ext_vector_type(2)));
+typedef float tq_f16v __attribute__((ext_vector_type(16)));
+typedef uint32_t tq_u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t tq_u2 __attribute__((ext_vector_type(2)));
+
+#define TQ_WAVE 64
+
+// Launch-time job descriptor (device view of tq_job, plus derived fields).
+struct TqDevJob {
+    const uint8_t *states;   // compress input / decompress output, byte pointer
+    uint8_t *idx_bytes;
+    uint16_t *vec_norms;
+    const uint8_t *table;
+    uint32_t n_vec;          // rows * tokens  (< 2^31)
+    uint32_t tokens;
+    long long row_stride;    // elements
+    long long token_stride;  // elements
+};
+
+// Byte offset of vector v inside `states`.
+template <int ELEM_BYTES>
+__device__ __forceinline__ long long tq_vec_offset(const TqDevJob &job, uint32_t v) {
+    if (job.tokens >= job.n_vec) return (long long)v * job.token_stride * ELEM_BYTES;  // one row
+    const uint32_t row = v / job.tokens;
+    const uint32_t tok = v - row * job.tokens;
+    return ((long long)row * job.row_stride + (long long)tok * job.token_stride) * ELEM_BYTES;
+}
+
+// Cooperative copy global -> LDS, 16 bytes per thread per trip.
+__device__ __forceinline__ void tq_copy_to_lds(uint8_t *dst, const uint8_t *src, uint32_t bytes,
+                                               uint32_t tid, uint32_t nthreads) {
+    const tq_u4 *s = reinterpret_cast<const tq_u4 *>(src);
+    tq_u4 *d = reinterpret_cast<tq_u4 *>(dst);
+    for (uint32_t i = tid; i < bytes / 16; i += nthreads) d[i] = s[i];
+}
+
+__device__ __forceinline__ tq_f16v tq_zero16() {
+    tq_f16v z;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) z[i] = 0.f;
+    return z;
+}

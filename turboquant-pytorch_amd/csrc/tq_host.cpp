@@ -1,0 +1,330 @@
+// Host side of the C ABI: status strings, size arithmetic, decision thresholds and the
+// codec-table builder.  No device code here.
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+#include <hip/hip_runtime_api.h>
+
+#include "../../include/tqamd.h"
+#include "tq_table.h"
+
+namespace {
+
+// ---- float <-> 16-bit formats, round to nearest even ------------------------------------
+inline uint32_t f32_bits(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
+inline float bits_f32(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+
+uint16_t to_bf16(float f) {
+    uint32_t u = f32_bits(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+float from_bf16(uint16_t h) { return bits_f32((uint32_t)h << 16); }
+
+uint16_t to_f16(float f) {
+    const uint32_t x = f32_bits(f);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    const uint32_t ex = (x >> 23) & 0xffu;
+    uint32_t man = x & 0x7fffffu;
+    if (ex == 0xffu) return (uint16_t)(sign | 0x7c00u | (man ? 0x200u | (man >> 13) : 0u));
+    const int e = (int)ex - 112;  // rebias 127 -> 15
+    if (e >= 31) return (uint16_t)(sign | 0x7c00u);
+    if (e <= 0) {
+        if (e < -10) return (uint16_t)sign;
+        man |= 0x800000u;
+        const uint32_t shift = (uint32_t)(14 - e);
+        uint32_t h = man >> shift;
+        const uint32_t rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (h & 1u))) ++h;
+        return (uint16_t)(sign | h);
+    }
+    uint32_t h = ((uint32_t)e << 10) | (man >> 13);
+    const uint32_t rem = man & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h;
+    return (uint16_t)(sign | h);
+}
+float from_f16(uint16_t h) {
+    const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    const uint32_t ex = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    if (ex == 0) {
+        if (!man) return bits_f32(sign);
+        int s = 0;
+        while (!(man & 0x400u)) { man <<= 1; ++s; }
+        return bits_f32(sign | ((uint32_t)(113 - s) << 23) | ((man & 0x3ffu) << 13));
+    }
+    if (ex == 31) return bits_f32(sign | 0x7f800000u | (man << 13));
+    return bits_f32(sign | ((ex + 112u) << 23) | (man << 13));
+}
+
+// ---- totally ordered integer key of a float (for binary searches over float values) -----
+inline int64_t fkey(float f) {
+    const uint32_t u = f32_bits(f);
+    return (u & 0x80000000u) ? -(int64_t)(u & 0x7fffffffu) : (int64_t)u;
+}
+inline float fkey_inv(int64_t k) {
+    return k < 0 ? bits_f32(0x80000000u | (uint32_t)(-k)) : bits_f32((uint32_t)k);
+}
+
+inline uint32_t round_up(uint32_t v, uint32_t a) { return (v + a - 1) / a * a; }
+
+bool valid_codebook(const float *c, int levels) {
+    for (int i = 0; i < levels; ++i) {
+        if (!std::isfinite(c[i])) return false;
+        if (i && !(c[i] > c[i - 1])) return false;
+    }
+    return true;
+}
+
+// smallest float r in (lo, hi] for which the upper centroid is strictly nearer in float math
+float threshold_between(float lo, float hi) {
+    auto upper_wins = [&](float r) { return std::fabs(r - hi) < std::fabs(r - lo); };
+    int64_t a = fkey(lo), b = fkey(hi);  // upper_wins(lo) is false, upper_wins(hi) is true
+    while (b - a > 1) {
+        const int64_t m = a + (b - a) / 2;
+        if (upper_wins(fkey_inv(m))) b = m; else a = m;
+    }
+    return fkey_inv(b);
+}
+
+inline uint32_t grid_cell(float r, float scale, float bias) {
+    return (f32_bits(std::fmaf(r, scale, bias)) & TQ_GRID_ADDR_MASK) >> 3;
+}
+
+struct Layout {
+    uint32_t off_a_f16, off_a_bf16, off_grid, off_at_f16, off_lut, off_centroids, off_thresholds, total;
+    uint32_t lut_entry_bytes;
+};
+Layout layout_for(int bits) {
+    const uint32_t levels = 1u << bits, ipb = 8u / (uint32_t)bits;
+    Layout L{};
+    uint32_t off = sizeof(TqTableHeader);
+    L.off_a_f16 = off;      off += 2 * TQ_OPERAND_BYTES;
+    L.off_a_bf16 = off;     off += 3 * TQ_OPERAND_BYTES;
+    L.off_at_f16 = off;     off += 2 * TQ_OPERAND_BYTES;
+    L.off_grid = off;       off += round_up(TQ_GRID_MAX_CELLS * sizeof(TqGridCell), 256);
+    L.lut_entry_bytes = 2 * ipb;
+    L.off_lut = off;        off += round_up(256 * L.lut_entry_bytes, 256);
+    L.off_centroids = off;  off += round_up(levels * 4, 256);
+    L.off_thresholds = off; off += round_up(levels * 4, 256);
+    L.total = off;
+    return L;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tq_abi_version(void) { return TQ_ABI_VERSION; }
+
+const char *tq_status_string(int status) {
+    switch (status) {
+        case TQ_OK: return "ok";
+        case TQ_ERR_NULL: return "null pointer argument";
+        case TQ_ERR_BITS: return "bits must be in 1..8";
+        case TQ_ERR_HEAD_DIM: return "unsupported head_dim (the gfx950 kernels handle 128)";
+        case TQ_ERR_DTYPE: return "unknown element type";
+        case TQ_ERR_SIZE: return "invalid size or stride";
+        case TQ_ERR_CODEBOOK: return "centroids must be finite and strictly ascending";
+        case TQ_ERR_TABLE: return "malformed codec table";
+        case TQ_ERR_ALIGN: return "pointer or stride not 16-byte aligned";
+        case TQ_ERR_NO_DEVICE: return "no usable HIP device";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString((hipError_t)status);
+    return "unknown status";
+}
+
+int tq_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+int tq_bytes_per_vector(int head_dim, int bits) {
+    if (bits < 1 || bits > 8) return TQ_ERR_BITS;
+    if (head_dim < 1) return TQ_ERR_HEAD_DIM;
+    const int ipb = 8 / bits;
+    return (head_dim + ipb - 1) / ipb;
+}
+
+int tq_decision_thresholds(const float *centroids, int levels, float *thresholds) {
+    if (!centroids || (levels > 1 && !thresholds)) return TQ_ERR_NULL;
+    if (levels < 1 || levels > 256) return TQ_ERR_SIZE;
+    if (!valid_codebook(centroids, levels)) return TQ_ERR_CODEBOOK;
+    for (int i = 0; i + 1 < levels; ++i) thresholds[i] = threshold_between(centroids[i], centroids[i + 1]);
+    return TQ_OK;
+}
+
+long long tq_table_bytes(int head_dim, int bits) {
+    if (bits < 1 || bits > 8) return TQ_ERR_BITS;
+    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
+    return layout_for(bits).total;
+}
+
+int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bits,
+                   void *table_host, size_t table_bytes) {
+    if (!Pi || !centroids || !table_host) return TQ_ERR_NULL;
+    if (bits < 1 || bits > 8) return TQ_ERR_BITS;
+    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
+    const Layout L = layout_for(bits);
+    if (table_bytes < L.total) return TQ_ERR_SIZE;
+    const int levels = 1 << bits;
+    const int D = TQ_HEAD_DIM;
+    if (!valid_codebook(centroids, levels)) return TQ_ERR_CODEBOOK;
+    for (int i = 0; i < D * D; ++i)
+        if (!std::isfinite(Pi[i])) return TQ_ERR_SIZE;
+
+    uint8_t *blob = static_cast<uint8_t *>(table_host);
+    std::memset(blob, 0, L.total);
+
+    // ---- thresholds ----
+    std::vector<float> thr((size_t)levels);
+    thr[levels - 1] = INFINITY;
+    if (levels > 1) {
+        const int rc = tq_decision_thresholds(centroids, levels, thr.data());
+        if (rc) return rc;
+    }
+    std::memcpy(blob + L.off_centroids, centroids, (size_t)levels * 4);
+    std::memcpy(blob + L.off_thresholds, thr.data(), (size_t)(levels - 1) * 4);
+
+    // ---- quantiser grid: smallest power-of-two resolution with <= 1 threshold per cell ----
+    const float range = 1.0625f;  // |rotated unit coordinate| <= 1 (+ rounding); cells beyond are never hit
+    float scale = 0.f, bias = 0.f;
+    uint32_t cells = 0;
+    std::vector<TqGridCell> grid;
+    bool ok = false;
+    for (int lg = 3; lg <= 10 && !ok; ++lg) {
+        scale = (float)(1 << lg);
+        cells = 2u * (uint32_t)std::ceil(range * scale);
+        if (cells > TQ_GRID_MAX_CELLS) break;
+        bias = (float)(cells / 2) + TQ_GRID_MAGIC;
+        grid.assign(cells, TqGridCell{INFINITY, 0});
+        // first float of every cell, by bisection on the monotone map r -> cell(r)
+        std::vector<float> first(cells + 1);
+        const float rmin = -(float)(cells / 2) / scale, rmax = (float)(cells / 2) / scale;
+        first[0] = -INFINITY;
+        for (uint32_t q = 1; q < cells; ++q) {
+            int64_t a = fkey(rmin), b = fkey(rmax);  // cell(rmin) = 0 < q <= cell(rmax - eps)
+            // invariant: cell(a) < q, cell(b) >= q   (b = rmax maps to `cells`, see below)
+            while (b - a > 1) {
+                const int64_t m = a + (b - a) / 2;
+                const float rm = fkey_inv(m);
+                // rmax itself maps one past the last cell; treat anything >= rmax as "beyond"
+                const uint32_t cm = rm >= rmax ? cells : grid_cell(rm, scale, bias);
+                if (cm >= q) b = m; else a = m;
+            }
+            first[q] = fkey_inv(b);
+        }
+        first[cells] = INFINITY;
+        ok = true;
+        int t = 0;  // thresholds are ascending; walk them alongside the cells
+        for (uint32_t q = 0; q < cells && ok; ++q) {
+            while (t < levels - 1 && thr[t] <= first[q]) ++t;  // counted for every r in the cell
+            grid[q].base = (uint32_t)t;
+            int inside = 0;
+            while (t + inside < levels - 1 && thr[t + inside] < first[q + 1]) ++inside;
+            if (inside > 1) { ok = false; break; }
+            if (inside == 1) grid[q].threshold = thr[t];
+            // the threshold inside this cell is not part of the next cell's base until passed:
+            // base of q+1 is recomputed by the first loop above.
+        }
+    }
+    if (!ok) return TQ_ERR_CODEBOOK;  // levels too dense for the grid
+    std::memcpy(blob + L.off_grid, grid.data(), (size_t)cells * sizeof(TqGridCell));
+
+    // ---- rotation operands ----
+    auto operand_index = [](int t, int s, int l, int i) { return (((size_t)t * TQ_STEPS + s) * 64 + l) * 8 + i; };
+    uint16_t *a_f16 = reinterpret_cast<uint16_t *>(blob + L.off_a_f16);
+    uint16_t *a_bf16 = reinterpret_cast<uint16_t *>(blob + L.off_a_bf16);
+    uint16_t *at_f16 = reinterpret_cast<uint16_t *>(blob + L.off_at_f16);
+    const size_t term = TQ_OPERAND_BYTES / 2;  // halves per operand set
+    const double pi_scale = (double)(1 << TQ_F16_PI_SHIFT);
+    for (int t = 0; t < TQ_TILES; ++t)
+        for (int s = 0; s < TQ_STEPS; ++s)
+            for (int l = 0; l < 64; ++l) {
+                const int m = l % 32, hk = l / 32;
+                // MFMA row m = 8a + 4h + b  <->  accumulator (h, r = 4a + b)  <->  output 64h + 16t + r
+                const int a = m / 8, h = (m / 4) % 2, b = m % 4;
+                const int out = 64 * h + 16 * t + 4 * a + b;
+                for (int i = 0; i < 8; ++i) {
+                    const size_t o = operand_index(t, s, l, i);
+                    {   // compress: rotated[out] = sum_k x[k] * Pi[out][k],  k = 16s + 8hk + i
+                        const int k = 16 * s + 8 * hk + i;
+                        const float p = Pi[out * D + k];
+                        const double ps = (double)p * pi_scale;
+                        const uint16_t hi = to_f16((float)ps);
+                        const uint16_t lo = to_f16((float)(ps - (double)from_f16(hi)));
+                        a_f16[o] = hi;
+                        a_f16[term + o] = lo;
+                        const uint16_t b0 = to_bf16(p);
+                        const float r1 = p - from_bf16(b0);
+                        const uint16_t b1 = to_bf16(r1);
+                        const float r2 = r1 - from_bf16(b1);
+                        a_bf16[o] = b0;
+                        a_bf16[term + o] = b1;
+                        a_bf16[2 * term + o] = to_bf16(r2);
+                    }
+                    {   // decompress: x[out] = sum_j y[j] * Pi[j][out],  j = 64hk + 8s + i
+                        const int j = 64 * hk + 8 * s + i;
+                        const float p = Pi[j * D + out];
+                        const uint16_t hi = to_f16(p);
+                        at_f16[o] = hi;
+                        at_f16[term + o] = to_f16((float)((double)p - (double)from_f16(hi)));
+                    }
+                }
+            }
+
+    // ---- decode table: byte value -> the ipb centroids it holds (MSB-first), as fp16 ----
+    const int ipb = 8 / bits;
+    const unsigned mask = (1u << bits) - 1u;
+    uint16_t *lut = reinterpret_cast<uint16_t *>(blob + L.off_lut);
+    for (int v = 0; v < 256; ++v)
+        for (int k = 0; k < ipb; ++k)
+            lut[v * ipb + k] = to_f16(centroids[((unsigned)v >> (bits * (ipb - 1 - k))) & mask]);
+
+    TqTableHeader hd{};
+    hd.magic = TQ_TABLE_MAGIC;
+    hd.version = TQ_TABLE_VERSION;
+    hd.head_dim = (uint32_t)D;
+    hd.bits = (uint32_t)bits;
+    hd.levels = (uint32_t)levels;
+    hd.ipb = (uint32_t)ipb;
+    hd.bytes_per_vec = (uint32_t)((D + ipb - 1) / ipb);
+    hd.grid_cells = cells;
+    hd.grid_scale = scale;
+    hd.grid_bias = bias;
+    hd.total_bytes = L.total;
+    hd.off_a_f16 = L.off_a_f16;
+    hd.off_a_bf16 = L.off_a_bf16;
+    hd.off_grid = L.off_grid;
+    hd.off_at_f16 = L.off_at_f16;
+    hd.off_lut = L.off_lut;
+    hd.off_centroids = L.off_centroids;
+    hd.off_thresholds = L.off_thresholds;
+    hd.lut_entry_bytes = L.lut_entry_bytes;
+    std::memcpy(blob, &hd, sizeof(hd));
+    return TQ_OK;
+}
+
+int tq_table_quantize_host(const void *table_host, const float *r, long long n, uint8_t *idx) {
+    if (!table_host || (n > 0 && (!r || !idx))) return TQ_ERR_NULL;
+    TqTableHeader hd;
+    std::memcpy(&hd, table_host, sizeof(hd));
+    if (hd.magic != TQ_TABLE_MAGIC || hd.version != TQ_TABLE_VERSION) return TQ_ERR_TABLE;
+    const TqGridCell *grid =
+        reinterpret_cast<const TqGridCell *>(static_cast<const uint8_t *>(table_host) + hd.off_grid);
+    for (long long i = 0; i < n; ++i) {
+        const uint32_t q = grid_cell(r[i], hd.grid_scale, hd.grid_bias);
+        const TqGridCell c = grid[q < hd.grid_cells ? q : 0];
+        idx[i] = (uint8_t)(c.base + (r[i] >= c.threshold ? 1u : 0u));
+    }
+    return TQ_OK;
+}
+
+}  // extern "C"

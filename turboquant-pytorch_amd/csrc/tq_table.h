@@ -1,0 +1,65 @@
+// Layout of the codec table blob shared by the host-side builder and the gfx950 kernels.
+//
+// One blob per compressor instance (rotation + codebook).  All section offsets are from the
+// start of the blob and 256-byte aligned.
+#pragma once
+#include <stdint.h>
+
+#define TQ_TABLE_MAGIC 0x54514d49u /* "TQMI" */
+#define TQ_TABLE_VERSION 3u
+#define TQ_HEAD_DIM 128
+
+// --- MFMA operand tiling (v_mfma_f32_32x32x16_{f16,bf16}) --------------------------------
+// A-operand tile (t, s): 64 lanes x 8 halves.  Lane l supplies row  m = l % 32  and the
+// contraction slice  (hk = l / 32, i = 0..7).  The accumulator register r (0..15) of lane
+// (n = l % 32, h = l / 32) holds row  m = 8*(r/4) + 4*h + (r%4)  of column n.
+//
+// Both kernels put the vectors on the MFMA columns (one vector per lane, two lanes per
+// vector) and choose the row order so that lane-half h ends up with 64 consecutive outputs:
+//     output(t, h, r) = 64*h + 16*t + r
+// and the contraction order so that lane-half hk consumes 64 consecutive inputs in 8 steps:
+//     input(s, hk, i) = 16*s + 8*hk + i      (compress:   element of x)
+//     input(s, hk, i) = 64*hk + 8*s + i      (decompress: code index)
+#define TQ_TILES 4  /* 128 outputs / 32 rows  */
+#define TQ_STEPS 8  /* 128 inputs  / 16 deep  */
+#define TQ_OPERAND_BYTES (TQ_TILES * TQ_STEPS * 64 * 16) /* one 128x128 16-bit operand set: 32 KiB */
+
+// The fp16 split of Pi is stored multiplied by 2^TQ_F16_PI_SHIFT so that the low term stays
+// in the fp16 normal range; the kernels fold 2^-shift into the per-vector scale.
+#define TQ_F16_PI_SHIFT 10
+
+// Quantiser grid: cell(r) = (bits(fma(r, grid_scale, grid_bias)) & TQ_GRID_ADDR_MASK) / 8,
+// entry = { float threshold; uint32 base }, code = base + (r >= threshold).
+#define TQ_GRID_ADDR_MASK 0x7ff8u
+#define TQ_GRID_MAX_CELLS 2176 /* what the kernels reserve in LDS (17 KiB) */
+#define TQ_GRID_LDS_BYTES (TQ_GRID_MAX_CELLS * 8)
+#define TQ_GRID_MAGIC 1572864.0f /* 1.5 * 2^20: one ulp = 1/8 */
+
+struct TqGridCell {
+    float threshold;
+    uint32_t base;
+};
+
+struct TqTableHeader {
+    uint32_t magic;
+    uint32_t version;
+    uint32_t head_dim;
+    uint32_t bits;
+    uint32_t levels;
+    uint32_t ipb;            // indices per byte = 8 / bits
+    uint32_t bytes_per_vec;  // ceil(head_dim / ipb)
+    uint32_t grid_cells;
+    float grid_scale;        // cells per unit of r (power of two)
+    float grid_bias;         // grid_cells/2 + TQ_GRID_MAGIC
+    uint32_t total_bytes;
+    uint32_t off_a_f16;      // compress operand, Pi * 2^shift as fp16 hi, lo     (2 x 32 KiB)
+    uint32_t off_a_bf16;     // compress operand, Pi as bf16 hi, mid, lo          (3 x 32 KiB)
+    uint32_t off_grid;       // TqGridCell[grid_cells]
+    uint32_t off_at_f16;     // decompress operand, Pi^T as fp16 hi, lo           (2 x 32 KiB)
+    uint32_t off_lut;        // decode table: 256 entries of ipb fp16 centroids (byte -> values)
+    uint32_t off_centroids;  // float[levels]
+    uint32_t off_thresholds; // float[levels - 1]
+    uint32_t lut_entry_bytes; // 2 * ipb
+    uint32_t reserved[45];
+};
+static_assert(sizeof(TqTableHeader) == 256, "header is one 256-byte block");
