@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV-cache compress + decompress hot path on one MI355X.
+
+A "step" is one pass over the whole synthetic cache: every layer's K and V tensor is compressed
+(packed codes + fp16 norms) and then de-quantised again, through the batched C-ABI entry points
+(one launch per bit-width group and direction).  Inputs, packed buffers and outputs are
+resident in HBM before the timed region starts.
+
+Default workload (the one BASELINE.json quotes its target on): Llama-3-8B-shaped cache,
+32 layers x [1, 8, 32768, 128] bf16, K4/V2, protected_layers=4 with the reference's semantics
+(the first and last 4 layers use 8-bit keys AND values, compressors_v3.py:158-160), no residual
+window.  `--workload llama3-8b-32k-k4v2` runs the same shape with every layer at K4/V2;
+`--workload qwen2.5-3b-8k` is BASELINE config 2 (fp16).
+
+Prints ONE JSON line (see README / DESIGN.md for the fields).
+"""
+import argparse
+import importlib
+import json
+import os
+import platform
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0     # MI355X published HBM3E bandwidth, GB/s
+
+WORKLOADS = {
+    # name: layers, batch, kv heads, tokens, dtype, key_bits, value_bits, protected_layers
+    "llama3-8b-32k": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2, protected=4),
+    "llama3-8b-32k-k4v2": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2, protected=0),
+    "qwen2.5-3b-8k": dict(layers=36, batch=1, heads=2, tokens=8192, dtype="f16", key_bits=4, value_bits=2, protected=0),
+}
+
+
+def packed_bytes(bits: int) -> int:
+    return -(-128 // (8 // bits))
+
+
+def algorithmic_bytes(bits: int, elem: int, direction: str) -> int:
+    """Bytes per vector that must cross HBM: the vector itself plus packed codes plus the fp16 norm.
+    Rotation tiles and codebook tables stay in L2/LDS and are not counted."""
+    return 128 * elem + packed_bytes(bits) + 2
+
+
+def synth_kv(torch, shape, seed, dtype, device):
+    """N(0,1) x per-channel log-normal(sigma=1) x per-token U[0.5, 2], generated on the device."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    x = torch.randn(shape, generator=g, device=device, dtype=torch.float32)
+    ch = torch.exp(torch.randn(shape[-1], generator=g, device=device))
+    tok = 0.5 + 1.5 * torch.rand(shape[:-1] + (1,), generator=g, device=device)
+    return (x * ch * tok).to(dtype)
+
+
+def cpu_baseline(pkg, widths, budget_s=20.0):
+    """The C restatement of the reference algorithm (oracle/tq_oracle.c, OpenMP over vectors), timed
+    on this machine's host cores on a bounded sample: `widths` = {bits: share of vectors}."""
+    import numpy as np
+    from oracle import tq_oracle as O
+
+    threads = O.COracle.threads()
+    rng = np.random.default_rng(0)
+    per_width = {}
+    sample_desc = []
+    for bits, share in sorted(widths.items()):
+        comp = pkg.MSECompressor(128, bits, seed=42, device="cpu")
+        orc = O.COracle(comp.Pi.numpy(), comp.centroids.numpy(), bits, accum_double=False)
+        n = 4096
+        x = rng.standard_normal((n, 128), dtype=np.float32)
+        t0 = time.perf_counter()
+        out = orc.compress(x, want_rotated=False)
+        orc.decompress(out["idx_bytes"], out["vec_norms"])
+        probe = time.perf_counter() - t0
+        target = budget_s * share
+        n = int(min(max(n * target / max(probe, 1e-6), 8192), 4_000_000))
+        x = rng.standard_normal((n, 128), dtype=np.float32)
+        t0 = time.perf_counter()
+        out = orc.compress(x, want_rotated=False)
+        orc.decompress(out["idx_bytes"], out["vec_norms"])
+        dt = time.perf_counter() - t0
+        per_width[bits] = n / dt
+        sample_desc.append(f"{n} x {bits}-bit")
+    # harmonic mix: time per vector of the workload = sum share_b / rate_b
+    rate = 1.0 / sum(share / per_width[b] for b, share in widths.items())
+    return {
+        "value": rate, "unit": "vectors/s", "cores": threads, "kind": "port",
+        "sample": "compress+decompress of " + ", ".join(sample_desc) + " random fp32 vectors, mixed in the workload's width shares",
+        "per_width_vectors_per_s": {str(b): r for b, r in per_width.items()},
+        "cpu": platform.processor() or platform.machine(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama3-8b-32k", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; the codec shards without communication "
+                 "(by layer / KV head / token range), so run one process per GPU instead of --gpus N>1")
+
+    import torch
+    pkg = importlib.import_module("turboquant-pytorch_amd")
+    native = pkg._native
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a HIP device")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    w = WORKLOADS[args.workload]
+    L, B, H, S = w["layers"], w["batch"], w["heads"], w["tokens"]
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16}[w["dtype"]]
+    n_vec = B * H * S
+
+    # ---- compressors (reference constructor semantics) and resident buffers -------------------
+    groups = {}   # bits -> list of job dicts
+    layers = []
+    for l in range(L):
+        tq = pkg.TurboQuantV3(128, key_bits=w["key_bits"], value_bits=w["value_bits"], residual_window=0,
+                              layer_idx=l, n_layers=L, protected_layers=w["protected"], device=str(dev))
+        layers.append(tq)
+        for which, comp in (("k", tq.key_compressor), ("v", tq.val_compressor)):
+            x = synth_kv(torch, (B, H, S, 128), seed=4_000_000 + 10 * l + (0 if which == "k" else 1), dtype=dtype, device=dev)
+            job = {
+                "states": x,
+                "idx_bytes": torch.empty((B, H, S, packed_bytes(comp.bits)), dtype=torch.uint8, device=dev),
+                "vec_norms": torch.empty((B, H, S), dtype=torch.float16, device=dev),
+                "table": comp.table(), "bits": comp.bits,
+                "out": torch.empty((B, H, S, 128), dtype=dtype, device=dev),
+            }
+            groups.setdefault(comp.bits, []).append(job)
+    comp_lists = {b: native.JobList(jobs, dev) for b, jobs in groups.items()}
+    deco_lists = {b: native.JobList([dict(j, states=j["out"]) for j in jobs], dev) for b, jobs in groups.items()}
+    order = sorted(groups)
+    torch.cuda.synchronize()
+
+    def step(events=None):
+        for b in order:
+            if events is not None:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+            comp_lists[b].compress()
+            if events is not None:
+                e1.record()
+                events.setdefault(("compress", b), []).append((e0, e1))
+        for b in order:
+            if events is not None:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+            deco_lists[b].decompress()
+            if events is not None:
+                e1.record()
+                events.setdefault(("decompress", b), []).append((e0, e1))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # ---- timed region: exactly `steps` steps ----------------------------------------------------
+    events = {}
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        step(events)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    gpu_ms = start.elapsed_time(stop)
+    ms_per_step = wall * 1000.0 / args.steps
+
+    # ---- sanity: what was timed is a real round trip ----------------------------------------------
+    j = groups[order[0]][0]
+    rel = float((j["out"].float() - j["states"].float()).norm() / j["states"].float().norm())
+    if not (0.0 < rel < 0.6):
+        sys.exit(f"bench.py: round trip looks wrong (relative error {rel})")
+
+    # ---- accounting ------------------------------------------------------------------------------------
+    elem = 2
+    total_vec = 2 * L * n_vec                       # K and V counted separately
+    kernels = {}
+    step_bytes = 0
+    for (direction, b), evs in events.items():
+        jobs = len(groups[b])
+        bytes_per_launch = jobs * n_vec * algorithmic_bytes(b, elem, direction)
+        avg_ms = sum(e0.elapsed_time(e1) for e0, e1 in evs) / len(evs)
+        step_bytes += bytes_per_launch
+        kernels[f"{direction}_b{b}"] = {
+            "launches_per_step": 1, "jobs": jobs, "vectors_per_launch": jobs * n_vec,
+            "algorithmic_bytes_per_launch": bytes_per_launch, "avg_ms": avg_ms,
+            "achieved_GBps": bytes_per_launch / avg_ms / 1e6,
+            "frac_of_hbm_peak": bytes_per_launch / avg_ms / 1e6 / HBM_PEAK_GBS,
+        }
+    dominant = max(kernels, key=lambda k: kernels[k]["avg_ms"])
+    dk = kernels[dominant]
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(args.workload, {}).get(dominant)
+        except Exception:
+            traffic = None
+
+    widths = {}
+    for b, jobs in groups.items():
+        widths[b] = len(jobs) / (2 * L)
+    result = {
+        "metric": "KV vectors/sec (compress+decompress)",
+        "value": total_vec * args.steps / wall,
+        "unit": "vectors/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": args.workload, "layers": L, "batch": B, "kv_heads": H, "tokens": S, "head_dim": 128,
+                   "key_bits": w["key_bits"], "value_bits": w["value_bits"], "protected_layers": w["protected"],
+                   "residual_window": 0, "width_groups": {str(b): len(groups[b]) for b in order},
+                   "vectors_per_step": total_vec},
+        "gpu_ms_per_step": gpu_ms / args.steps,
+        "step_algorithmic_GB": step_bytes / 1e9,
+        "step_GBps": step_bytes / (wall / args.steps) / 1e9,
+        "step_frac_of_hbm_peak": step_bytes / (wall / args.steps) / 1e9 / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dk["achieved_GBps"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": dk["frac_of_hbm_peak"], "traffic": traffic},
+        "kernels": kernels,
+        "round_trip_rel_error": rel,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(pkg, widths, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,283 @@
+"""Host logic of the package and the C ABI surface -- no GPU needed.
+
+Codebook and rotation against tables written by the reference, the quantiser tables against
+brute force, byte accounting and layer-bit selection against the reference's outputs, error
+behaviour of the C entry points, and that the library exports what include/tqamd.h declares.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    header = open(os.path.join(ROOT, "include", "tqamd.h")).read()
+    declared = sorted(set(re.findall(r"\b(tq_[a-z_0-9]+)\s*\(", header)))
+    assert len(declared) >= 12
+    lib = pkg._native.lib()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert sorted(pkg._native.EXPORTS) == declared
+    assert lib.tq_abi_version() == 1
+    assert lib.tq_status_string(0) == b"ok"
+    assert b"bits" in lib.tq_status_string(-2)
+
+
+def test_job_struct_layout_matches_header(pkg):
+    # 4 pointers + 4 int64 + 2 int32 = 72 bytes, no padding surprises
+    assert ctypes.sizeof(pkg._native.TqJob) == 72
+
+
+def test_codebooks_match_reference_bits(pkg, golden):
+    """Closed-form replay of the reference's 200-step Lloyd iteration == its quadrature result,
+    float32 bit for bit, for every (d, bits) the fixtures hold."""
+    cb = golden["codebooks"]
+    n = 0
+    for key in cb.files:
+        m = re.fullmatch(r"centroids_d(\d+)_b(\d+)", key)
+        if not m:
+            continue
+        d, b = int(m.group(1)), int(m.group(2))
+        cent, bounds = pkg.solve_lloyd_max(d, b)
+        assert np.array_equal(cent.numpy().view(np.uint32), cb[key].view(np.uint32)), key
+        assert np.abs(bounds.numpy() - cb[f"boundaries_d{d}_b{b}"]).max() < 1e-12
+        assert cent.dtype == torch.float32 and cent.numel() == 2 ** b
+        n += 1
+    assert n == 12
+
+
+def test_codebook_textbook_values(pkg):
+    """Where the iteration converges (bits <= 3) the table is Max's Gaussian quantiser times sigma."""
+    s = 1 / np.sqrt(128)
+    c1, _ = pkg.solve_lloyd_max(128, 1)
+    assert np.allclose(c1.numpy() / s, [-0.7978846, 0.7978846], atol=1e-6)
+    c2, _ = pkg.solve_lloyd_max(128, 2)
+    assert np.allclose(c2.numpy() / s, [-1.5104, -0.4528, 0.4528, 1.5104], atol=1e-4)
+    c3, _ = pkg.solve_lloyd_max(128, 3)
+    assert np.allclose(c3.numpy()[[0, 3, 4, 7]] / s, [-2.1520, -0.2451, 0.2451, 2.1520], atol=1e-4)
+    for b in range(1, 9):
+        c, _ = pkg.solve_lloyd_max(128, b)
+        assert abs(float(c.sum())) < 1e-5 and bool((c[1:] > c[:-1]).all())
+    cb = pkg.LloydMaxCodebook(128, 3)   # the one assert of the reference's own test script
+    assert cb.centroids.sum().abs().item() < 0.01 and cb.n_levels == 8
+
+
+def test_rotation_matches_reference(pkg, golden):
+    rots = golden["rotations"]
+    threads = torch.get_num_threads()
+    try:
+        for key in rots.files:
+            m = re.fullmatch(r"Pi_d(\d+)_s(\d+)", key)
+            d, seed = int(m.group(1)), int(m.group(2))
+            torch.set_num_threads(1)    # the fixtures were written single-threaded (LAPACK order)
+            one = pkg.generate_rotation_matrix(d, seed=seed).numpy()
+            torch.set_num_threads(threads)
+            many = pkg.generate_rotation_matrix(d, seed=seed).numpy()
+            # same recipe -> same matrix up to LAPACK rounding; bit-exact on the build container
+            assert np.abs(one - rots[key]).max() < 1e-5
+            assert np.abs(many - rots[key]).max() < 1e-5
+            eye = one.astype(np.float64) @ one.astype(np.float64).T
+            assert np.abs(eye - np.eye(d)).max() < 1e-5
+    finally:
+        torch.set_num_threads(threads)
+    a = pkg.generate_rotation_matrix(128, seed=7)
+    b = pkg.generate_rotation_matrix(128, seed=7)
+    c = pkg.generate_rotation_matrix(128, seed=8)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+
+
+@pytest.mark.parametrize("bits", range(1, 9))
+def test_thresholds_and_grid_equal_argmin(pkg, golden, oracle, bits):
+    """Both forms of the code search the kernels rely on -- counting thresholds, and the
+    fused-multiply-add grid lookup -- equal the reference's argmin for every probed float,
+    including the floats adjacent to every threshold."""
+    cent = golden["codebooks"][f"centroids_d128_b{bits}"]
+    Pi = golden["rotations"]["Pi_d128_s42"]
+    thr = pkg._native.decision_thresholds(cent)
+    assert thr.size == cent.size - 1 and np.all(np.diff(thr) > 0)
+    mids = (cent[:-1].astype(np.float64) + cent[1:]) / 2
+    assert np.abs(thr - mids).max() < 1e-7
+    table = pkg._native.build_table(torch.from_numpy(Pi), torch.from_numpy(cent), bits)
+    rng = np.random.default_rng(bits)
+    probes = [rng.normal(0, 1 / np.sqrt(128), 200000).astype(np.float32),
+              rng.uniform(-1.03, 1.03, 100000).astype(np.float32),
+              np.array([0.0, -0.0, 1.0, -1.0, 1.03, -1.03], np.float32)]
+    near = []
+    for t in thr:
+        lo = hi = np.float32(t)
+        near.append(lo)
+        for _ in range(4):
+            lo = np.nextafter(lo, np.float32(-np.inf))
+            hi = np.nextafter(hi, np.float32(np.inf))
+            near += [lo, hi]
+    probes.append(np.array(near, np.float32))
+    # the first float of every grid cell and its predecessor
+    hdr = table[:256].view(np.uint32)
+    cells = int(hdr[7])
+    scale = float(table[32:36].view(np.float32)[0])
+    edges = ((np.arange(cells + 1) - cells // 2) / scale).astype(np.float32)
+    edges = edges[np.abs(edges) <= 1.03]   # the grid covers |r| <= 1.05; unit coordinates stay below 1
+    probes += [edges, np.nextafter(edges, np.float32(-np.inf)), np.nextafter(edges, np.float32(np.inf))]
+    r = np.concatenate(probes)
+    ref = np.empty(r.size, np.uint8)
+    oracle._load().tqo_nearest(r, r.size, cent, cent.size, ref)
+    counted = (r[:, None] >= thr[None, :]).sum(-1) if thr.size else np.zeros(r.size, np.int64)
+    assert np.array_equal(counted.astype(np.uint8), ref)
+    assert np.array_equal(pkg._native.quantize_host(table, r), ref)
+
+
+def test_table_rotation_split_reconstructs_pi(pkg, golden):
+    """The 16-bit operand tiles in the table sum back to Pi: fp16 hi+lo to ~2^-21 relative,
+    bf16 three terms exactly, and the tiling puts element (out, k) where the kernels read it."""
+    Pi = golden["rotations"]["Pi_d128_s42"]
+    cent = golden["codebooks"]["centroids_d128_b4"]
+    table = pkg._native.build_table(torch.from_numpy(Pi), torch.from_numpy(cent), 4)
+    hdr = table[:256].view(np.uint32)
+    off_a_f16, off_a_bf16, off_grid, off_at = (int(x) for x in hdr[11:15])
+    op = 32768
+
+    def tiles(raw16, transpose):
+        a = raw16.reshape(4, 8, 64, 8)    # t, s, lane, i
+        out = np.zeros((128, 128), raw16.dtype)
+        for t in range(4):
+            for s in range(8):
+                for lane in range(64):
+                    m, hk = lane % 32, lane // 32
+                    o = 64 * ((m // 4) % 2) + 16 * t + 4 * (m // 8) + (m % 4)
+                    for i in range(8):
+                        if transpose:
+                            out[64 * hk + 8 * s + i, o] = a[t, s, lane, i]
+                        else:
+                            out[o, 16 * s + 8 * hk + i] = a[t, s, lane, i]
+        return out
+
+    f16 = table[off_a_f16:off_a_f16 + 2 * op].view(np.float16).reshape(2, -1)
+    hi, lo = tiles(f16[0], False).astype(np.float64), tiles(f16[1], False).astype(np.float64)
+    assert np.abs((hi + lo) / 1024 - Pi).max() < 2.0 ** -21 * np.abs(Pi).max()
+    bf = table[off_a_bf16:off_a_bf16 + 3 * op].view(np.uint16).reshape(3, -1)
+    terms = [(tiles(bf[i], False).astype(np.uint32) << 16).view(np.float32).astype(np.float64) for i in range(3)]
+    assert np.array_equal((terms[0] + terms[1] + terms[2]).astype(np.float32), Pi)
+    assert np.abs(terms[0] + terms[1] - Pi).max() < 2.0 ** -16 * np.abs(Pi).max()
+    at = table[off_at:off_at + 2 * op].view(np.float16).reshape(2, -1)
+    assert np.abs(tiles(at[0], True).astype(np.float64) + tiles(at[1], True).astype(np.float64) - Pi).max() < 1e-6
+
+
+def test_memory_bytes_match_reference(pkg, golden):
+    j = golden["json"]
+    for key, meta in j["mse_roundtrip"].items():
+        bits = int(key.split("_")[0][1:])
+        comp = pkg.MSECompressor(128, bits, seed=42 + bits, device="cpu")
+        assert comp.memory_bytes(1, 2, 48) == meta["memory_bytes"]
+        assert meta["idx_pad"] == 0 and meta["idx_bytes_shape"][-1] == -(-128 // (8 // bits))
+    assert pkg.MSECompressor(128, 4, seed=42, device="cpu").memory_bytes(1, 8, 1024) == j["config1"]["memory_bytes"]
+    for row in j["v3"]["memory_bytes_table"]:
+        kb, vb, rw, pl, li, nl, B, H, S = row["args"]
+        t = pkg.TurboQuantV3(128, key_bits=kb, value_bits=vb, residual_window=rw, layer_idx=li, n_layers=nl,
+                             protected_layers=pl, device="cpu")
+        assert t.memory_bytes(B, H, S) == row["memory_bytes"], row
+    # README closed forms: K4/V2 = 100 B per 512 B pair; rw128 + protected-4 at 8K over 36 layers = 3.62x
+    total = sum(pkg.TurboQuantV3(128, 4, 2, 128, li, 36, 4, device="cpu").memory_bytes(1, 2, 8192)["compressed_bytes"]
+                for li in range(36))
+    assert total == 2 * 41711616 and abs(36 * 8388608 / total - 3.62) < 0.005     # README: 3.6x
+    assert pkg.TurboQuantV3(128, 4, 2, 0, 10, 36, 4, device="cpu").memory_bytes(1, 1, 1)["compressed_bytes"] == 100
+
+
+def test_layer_bit_selection_matches_reference(pkg, golden):
+    v3 = golden["json"]["v3"]
+    for row in v3["bit_selection_cheap"]:
+        kb, vb, pl, nl, pb, li = row["args"]
+        t = pkg.TurboQuantV3(128, key_bits=kb, value_bits=vb, layer_idx=li, n_layers=nl, protected_layers=pl,
+                             protected_bits=pb, device="cpu")
+        assert (t.key_bits, t.value_bits) == (row["key_bits"], row["value_bits"]), row
+    for row in v3["protected_default"]:
+        t = pkg.TurboQuantV3(128, key_bits=4, value_bits=2, layer_idx=row["layer_idx"], n_layers=36,
+                             protected_layers=4, device="cpu")
+        assert (t.key_bits, t.value_bits) == (row["key_bits"], row["value_bits"])
+        assert t.memory_bytes(1, 2, 8192) == row["memory_bytes_1_2_8192"]
+    # protected_bits above 8 is capped at 8; seeds follow seed + 1000*layer (+500 for values)
+    t = pkg.TurboQuantV3(128, 4, 2, layer_idx=0, n_layers=8, protected_layers=1, protected_bits=16, device="cpu")
+    assert (t.key_bits, t.value_bits) == (8, 8)
+    t = pkg.TurboQuantV3(128, 4, 2, layer_idx=5, n_layers=36, protected_layers=4, device="cpu")
+    assert torch.equal(t.key_compressor.Pi, pkg.generate_rotation_matrix(128, seed=5042))
+    assert torch.equal(t.val_compressor.Pi, pkg.generate_rotation_matrix(128, seed=5542))
+
+
+def test_passthrough_and_errors_without_gpu(pkg):
+    t = pkg.TurboQuantV3(128, 4, 2, residual_window=16, layer_idx=5, n_layers=36, device="cpu")
+    k = torch.randn(1, 2, 16, 128)
+    v = torch.randn(1, 2, 16, 128)
+    ck, cv = t.compress_kv(k, v)               # S <= window: nothing is compressed, same objects back
+    assert ck["compressed"] is None and ck["fp16"] is k and cv["fp16"] is v and ck["split_at"] == 16
+    rk, rv = t.decompress_kv(ck, cv)
+    assert rk is k and rv is v
+    with pytest.raises(RuntimeError):          # no CPU fallback
+        t.compress_kv(torch.randn(1, 2, 17, 128), torch.randn(1, 2, 17, 128))
+    with pytest.raises(ValueError):            # non-4-D input, like the reference's tuple unpack
+        t.key_compressor.compress(torch.randn(4, 128))
+    wide = pkg.MSECompressor(128, 9, seed=1, device="cpu")   # constructs, like the reference ...
+    with pytest.raises(ZeroDivisionError):                     # ... and fails at 8 // bits in compress
+        wide.compress(torch.randn(1, 1, 4, 128))
+
+
+def test_c_abi_argument_errors(pkg):
+    lib = pkg._native.lib()
+    E = {k: v for k, v in (("NULL", -1), ("BITS", -2), ("HEAD_DIM", -3), ("DTYPE", -4), ("SIZE", -5),
+                           ("CODEBOOK", -6), ("TABLE", -7), ("ALIGN", -8))}
+    assert lib.tq_bytes_per_vector(128, 4) == 64 and lib.tq_bytes_per_vector(128, 3) == 64
+    assert lib.tq_bytes_per_vector(128, 6) == 128 and lib.tq_bytes_per_vector(128, 1) == 16
+    assert lib.tq_bytes_per_vector(6, 2) == 2
+    assert lib.tq_bytes_per_vector(128, 0) == E["BITS"] and lib.tq_bytes_per_vector(128, 9) == E["BITS"]
+    assert lib.tq_table_bytes(64, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(128, 9) == E["BITS"]
+    cent = np.array([0.1, -0.1], np.float32)
+    thr = np.zeros(1, np.float32)
+    assert lib.tq_decision_thresholds(cent.ctypes.data, 2, thr.ctypes.data) == E["CODEBOOK"]
+    assert lib.tq_decision_thresholds(None, 2, thr.ctypes.data) == E["NULL"]
+    pi = np.eye(128, dtype=np.float32)
+    good = np.array([-0.1, 0.1], np.float32)
+    blob = np.zeros(lib.tq_table_bytes(128, 1), np.uint8)
+    assert lib.tq_table_build(pi.ctypes.data, good.ctypes.data, 128, 1, blob.ctypes.data, 16) == E["SIZE"]
+    assert lib.tq_table_build(pi.ctypes.data, cent.ctypes.data, 128, 1, blob.ctypes.data, blob.size) == E["CODEBOOK"]
+    assert lib.tq_table_build(pi.ctypes.data, good.ctypes.data, 128, 1, blob.ctypes.data, blob.size) == 0
+    bad = np.zeros(256, np.uint8)
+    out = np.zeros(1, np.uint8)
+    assert lib.tq_table_quantize_host(bad.ctypes.data, thr.ctypes.data, 1, out.ctypes.data) == E["TABLE"]
+    # launch entry points validate before touching the device
+    buf = np.zeros(4096, np.uint8)
+    p = buf.ctypes.data + (-buf.ctypes.data) % 16
+    args = dict(rows=1, tokens=4, rs=0, ts=128)
+    call = lambda states, dtype, bits, hd, idx=p, norms=p, table=p, **kw: lib.tq_compress(
+        states, dtype, kw.get("rows", 1), kw.get("tokens", 4), kw.get("rs", 0), kw.get("ts", 128), table, hd, bits,
+        idx, norms, None)
+    assert call(p, 1, 0, 128) == E["BITS"]
+    assert call(p, 1, 4, 64) == E["HEAD_DIM"]
+    assert call(p, 7, 4, 128) == E["DTYPE"]
+    assert call(None, 1, 4, 128) == E["NULL"]
+    assert call(p + 2, 1, 4, 128) == E["ALIGN"]
+    assert call(p, 1, 4, 128, ts=100) == E["SIZE"]
+    assert call(p, 1, 4, 128, tokens=-1) == E["SIZE"]
+    assert call(p, 1, 4, 128, ts=132) == E["ALIGN"]
+    assert call(None, 1, 4, 128, tokens=0) == 0          # empty input: nothing to do, not an error
+    assert lib.tq_decompress(p, p, 1, 4, p, 128, 9, p, 0, 0, 128, None) == E["BITS"]
+    assert lib.tq_decompress(p, p, 1, 4, p, 128, 4, None, 0, 0, 128, None) == E["NULL"]
+    assert lib.tq_decompress(p, p, 1, 0, p, 128, 4, None, 0, 0, 128, None) == 0
+    assert lib.tq_compress_batched(None, None, 0, 128, None) == 0
+    assert lib.tq_compress_batched(None, None, 3, 128, None) == E["NULL"]
+
+
+def test_vector_layout_reduction(pkg):
+    vl = pkg._native.vector_layout
+    x = torch.zeros(2, 3, 40, 128, dtype=torch.float16)
+    assert vl(x) == (1, 240, 0, 128)
+    assert vl(x[:, :, :24]) == (6, 24, 40 * 128, 128)
+    assert vl(x[:, :, 24:]) == (6, 16, 40 * 128, 128)
+    assert vl(x[:1, :, :24]) == (3, 24, 40 * 128, 128)
+    hf = torch.zeros(1, 40, 3, 128, dtype=torch.float16).transpose(1, 2)      # [B,S,H,D] storage, B = 1
+    assert vl(hf) == (3, 40, 128, 384)
+    assert vl(torch.zeros(2, 40, 3, 128).transpose(1, 2)) is None            # three stride levels
+    assert vl(torch.zeros(1, 1, 0, 128)) == (0, 0, 0, 128)
+    assert vl(torch.zeros(2, 3, 40, 130, dtype=torch.float16)[..., :128]) is None   # rows not 16-byte aligned

@@ -1,0 +1,231 @@
+"""The CPU oracle against the reference's own outputs and against what the mathematics fixes.
+
+Nothing here needs a GPU.  Two independent restatements (numpy op-sequence, scalar C) are checked
+against tests/golden/*.npz (written by the real reference), against each other, against exhaustive
+enumeration of the packing and brute-force nearest-centroid search.
+"""
+import hashlib
+
+import numpy as np
+import pytest
+import torch
+
+BITS = (1, 2, 3, 4, 5, 6, 7, 8)
+
+
+def _cases(golden):
+    fx = golden["mse_roundtrip"]
+    for b in BITS:
+        for dn in ("f32", "f16", "bf16"):
+            if f"b{b}_{dn}_x" in fx:
+                yield b, dn
+
+
+def test_roundtrip_fixtures_numpy_bit_exact(golden, oracle):
+    """The numpy op-sequence restatement reproduces the reference's bytes, norms and fp32
+    reconstruction bit for bit on every fixture (same BLAS, same op order)."""
+    fx = golden["mse_roundtrip"]
+    n = 0
+    for b, dn in _cases(golden):
+        orc = oracle.NumpyOracle(fx[f"Pi_b{b}"], fx[f"centroids_b{b}"], b)
+        x = oracle.widen(fx[f"b{b}_{dn}_x"], dn)
+        with np.errstate(over="ignore", invalid="ignore"):
+            out = orc.compress(x)
+        ref_bytes = fx[f"b{b}_{dn}_idx_bytes"]
+        assert np.array_equal(out["idx_bytes"], ref_bytes.reshape(-1, ref_bytes.shape[-1])), (b, dn)
+        assert np.array_equal(out["vec_norms"], fx[f"b{b}_{dn}_vec_norms"].reshape(-1)), (b, dn)
+        rec = orc.decompress(ref_bytes, fx[f"b{b}_{dn}_vec_norms"])
+        assert np.array_equal(rec.view(np.uint32), fx[f"b{b}_{dn}_recon"].reshape(-1, 128).view(np.uint32)), (b, dn)
+        n += 1
+    assert n == 20
+
+
+@pytest.mark.parametrize("accum_double", [False, True])
+def test_roundtrip_fixtures_c(golden, oracle, accum_double):
+    """The scalar C restatement: same codes except inside the 1e-5 boundary window (none seen),
+    norms within one fp16 ulp, reconstruction to fp32 rounding."""
+    fx = golden["mse_roundtrip"]
+    for b, dn in _cases(golden):
+        cent = fx[f"centroids_b{b}"]
+        orc = oracle.COracle(fx[f"Pi_b{b}"], cent, b, accum_double)
+        x = oracle.widen(fx[f"b{b}_{dn}_x"], dn)
+        out = orc.compress(x)
+        ref_bytes = fx[f"b{b}_{dn}_idx_bytes"]
+        ref_bytes = ref_bytes.reshape(-1, ref_bytes.shape[-1])
+        rep = oracle.code_mismatch_report(out["idx_bytes"], ref_bytes, out["rotated"], cent, b)
+        assert rep["outside_window"] == 0, (b, dn, rep)
+        assert rep["differ"] <= 2, (b, dn, rep)
+        ulp = oracle.fp16_ulp_distance(out["vec_norms"], fx[f"b{b}_{dn}_vec_norms"].reshape(-1))
+        assert ulp.max() <= 1
+        rec = orc.decompress(ref_bytes, fx[f"b{b}_{dn}_vec_norms"].reshape(-1))
+        ref = fx[f"b{b}_{dn}_recon"].reshape(-1, 128)
+        finite = np.isfinite(ref).all(-1)
+        assert np.array_equal(np.isfinite(rec).all(-1), finite)
+        rel = np.linalg.norm(rec[finite] - ref[finite]) / np.linalg.norm(ref[finite])
+        assert rel < 1e-6, (b, dn, rel)
+
+
+def test_config1_known_answer(golden, oracle):
+    """BASELINE config 1 (K [1,8,1024,128] fp32 N(0,1) seed 0, 4-bit, rotation seed 42): the
+    reference's SHA-256 of packed bytes, norms and reconstruction, its MSE and cosine."""
+    meta = golden["json"]["config1"]
+    torch.manual_seed(0)
+    k = torch.randn(1, 8, 1024, 128).numpy()
+    assert hashlib.sha256(k.tobytes()).hexdigest() == meta["input_sha256"]
+    Pi = golden["rotations"]["Pi_d128_s42"]
+    cent = golden["codebooks"]["centroids_d128_b4"]
+    ref_bytes = golden["config1"]["idx_bytes"].reshape(-1, 64)
+    ref_norms = golden["config1"]["vec_norms"].reshape(-1)
+    assert meta["packed_bytes"] == ref_bytes.size + 2 * ref_norms.size == 540672
+
+    out = oracle.NumpyOracle(Pi, cent, 4).compress(k)
+    assert hashlib.sha256(out["idx_bytes"].tobytes()).hexdigest() == meta["idx_bytes_sha256"]
+    assert hashlib.sha256(out["vec_norms"].tobytes()).hexdigest() == meta["vec_norms_sha256"]
+    rec = oracle.NumpyOracle(Pi, cent, 4).decompress(ref_bytes, ref_norms)
+    assert hashlib.sha256(rec.tobytes()).hexdigest() == meta["recon_sha256"]
+    flat = k.reshape(-1, 128)
+    mse = float(((flat - rec) ** 2).mean())
+    cos = (flat * rec).sum(-1) / (np.linalg.norm(flat, axis=-1) * np.linalg.norm(rec, axis=-1))
+    assert abs(mse - meta["mse_per_element"]) < 1e-7
+    assert abs(float(cos.mean()) - meta["cosine_mean"]) < 1e-6
+    # textbook 4-bit Gaussian Lloyd-Max distortion is 0.009497 per unit variance
+    assert 0.0090 < meta["rel_mse"] < 0.0098
+
+    for dbl in (False, True):
+        c = oracle.COracle(Pi, cent, 4, dbl).compress(k)
+        rep = oracle.code_mismatch_report(c["idx_bytes"], ref_bytes, c["rotated"], cent, 4)
+        assert rep["outside_window"] == 0 and rep["differ"] <= 8, rep
+        assert oracle.fp16_ulp_distance(c["vec_norms"], ref_norms).max() <= 1
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_pack_unpack_exhaustive(oracle, bits):
+    """Closed form of the packing: byte = sum code_k << bits*(ipb-1-k), MSB first; every byte value
+    decodes and re-encodes to itself (masked to the used bits); C and numpy agree."""
+    ipb = 8 // bits
+    used = (1 << (bits * ipb)) - 1
+    D = 128
+    G = -(-D // ipb)
+    assert oracle.bytes_per_vector(D, bits) == G == {1: 16, 2: 32, 3: 64, 4: 64}.get(bits, 128)
+    npo = oracle.NumpyOracle(np.eye(D, dtype=np.float32), np.zeros(1 << bits, np.float32), bits)
+    lib = oracle._load()
+    # all 256 byte values in every byte position class
+    allbytes = ((np.arange(256)[:, None] + 37 * np.arange(G)[None, :]) % 256).astype(np.uint8)
+    codes = npo.unpack(allbytes)
+    assert codes.shape == (256, D) and codes.max() <= (1 << bits) - 1
+    assert np.array_equal(npo.pack(codes), allbytes & used)
+    for row in range(0, 256, 17):
+        c_codes = np.empty(D, np.uint8)
+        lib.tqo_unpack(np.ascontiguousarray(allbytes[row]), D, bits, c_codes)
+        assert np.array_equal(c_codes, codes[row])
+        c_bytes = np.empty(G, np.uint8)
+        lib.tqo_pack(c_codes, D, bits, c_bytes)
+        assert np.array_equal(c_bytes, allbytes[row] & used)
+    # hand-computed example: codes 1,2,3,... -> first byte
+    seq = (np.arange(D) % (1 << bits)).astype(np.uint8)
+    first = 0
+    for k in range(ipb):
+        first |= int(seq[k]) << (bits * (ipb - 1 - k))
+    assert npo.pack(seq[None])[0, 0] == first
+
+
+def test_pack_with_padding(oracle):
+    """head_dim not a multiple of ipb: zero padding at the end (compressors_v3.py:65-68)."""
+    npo = oracle.NumpyOracle(np.eye(6, dtype=np.float32), np.zeros(4, np.float32), 2)
+    codes = np.array([[3, 2, 1, 0, 1, 2]], dtype=np.uint8)
+    packed = npo.pack(codes)
+    assert packed.tolist() == [[0b11100100, 0b01100000]]
+    assert np.array_equal(npo.unpack(packed), codes)
+    c = np.empty(2, np.uint8)
+    oracle._load().tqo_pack(np.ascontiguousarray(codes[0]), 6, 2, c)
+    assert c.tolist() == [0b11100100, 0b01100000]
+
+
+@pytest.mark.parametrize("bits", (1, 2, 4, 8))
+def test_nearest_bruteforce(golden, oracle, bits):
+    """argmin with first-minimum ties: C loop == numpy argmin == literal Python on tiny inputs."""
+    cent = golden["codebooks"][f"centroids_d128_b{bits}"]
+    rng = np.random.default_rng(bits)
+    r = rng.normal(0, 0.1, 4000).astype(np.float32)
+    mids = ((cent[:-1].astype(np.float64) + cent[1:]) / 2).astype(np.float32)
+    r = np.concatenate([r, cent, mids, np.nextafter(mids, np.float32(1)), np.nextafter(mids, np.float32(-1)),
+                        np.array([0.0, -0.0, 1.0, -1.0], np.float32)])
+    got = np.empty(r.size, np.uint8)
+    oracle._load().tqo_nearest(r, r.size, cent, cent.size, got)
+    ref = np.abs(r[:, None] - cent[None, :]).argmin(-1)
+    assert np.array_equal(got, ref)
+    for i in range(0, r.size, 97):
+        best, bd = 0, abs(np.float32(r[i] - cent[0]))
+        for j in range(1, cent.size):
+            d = abs(np.float32(r[i] - cent[j]))
+            if d < bd:
+                best, bd = j, d
+        assert best == got[i]
+    # exact ties go to the lower index
+    two = np.array([-0.5, 0.5], np.float32)
+    t = np.empty(1, np.uint8)
+    oracle._load().tqo_nearest(np.zeros(1, np.float32), 1, two, 2, t)
+    assert t[0] == 0
+
+
+def test_fp16_conversion_matches_numpy(oracle):
+    """The C oracle's fp16 rounding == numpy's (round to nearest even, overflow to inf, subnormals)."""
+    rng = np.random.default_rng(0)
+    x = np.concatenate([
+        rng.normal(0, 1, 20000).astype(np.float32) * np.float32(10) ** rng.integers(-9, 6, 20000).astype(np.float32),
+        np.array([0, -0.0, 65504, 65519.99, 65520, 70000, 1e-8, 5.96e-8, 2.98e-8, 2.9802325e-8, 6.1e-5, np.inf, -np.inf],
+                 np.float32)])
+    out = np.empty(x.size, np.uint16)
+    oracle._load().tqo_f32_to_f16(x, out, x.size)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(out, x.astype(np.float16).view(np.uint16))
+    allh = np.arange(65536, dtype=np.uint16)
+    back = np.empty(65536, np.float32)
+    oracle._load().tqo_f16_to_f32(allh, back, 65536)
+    ref = allh.view(np.float16).astype(np.float32)
+    ok = np.isnan(ref) | (back.view(np.uint32) == ref.view(np.uint32))
+    assert ok.all()
+
+
+def test_norm_has_no_epsilon_and_unit_scale(golden, oracle):
+    """The stored norm is the plain L2 norm in fp16 (eps only in the divisor); scaling a vector by
+    a power of two leaves its codes unchanged and scales the norm (linearity / invariance)."""
+    Pi = golden["rotations"]["Pi_d128_s42"]
+    cent = golden["codebooks"]["centroids_d128_b4"]
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 1, (64, 128)).astype(np.float32)
+    for orc in (oracle.NumpyOracle(Pi, cent, 4), oracle.COracle(Pi, cent, 4)):
+        a = orc.compress(x)
+        b = orc.compress(x * np.float32(4))
+        assert np.array_equal(a["idx_bytes"], b["idx_bytes"])
+        na = a["vec_norms"].view(np.float16).astype(np.float32)
+        nb = b["vec_norms"].view(np.float16).astype(np.float32)
+        assert np.array_equal(na * 4, nb)
+        assert np.abs(na - np.linalg.norm(x, axis=-1)).max() < 0.01
+        # identity rotation + one-hot input: the hot coordinate gets the top code, the rest the
+        # code nearest to zero
+    eye = np.eye(128, dtype=np.float32)
+    onehot = np.zeros((1, 128), np.float32)
+    onehot[0, 5] = 2.0
+    out = oracle.COracle(eye, cent, 4).compress(onehot)
+    codes = oracle.unpack_codes(out["idx_bytes"], 128, 4)[0]
+    assert codes[5] == 15 and set(np.delete(codes, 5)) == {7}
+    assert out["vec_norms"].view(np.float16)[0] == np.float16(2.0)
+
+
+def test_decompress_inverts_rotation(golden, oracle):
+    """Orthogonality: decompress(codes) = (centroids[codes] @ Pi) * norm, so rotating it back
+    returns the centroids; checked against a float64 evaluation."""
+    Pi = golden["rotations"]["Pi_d128_s542"]
+    cent = golden["codebooks"]["centroids_d128_b2"]
+    rng = np.random.default_rng(9)
+    codes = rng.integers(0, 4, (32, 128)).astype(np.uint8)
+    npo = oracle.NumpyOracle(Pi, cent, 2)
+    packed = npo.pack(codes)
+    norms = np.full(32, np.float16(3.0)).view(np.uint16)
+    ref = (cent[codes].astype(np.float64) @ Pi.astype(np.float64)) * 3.0
+    for orc in (npo, oracle.COracle(Pi, cent, 2), oracle.COracle(Pi, cent, 2, True)):
+        rec = orc.decompress(packed, norms)
+        assert np.abs(rec - ref).max() < 2e-6
+        back = (rec.astype(np.float64) / 3.0) @ Pi.astype(np.float64).T
+        assert np.abs(back - cent[codes]).max() < 2e-6

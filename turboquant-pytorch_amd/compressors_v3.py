@@ -55,7 +55,8 @@ class MSECompressor:
         self.Pi = pi_host.to(device)
         self.centroids = cent_host.to(device)
         # Everything the kernels read, baked once: split rotation tiles, quantiser grid, decode tables.
-        self._table_host = _native.build_table(pi_host, cent_host, bits)
+        # (above 8 bits the reference constructs fine and fails in compress(); keep that order)
+        self._table_host = _native.build_table(pi_host, cent_host, bits) if 1 <= bits <= 8 else None
         self._table = None
 
     @classmethod
@@ -99,7 +100,8 @@ class MSECompressor:
     def decompress(self, compressed: dict) -> torch.Tensor:
         """Back to a float32 (B, H, S, D) tensor."""
         B, H, S, D = compressed["shape"]
-        idx_bytes = compressed["idx_bytes"].reshape(B, H, S, -1)
+        width = math.ceil(D / (8 // self.bits))
+        idx_bytes = compressed["idx_bytes"].reshape(B, H, S, width)
         vec_norms = compressed["vec_norms"].reshape(B, H, S)
         return torch.ops.tqamd.decompress(idx_bytes, vec_norms, self.table(), self.bits, D, torch.float32)
 
@@ -109,7 +111,8 @@ class MSECompressor:
         B, H, S, D = compressed["shape"]
         if tuple(out.shape) != (B, H, S, D):
             raise ValueError(f"output shape {tuple(out.shape)} does not match compressed shape {(B, H, S, D)}")
-        torch.ops.tqamd.decompress_into(compressed["idx_bytes"].reshape(B, H, S, -1),
+        width = math.ceil(D / (8 // self.bits))
+        torch.ops.tqamd.decompress_into(compressed["idx_bytes"].reshape(B, H, S, width),
                                         compressed["vec_norms"].reshape(B, H, S), self.table(), self.bits, out)
         return out
 

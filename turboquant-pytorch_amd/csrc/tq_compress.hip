@@ -47,12 +47,18 @@ __device__ __forceinline__ tq_f16v mfma_bf16(tq_u4 a, tq_u4 b, tq_f16v c) {
 // sum of squares of the eight 16-bit values in v, added to acc (fp32)
 template <int DTYPE>
 __device__ __forceinline__ float sumsq8(tq_u4 v, float acc) {
+    if constexpr (DTYPE == TQ_F16) {
+        // (pairs are taken from the whole-vector cast: casting one 32-bit element of `v` to a
+        // half pair made the compiler read element 0 four times)
+        const tq_half8 h8 = __builtin_bit_cast(tq_half8, v);
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        if (DTYPE == TQ_F16) {
-            const tq_half2 h = __builtin_bit_cast(tq_half2, v[d]);
+        for (int d = 0; d < 4; ++d) {
+            const tq_half2 h = {h8[2 * d], h8[2 * d + 1]};
             acc = __builtin_amdgcn_fdot2(h, h, acc, false);
-        } else {
+        }
+    } else {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
             const float lo = __uint_as_float(v[d] << 16), hi = __uint_as_float(v[d] & 0xffff0000u);
             acc = fmaf(lo, lo, acc);
             acc = fmaf(hi, hi, acc);
@@ -293,10 +299,7 @@ int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uin
         configured[dev] = true;
     }
     const uint32_t want = (max_tiles + T::WAVES - 1) / T::WAVES;
-    uint32_t per_job = (uint32_t)((info.cus * 2 + n_jobs - 1) / n_jobs);
-    if (n_jobs == 1) per_job = (uint32_t)info.cus;
-    uint32_t bx = want < per_job ? want : per_job;
-    if (bx == 0) bx = 1;
+    const uint32_t bx = tq_blocks_per_job(want, info.cus, n_jobs);
     dim3 grid(bx, (unsigned)n_jobs, 1), block(T::WAVES * TQ_WAVE, 1, 1);
     hipLaunchKernelGGL((tq_compress_kernel<DTYPE, BITS>), grid, block, lds, stream, job, jobs_dev);
     return (int)hipGetLastError();

@@ -243,10 +243,7 @@ int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, u
         configured[dev] = true;
     }
     const uint32_t want = (max_tiles + T::WAVES - 1) / T::WAVES;
-    uint32_t per_job = (uint32_t)((cus * 2 + n_jobs - 1) / n_jobs);
-    if (n_jobs == 1) per_job = (uint32_t)cus;
-    uint32_t bx = want < per_job ? want : per_job;
-    if (bx == 0) bx = 1;
+    const uint32_t bx = tq_blocks_per_job(want, cus, n_jobs);
     dim3 grid(bx, (unsigned)n_jobs, 1), block(T::WAVES * TQ_WAVE, 1, 1);
     hipLaunchKernelGGL((tq_decompress_kernel<DTYPE, IPB>), grid, block, lds, stream, job, jobs_dev);
     return (int)hipGetLastError();

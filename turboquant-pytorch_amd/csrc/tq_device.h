@@ -51,3 +51,23 @@ __device__ __forceinline__ tq_f16v tq_zero16() {
     for (int i = 0; i < 16; ++i) z[i] = 0.f;
     return z;
 }
+
+// Blocks per job for a (blocks_per_job x n_jobs) grid of equal-cost blocks on `cus` compute units
+// that hold one block each: enough blocks to fill the device a few times over, with the total as
+// close to a whole number of device-wide rounds as possible (a partial last round idles CUs).
+static inline uint32_t tq_blocks_per_job(uint32_t want, int cus, int n_jobs) {
+    if (n_jobs <= 1) return want < (uint32_t)cus ? (want ? want : 1u) : (uint32_t)cus;
+    uint32_t best = 1;
+    double best_waste = 1e30;
+    for (int rounds = 1; rounds <= 8; ++rounds) {
+        uint32_t per_job = (uint32_t)((long long)cus * rounds / n_jobs);
+        if (per_job == 0) continue;
+        if (per_job > want) per_job = want ? want : 1u;
+        const long long total = (long long)per_job * n_jobs;
+        const long long padded = (total + cus - 1) / cus * cus;
+        const double waste = (double)(padded - total) / (double)total;
+        if (waste < best_waste - 1e-9) { best_waste = waste; best = per_job; }
+        if (per_job >= want) break;
+    }
+    return best;
+}
