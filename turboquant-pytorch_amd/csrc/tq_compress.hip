@@ -34,7 +34,7 @@ template <> struct InTraits<TQ_F32> {
 template <int DTYPE>
 constexpr size_t compress_lds_bytes() {
     using T = InTraits<DTYPE>;
-    return (size_t)T::TERMS * TQ_OPERAND_BYTES + TQ_GRID_LDS_BYTES + (size_t)T::WAVES * 32 * TQ_HEAD_DIM * T::ELEM;
+    return (size_t)T::TERMS * TQ_OPERAND_BYTES + (size_t)T::WAVES * 32 * TQ_HEAD_DIM * T::ELEM;   // dynamic part
 }
 
 __device__ __forceinline__ tq_f16v mfma_f16(tq_u4 a, tq_u4 b, tq_f16v c) {
@@ -44,12 +44,12 @@ __device__ __forceinline__ tq_f16v mfma_bf16(tq_u4 a, tq_u4 b, tq_f16v c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(tq_bf8, a), __builtin_bit_cast(tq_bf8, b), c, 0, 0, 0);
 }
 
-// sum of squares of the eight 16-bit values in v, added to acc (fp32)
+// sum of squares of the eight 16-bit values in v, added to acc (fp32).
+// (Pairs are taken from the whole-vector cast: casting one 32-bit element of `v` to a 16-bit
+// pair made the compiler read element 0 four times.)
 template <int DTYPE>
 __device__ __forceinline__ float sumsq8(tq_u4 v, float acc) {
     if constexpr (DTYPE == TQ_F16) {
-        // (pairs are taken from the whole-vector cast: casting one 32-bit element of `v` to a
-        // half pair made the compiler read element 0 four times)
         const tq_half8 h8 = __builtin_bit_cast(tq_half8, v);
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -57,11 +57,11 @@ __device__ __forceinline__ float sumsq8(tq_u4 v, float acc) {
             acc = __builtin_amdgcn_fdot2(h, h, acc, false);
         }
     } else {
+        const tq_bf8 b8 = __builtin_bit_cast(tq_bf8, v);
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-            const float lo = __uint_as_float(v[d] << 16), hi = __uint_as_float(v[d] & 0xffff0000u);
-            acc = fmaf(lo, lo, acc);
-            acc = fmaf(hi, hi, acc);
+            const tq_bf2 b = {b8[2 * d], b8[2 * d + 1]};
+            acc = __builtin_amdgcn_fdot2_f32_bf16(b, b, acc, false);
         }
     }
     return acc;
@@ -87,32 +87,59 @@ __device__ __forceinline__ void split_f32x8(const float (&x)[8], tq_u4 &t0, tq_u
     }
 }
 
+// ---- packing geometry -------------------------------------------------------------------
+// A lane owns 64 consecutive codes = NB packed bytes = NB/4 dwords.  Inside a dword, code number
+// i (in the order "byte 3 first, most significant code of the byte first") sits at bit
+// shift(i); FIELD is the spacing the sign-collecting funnel shift uses.
+template <int BITS> struct Pack {
+    static constexpr int IPB = 8 / BITS;                 // codes per byte
+    static constexpr int CPD = 4 * IPB;                  // codes per dword
+    static constexpr int NB = 64 / IPB;                  // bytes per lane
+    static constexpr int FIELD = IPB == 1 ? 8 : BITS;    // bits the funnel shift advances per code
+    static constexpr int COPIES = TQ_GRID_COPIES(BITS);
+    static constexpr int COPY_STRIDE = TQ_GRID_COPY_STRIDE(BITS);
+    // i-th code in descending bit position
+    static constexpr int byte_of(int i) { return 3 - i / IPB; }
+    static constexpr int k_of(int i) { return i % IPB; }
+    static constexpr int shift_of(int i) { return 8 * byte_of(i) + BITS * (IPB - 1 - k_of(i)); }
+    static constexpr int local_code(int w, int i) { return w * CPD + byte_of(i) * IPB + k_of(i); }
+    // grid copy used for a code at bit position `shift`: its base is pre-shifted by copy_shift
+    static constexpr int copy_of(int i) {
+        return IPB == 1 ? (byte_of(i) & 1) : byte_of(i) * IPB + (IPB - 1 - k_of(i));
+    }
+    static constexpr int copy_shift(int c) {   // shift baked into copy c
+        return IPB == 1 ? 8 * c : 8 * (c / IPB) + BITS * (c % IPB);
+    }
+    static constexpr uint32_t sign_mask() {
+        uint32_t m = 0;
+        for (int i = 0; i < CPD; ++i) m |= 1u << (shift_of(i) + FIELD - 1);
+        return m;
+    }
+};
+
+template <int BITS>
+__device__ __forceinline__ uint32_t copy_shift_rt(uint32_t c) {
+    constexpr int IPB = 8 / BITS;
+    return IPB == 1 ? 8u * c : 8u * (c / IPB) + (uint32_t)BITS * (c % IPB);
+}
+
 template <int DTYPE, int BITS>
 __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_kernel(TqDevJob job0, const tq_job *jobs) {
     using T = InTraits<DTYPE>;
+    using P = Pack<BITS>;
     constexpr int ELEM = T::ELEM;
     constexpr int VEC_BYTES = TQ_HEAD_DIM * ELEM;      // 256 or 512
     constexpr int STAGE = 32 * VEC_BYTES;              // wave-private tile buffer
     constexpr int NLOAD = STAGE / 1024;                // 16-byte loads per lane per tile
     constexpr int PIECES = VEC_BYTES / 16;             // 16-byte pieces per vector
     constexpr int VEC_PER_LOAD = 64 / PIECES;          // vectors covered by one load instruction
-    constexpr int IPB = 8 / BITS;                      // codes per byte
-    constexpr int NB = 64 / IPB;                       // packed bytes per lane (half a vector)
+    constexpr int NB = P::NB;
 
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // grid copies first (static, so that their LDS addresses are compile-time immediates)
+    __shared__ __attribute__((aligned(16))) uint8_t lds_grid[TQ_GRID_LDS_BYTES];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_dyn[];
 
-    TqDevJob job = job0;
-    if (jobs) {
-        const tq_job &j = jobs[blockIdx.y];
-        job.states = static_cast<const uint8_t *>(j.states);
-        job.idx_bytes = j.idx_bytes;
-        job.vec_norms = j.vec_norms;
-        job.table = static_cast<const uint8_t *>(j.table_dev);
-        job.n_vec = (uint32_t)(j.rows * j.tokens);
-        job.tokens = (uint32_t)j.tokens;
-        job.row_stride = j.row_stride;
-        job.token_stride = j.token_stride;
-    }
+    const TqDevJob job = tq_load_job(job0, jobs, blockIdx.y, ELEM);
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
@@ -121,13 +148,21 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
     if (blockIdx.x * T::WAVES >= n_tiles) return;  // whole block idle (uniform)
 
     const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
-    uint8_t *lds_a = lds;
-    uint8_t *lds_grid = lds + T::TERMS * TQ_OPERAND_BYTES;
-    uint8_t *stage = lds_grid + TQ_GRID_LDS_BYTES + wave * STAGE;
+    uint8_t *lds_a = lds_dyn;
+    uint8_t *stage = lds_dyn + T::TERMS * TQ_OPERAND_BYTES + wave * STAGE;
 
     tq_copy_to_lds(lds_a, job.table + (DTYPE == TQ_F16 ? hd->off_a_f16 : hd->off_a_bf16),
                    T::TERMS * TQ_OPERAND_BYTES, tid, T::WAVES * TQ_WAVE);
-    tq_copy_to_lds(lds_grid, job.table + hd->off_grid, (hd->grid_cells * 8u + 15u) & ~15u, tid, T::WAVES * TQ_WAVE);
+    {   // one grid copy per code position, base pre-shifted
+        const uint32_t cells = hd->grid_cells;
+        const uint8_t *src = job.table + hd->off_grid;
+        for (uint32_t i = tid; i < cells * P::COPIES; i += T::WAVES * TQ_WAVE) {
+            const uint32_t c = i / cells, q = i - c * cells;
+            tq_u2 e = tq_gload8(src + 8u * q);
+            e[1] <<= copy_shift_rt<BITS>(c);
+            *reinterpret_cast<tq_u2 *>(lds_grid + c * P::COPY_STRIDE + 8u * q) = e;
+        }
+    }
     const float grid_scale = hd->grid_scale, grid_bias = hd->grid_bias;
     __syncthreads();
 
@@ -136,28 +171,42 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
 
     const uint32_t ld_vec = lane / PIECES, ld_piece = lane % PIECES;  // role in the coalesced loads
     const uint32_t n = lane & 31u, hk = lane >> 5;                    // role in the MFMA: column, half
+    const bool one_row = job.tokens >= job.n_vec;
 
     tq_u4 pre[NLOAD];
     auto issue_loads = [&](uint32_t tl) {
+        const uint32_t v0 = tl * 32u + ld_vec;
+        if (one_row && tl * 32u + 32u <= job.n_vec) {
+            // full tile of a single row: one 64-bit base, constant steps
+            const uint8_t *p = job.states + (long long)v0 * job.token_stride + ld_piece * 16u;
+            const long long step = (long long)VEC_PER_LOAD * job.token_stride;
 #pragma unroll
-        for (int j = 0; j < NLOAD; ++j) {
-            const uint32_t v = tl * 32u + j * VEC_PER_LOAD + ld_vec;
-            tq_u4 val = {0u, 0u, 0u, 0u};
-            if (v < job.n_vec)
-                val = *reinterpret_cast<const tq_u4 *>(job.states + tq_vec_offset<ELEM>(job, v) + ld_piece * 16u);
-            pre[j] = val;
+            for (int j = 0; j < NLOAD; ++j) pre[j] = tq_gload16(p + j * step);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NLOAD; ++j) {
+                uint32_t v = v0 + j * VEC_PER_LOAD;
+                v = v < job.n_vec ? v : job.n_vec - 1u;   // tail: re-read the last vector, never stored
+                pre[j] = tq_gload16(job.states + tq_vec_offset(job, v) + ld_piece * 16u);
+            }
         }
     };
     if (tile < n_tiles) issue_loads(tile);
 
+    // LDS addresses that do not change from tile to tile
+    uint32_t st_off[NLOAD];
+#pragma unroll
+    for (int j = 0; j < NLOAD; ++j) {
+        const uint32_t vl = j * VEC_PER_LOAD + ld_vec;
+        const uint32_t swz = (ELEM == 2) ? (vl & 15u) : ((vl & 15u) << 1);
+        st_off[j] = vl * VEC_BYTES + ((ld_piece ^ swz) << 4);
+    }
+    const tq_u4 *a_lane = reinterpret_cast<const tq_u4 *>(lds_a) + lane;
+
     while (tile < n_tiles) {
         // ---- park the tile in LDS (swizzled so that the operand reads below are conflict free)
 #pragma unroll
-        for (int j = 0; j < NLOAD; ++j) {
-            const uint32_t vl = j * VEC_PER_LOAD + ld_vec;
-            const uint32_t swz = (ELEM == 2) ? (vl & 15u) : ((vl & 15u) << 1);
-            *reinterpret_cast<tq_u4 *>(stage + vl * VEC_BYTES + ((ld_piece ^ swz) << 4)) = pre[j];
-        }
+        for (int j = 0; j < NLOAD; ++j) *reinterpret_cast<tq_u4 *>(stage + st_off[j]) = pre[j];
         const uint32_t next = tile + tile_stride;
         if (next < n_tiles) issue_loads(next);
 
@@ -169,7 +218,7 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
 
 #pragma unroll
         for (int s = 0; s < TQ_STEPS; ++s) {
-            const tq_u4 *a_base = reinterpret_cast<const tq_u4 *>(lds_a) + (size_t)s * 64 + lane;
+            const tq_u4 *a_base = a_lane + (size_t)s * 64;
             constexpr int TILE_STRIDE = TQ_STEPS * 64;          // tq_u4 units between tiles
             constexpr int TERM_STRIDE = TQ_OPERAND_BYTES / 16;  // tq_u4 units between terms
             if constexpr (ELEM == 2) {
@@ -213,44 +262,54 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
         float ss = ss0 + ss1;
         ss += __shfl_xor(ss, 32);
         const float nrm = sqrtf(ss);
-        float inv = 1.0f / (nrm + 1e-8f);
+        // 1 / (norm + 1e-8): the reciprocal only scales the coordinates, one ulp is irrelevant
+        float inv = __builtin_amdgcn_rcpf(nrm + 1e-8f);
         if (DTYPE == TQ_F16) inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
+        const float inv_cell = inv * grid_scale;   // grid_scale is a power of two: exact
 
         // ---- code search + packing.  Lane (n, hk) holds coordinates 64*hk + 16*t + r.
+        // Per coordinate: cell address (fma, and), one 8-byte LDS lookup from the copy whose base
+        // is pre-shifted to the code's bit position, exact comparison by fma, sign bit funnelled
+        // into `lt`, bases OR-ed together.  code = base + !(rho < threshold).
         uint32_t words[NB / 4];
 #pragma unroll
-        for (int w = 0; w < NB / 4; ++w) words[w] = 0u;
+        for (int w = 0; w < NB / 4; ++w) {
+            uint32_t lt = 0u, lo = 0u, hi = 0u;
+            int cursor = 32;
 #pragma unroll
-        for (int t = 0; t < TQ_TILES; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float rot = acc[t][r] * inv;
-                const uint32_t addr = __float_as_uint(fmaf(rot, grid_scale, grid_bias)) & TQ_GRID_ADDR_MASK;
-                const TqGridCell cell = *reinterpret_cast<const TqGridCell *>(lds_grid + addr);
-                const uint32_t code = cell.base + (rot >= cell.threshold ? 1u : 0u);
-                const int c = 16 * t + r;            // local coordinate 0..63
-                const int byte = c / IPB;            // local byte
-                const int k = c % IPB;               // position inside the byte, MSB first
-                const int shift = 8 * (byte % 4) + BITS * (IPB - 1 - k);
-                words[byte / 4] |= code << shift;
+            for (int i = 0; i < P::CPD; ++i) {
+                const int c = P::local_code(w, i);
+                const float a = acc[c / 16][c % 16];
+                const uint32_t addr = __float_as_uint(fmaf(a, inv_cell, grid_bias)) & TQ_GRID_ADDR_MASK;
+                const tq_u2 cell = *reinterpret_cast<const tq_u2 *>(lds_grid + P::copy_of(i) * P::COPY_STRIDE + addr);
+                const float t = fmaf(a, inv, -__uint_as_float(cell[0]));
+                const int gap = cursor - (P::shift_of(i) + P::FIELD);
+                if (gap > 0) lt = __builtin_amdgcn_alignbit(lt, 0u, 32 - gap);
+                lt = __builtin_amdgcn_alignbit(lt, __float_as_uint(t), 32 - P::FIELD);
+                cursor = P::shift_of(i);
+                if (P::IPB == 1 && P::byte_of(i) >= 2) hi |= cell[1]; else lo |= cell[1];
             }
+            const uint32_t bases = P::IPB == 1 ? (lo | (hi << 16)) : lo;
+            const uint32_t ge = (~lt & P::sign_mask()) >> (P::FIELD - 1);
+            words[w] = bases + ge;
+        }
 
         const uint32_t v = tile * 32u + n;
         if (v < job.n_vec) {
             uint8_t *dst = job.idx_bytes + (size_t)v * (2 * NB) + hk * NB;
-            if (NB == 8) {
+            if constexpr (NB == 8) {
                 tq_u2 o = {words[0], words[1]};
-                *reinterpret_cast<tq_u2 *>(dst) = o;
+                tq_gstore8(dst, o);
             } else {
 #pragma unroll
                 for (int q = 0; q < NB / 16; ++q) {
                     tq_u4 o = {words[4 * q], words[4 * q + 1], words[4 * q + 2], words[4 * q + 3]};
-                    *reinterpret_cast<tq_u4 *>(dst + 16 * q) = o;
+                    tq_gstore16(dst + 16 * q, o);
                 }
             }
             if (hk == 0) {
                 const _Float16 hn = (_Float16)nrm;
-                job.vec_norms[v] = __builtin_bit_cast(uint16_t, hn);
+                tq_gstore2(job.vec_norms + v, __builtin_bit_cast(uint16_t, hn));
             }
         }
         tile = next;
@@ -366,8 +425,8 @@ extern "C" int tq_compress(const void *states, int dtype, long long rows, long l
     job.table = static_cast<const uint8_t *>(table_dev);
     job.n_vec = (uint32_t)n_vec;
     job.tokens = (uint32_t)tokens;
-    job.row_stride = row_stride;
-    job.token_stride = token_stride;
+    job.row_stride = row_stride * elem_bytes(dtype);
+    job.token_stride = token_stride * elem_bytes(dtype);
     return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), static_cast<hipStream_t>(stream));
 }
 

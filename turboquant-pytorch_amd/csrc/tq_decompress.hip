@@ -81,18 +81,7 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    TqDevJob job = job0;
-    if (jobs) {
-        const tq_job &j = jobs[blockIdx.y];
-        job.states = static_cast<const uint8_t *>(j.states);
-        job.idx_bytes = j.idx_bytes;
-        job.vec_norms = j.vec_norms;
-        job.table = static_cast<const uint8_t *>(j.table_dev);
-        job.n_vec = (uint32_t)(j.rows * j.tokens);
-        job.tokens = (uint32_t)j.tokens;
-        job.row_stride = j.row_stride;
-        job.token_stride = j.token_stride;
-    }
+    const TqDevJob job = tq_load_job(job0, jobs, blockIdx.y, ELEM);
     uint8_t *out_base = const_cast<uint8_t *>(job.states);
 
     const uint32_t tid = threadIdx.x;
@@ -123,18 +112,18 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
         const uint8_t *src = job.idx_bytes + (size_t)(ok ? v : 0u) * (2 * NB) + hk * NB;
         if constexpr (NW == 2) {
             tq_u2 t = {0u, 0u};
-            if (ok) t = *reinterpret_cast<const tq_u2 *>(src);
+            if (ok) t = tq_gload8(src);
             raw[0] = t[0]; raw[1] = t[1];
         } else {
 #pragma unroll
             for (int q = 0; q < NW / 4; ++q) {
                 tq_u4 t = {0u, 0u, 0u, 0u};
-                if (ok) t = *reinterpret_cast<const tq_u4 *>(src + 16 * q);
+                if (ok) t = tq_gload16(src + 16 * q);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) raw[4 * q + i] = t[i];
             }
         }
-        norm_bits = ok ? job.vec_norms[v] : (uint16_t)0;
+        norm_bits = ok ? tq_gload2(job.vec_norms + v) : (uint16_t)0;
     };
     if (tile < n_tiles) issue_loads(tile);
 
@@ -202,7 +191,7 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
             const tq_u4 o = *reinterpret_cast<const tq_u4 *>(stage + vl * VEC_BYTES + ((st_piece ^ swz) << 4));
             const uint32_t v = tile * 32u + vl;
             if (v < job.n_vec)
-                *reinterpret_cast<tq_u4 *>(out_base + tq_vec_offset<ELEM>(job, v) + st_piece * 16u) = o;
+                tq_gstore16(out_base + tq_vec_offset(job, v) + st_piece * 16u, o);
         }
         tile = next;
     }
@@ -307,8 +296,8 @@ extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms
     job.table = static_cast<const uint8_t *>(table_dev);
     job.n_vec = (uint32_t)n_vec;
     job.tokens = (uint32_t)tokens;
-    job.row_stride = row_stride;
-    job.token_stride = token_stride;
+    job.row_stride = row_stride * elem_bytes(out_dtype);
+    job.token_stride = token_stride * elem_bytes(out_dtype);
     return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), static_cast<hipStream_t>(stream));
 }
 

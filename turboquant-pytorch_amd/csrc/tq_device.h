@@ -15,6 +15,7 @@ typedef uint32_t tq_u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t tq_u2 __attribute__((ext_vector_type(2)));
 
 #define TQ_WAVE 64
+#define TQ_GLOBAL __attribute__((address_space(1)))
 
 // Launch-time job descriptor (device view of tq_job, plus derived fields).
 struct TqDevJob {
@@ -24,25 +25,59 @@ struct TqDevJob {
     const uint8_t *table;
     uint32_t n_vec;          // rows * tokens  (< 2^31)
     uint32_t tokens;
-    long long row_stride;    // elements
-    long long token_stride;  // elements
+    long long row_stride;    // bytes
+    long long token_stride;  // bytes
 };
 
+__device__ __forceinline__ TqDevJob tq_load_job(const TqDevJob &single, const tq_job *jobs, uint32_t index, int elem_bytes) {
+    if (!jobs) return single;
+    const tq_job &j = jobs[index];
+    TqDevJob job;
+    job.states = static_cast<const uint8_t *>(j.states);
+    job.idx_bytes = j.idx_bytes;
+    job.vec_norms = j.vec_norms;
+    job.table = static_cast<const uint8_t *>(j.table_dev);
+    job.n_vec = (uint32_t)(j.rows * j.tokens);
+    job.tokens = (uint32_t)j.tokens;
+    job.row_stride = j.row_stride * elem_bytes;
+    job.token_stride = j.token_stride * elem_bytes;
+    return job;
+}
+
 // Byte offset of vector v inside `states`.
-template <int ELEM_BYTES>
 __device__ __forceinline__ long long tq_vec_offset(const TqDevJob &job, uint32_t v) {
-    if (job.tokens >= job.n_vec) return (long long)v * job.token_stride * ELEM_BYTES;  // one row
+    if (job.tokens >= job.n_vec) return (long long)v * job.token_stride;  // one row
     const uint32_t row = v / job.tokens;
     const uint32_t tok = v - row * job.tokens;
-    return ((long long)row * job.row_stride + (long long)tok * job.token_stride) * ELEM_BYTES;
+    return (long long)row * job.row_stride + (long long)tok * job.token_stride;
+}
+
+// Global-memory accessors (explicit address space: plain pointers read from a descriptor
+// would otherwise be accessed with flat instructions, which also occupy the LDS counter).
+__device__ __forceinline__ tq_u4 tq_gload16(const uint8_t *p) {
+    return *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL uint8_t *)p);
+}
+__device__ __forceinline__ tq_u2 tq_gload8(const uint8_t *p) {
+    return *reinterpret_cast<const TQ_GLOBAL tq_u2 *>((const TQ_GLOBAL uint8_t *)p);
+}
+__device__ __forceinline__ uint16_t tq_gload2(const uint16_t *p) {
+    return *((const TQ_GLOBAL uint16_t *)p);
+}
+__device__ __forceinline__ void tq_gstore16(uint8_t *p, tq_u4 v) {
+    *reinterpret_cast<TQ_GLOBAL tq_u4 *>((TQ_GLOBAL uint8_t *)p) = v;
+}
+__device__ __forceinline__ void tq_gstore8(uint8_t *p, tq_u2 v) {
+    *reinterpret_cast<TQ_GLOBAL tq_u2 *>((TQ_GLOBAL uint8_t *)p) = v;
+}
+__device__ __forceinline__ void tq_gstore2(uint16_t *p, uint16_t v) {
+    *((TQ_GLOBAL uint16_t *)p) = v;
 }
 
 // Cooperative copy global -> LDS, 16 bytes per thread per trip.
 __device__ __forceinline__ void tq_copy_to_lds(uint8_t *dst, const uint8_t *src, uint32_t bytes,
                                                uint32_t tid, uint32_t nthreads) {
-    const tq_u4 *s = reinterpret_cast<const tq_u4 *>(src);
     tq_u4 *d = reinterpret_cast<tq_u4 *>(dst);
-    for (uint32_t i = tid; i < bytes / 16; i += nthreads) d[i] = s[i];
+    for (uint32_t i = tid; i < bytes / 16; i += nthreads) d[i] = tq_gload16(src + 16u * i);
 }
 
 __device__ __forceinline__ tq_f16v tq_zero16() {

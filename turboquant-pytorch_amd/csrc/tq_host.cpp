@@ -104,7 +104,7 @@ Layout layout_for(int bits) {
     L.off_a_f16 = off;      off += 2 * TQ_OPERAND_BYTES;
     L.off_a_bf16 = off;     off += 3 * TQ_OPERAND_BYTES;
     L.off_at_f16 = off;     off += 2 * TQ_OPERAND_BYTES;
-    L.off_grid = off;       off += round_up(TQ_GRID_MAX_CELLS * sizeof(TqGridCell), 256);
+    L.off_grid = off;       off += round_up(TQ_GRID_LDS_BYTES, 256);
     L.lut_entry_bytes = 2 * ipb;
     L.off_lut = off;        off += round_up(256 * L.lut_entry_bytes, 256);
     L.off_centroids = off;  off += round_up(levels * 4, 256);
@@ -194,48 +194,33 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     std::memcpy(blob + L.off_thresholds, thr.data(), (size_t)(levels - 1) * 4);
 
     // ---- quantiser grid: smallest power-of-two resolution with <= 1 threshold per cell ----
-    const float range = 1.0625f;  // |rotated unit coordinate| <= 1 (+ rounding); cells beyond are never hit
+    // Cell k covers the reals [edge(k), edge(k+1)), edge(k) = (k - cells/2 - 1/16) / scale (see
+    // tq_table.h); unit-sphere coordinates satisfy |rho| <= 1 + rounding, the grid spans +-1.0625.
+    const double range = 1.0625;
     float scale = 0.f, bias = 0.f;
     uint32_t cells = 0;
     std::vector<TqGridCell> grid;
     bool ok = false;
-    for (int lg = 3; lg <= 10 && !ok; ++lg) {
+    for (int lg = 3; lg <= 12 && !ok; ++lg) {
         scale = (float)(1 << lg);
         cells = 2u * (uint32_t)std::ceil(range * scale);
-        if (cells > TQ_GRID_MAX_CELLS) break;
+        if (cells > (uint32_t)TQ_GRID_MAX_CELLS(bits)) break;
         bias = (float)(cells / 2) + TQ_GRID_MAGIC;
         grid.assign(cells, TqGridCell{INFINITY, 0});
-        // first float of every cell, by bisection on the monotone map r -> cell(r)
-        std::vector<float> first(cells + 1);
-        const float rmin = -(float)(cells / 2) / scale, rmax = (float)(cells / 2) / scale;
-        first[0] = -INFINITY;
-        for (uint32_t q = 1; q < cells; ++q) {
-            int64_t a = fkey(rmin), b = fkey(rmax);  // cell(rmin) = 0 < q <= cell(rmax - eps)
-            // invariant: cell(a) < q, cell(b) >= q   (b = rmax maps to `cells`, see below)
-            while (b - a > 1) {
-                const int64_t m = a + (b - a) / 2;
-                const float rm = fkey_inv(m);
-                // rmax itself maps one past the last cell; treat anything >= rmax as "beyond"
-                const uint32_t cm = rm >= rmax ? cells : grid_cell(rm, scale, bias);
-                if (cm >= q) b = m; else a = m;
-            }
-            first[q] = fkey_inv(b);
-        }
-        first[cells] = INFINITY;
+        auto edge = [&](uint32_t k) { return ((double)k - (double)(cells / 2) - 0.0625) / (double)scale; };
         ok = true;
         int t = 0;  // thresholds are ascending; walk them alongside the cells
         for (uint32_t q = 0; q < cells && ok; ++q) {
-            while (t < levels - 1 && thr[t] <= first[q]) ++t;  // counted for every r in the cell
+            const double lo = q == 0 ? -INFINITY : edge(q), hi = q + 1 == cells ? INFINITY : edge(q + 1);
+            while (t < levels - 1 && (double)thr[t] < lo) ++t;   // below the cell: counted for all of it
             grid[q].base = (uint32_t)t;
             int inside = 0;
-            while (t + inside < levels - 1 && thr[t + inside] < first[q + 1]) ++inside;
+            while (t + inside < levels - 1 && (double)thr[t + inside] < hi) ++inside;
             if (inside > 1) { ok = false; break; }
             if (inside == 1) grid[q].threshold = thr[t];
-            // the threshold inside this cell is not part of the next cell's base until passed:
-            // base of q+1 is recomputed by the first loop above.
         }
     }
-    if (!ok) return TQ_ERR_CODEBOOK;  // levels too dense for the grid
+    if (!ok) return TQ_ERR_CODEBOOK;  // levels too dense for the grid the kernels keep in LDS
     std::memcpy(blob + L.off_grid, grid.data(), (size_t)cells * sizeof(TqGridCell));
 
     // ---- rotation operands ----
@@ -322,7 +307,8 @@ int tq_table_quantize_host(const void *table_host, const float *r, long long n, 
     for (long long i = 0; i < n; ++i) {
         const uint32_t q = grid_cell(r[i], hd.grid_scale, hd.grid_bias);
         const TqGridCell c = grid[q < hd.grid_cells ? q : 0];
-        idx[i] = (uint8_t)(c.base + (r[i] >= c.threshold ? 1u : 0u));
+        // the kernels evaluate fma(acc, inv, -threshold) >= 0; with acc = r, inv = 1 that is r - threshold
+        idx[i] = (uint8_t)(c.base + (std::fmaf(r[i], 1.0f, -c.threshold) >= 0.0f ? 1u : 0u));
     }
     return TQ_OK;
 }

@@ -6,7 +6,7 @@
 #include <stdint.h>
 
 #define TQ_TABLE_MAGIC 0x54514d49u /* "TQMI" */
-#define TQ_TABLE_VERSION 3u
+#define TQ_TABLE_VERSION 4u
 #define TQ_HEAD_DIM 128
 
 // --- MFMA operand tiling (v_mfma_f32_32x32x16_{f16,bf16}) --------------------------------
@@ -28,12 +28,24 @@
 // in the fp16 normal range; the kernels fold 2^-shift into the per-vector scale.
 #define TQ_F16_PI_SHIFT 10
 
-// Quantiser grid: cell(r) = (bits(fma(r, grid_scale, grid_bias)) & TQ_GRID_ADDR_MASK) / 8,
-// entry = { float threshold; uint32 base }, code = base + (r >= threshold).
+// Quantiser grid.  With rho = acc * inv (the exact real product; acc = raw rotated coordinate,
+// inv = 1 / (norm + 1e-8)) the kernels compute
+//     cell(rho) = (bits(fma(acc, inv * grid_scale, grid_bias)) & TQ_GRID_ADDR_MASK) / 8
+//     code      = base[cell] + (fma(acc, inv, -threshold[cell]) >= 0)
+// Both fused multiply-adds see the same exact product, so cell edges are the exact reals
+// (k - cells/2 - 1/16) / grid_scale (grid_bias carries 1.5 * 2^20, one ulp = 1/8) and the
+// comparison is exact.  entry = { float threshold; uint32 base }, at most one threshold per cell.
+//
+// In LDS the kernels keep one copy of the grid per position of a code inside a 32-bit word,
+// with `base` pre-shifted to that position, at a fixed stride so that the copy is selected by
+// the immediate offset of the LDS read.
 #define TQ_GRID_ADDR_MASK 0x7ff8u
-#define TQ_GRID_MAX_CELLS 2176 /* what the kernels reserve in LDS (17 KiB) */
-#define TQ_GRID_LDS_BYTES (TQ_GRID_MAX_CELLS * 8)
+#define TQ_GRID_LDS_BYTES 18432
 #define TQ_GRID_MAGIC 1572864.0f /* 1.5 * 2^20: one ulp = 1/8 */
+// copies: one per code position in a dword (32 / bits), two for the one-code-per-byte widths
+#define TQ_GRID_COPIES(bits) ((bits) >= 5 ? 2 : (bits) == 3 ? 8 : 32 / (bits))
+#define TQ_GRID_COPY_STRIDE(bits) (TQ_GRID_LDS_BYTES / TQ_GRID_COPIES(bits))
+#define TQ_GRID_MAX_CELLS(bits) (TQ_GRID_COPY_STRIDE(bits) / 8)
 
 struct TqGridCell {
     float threshold;
