@@ -148,7 +148,8 @@ def test_table_rotation_split_reconstructs_pi(pkg, golden):
             for s in range(8):
                 for lane in range(64):
                     m, hk = lane % 32, lane // 32
-                    o = 64 * ((m // 4) % 2) + 16 * t + 4 * (m // 8) + (m % 4)
+                    h, r = (m // 4) % 2, 4 * (m // 8) + (m % 4)
+                    o = 64 * h + 16 * t + r if transpose else 32 * t + 16 * h + r
                     for i in range(8):
                         if transpose:
                             out[64 * hk + 8 * s + i, o] = a[t, s, lane, i]

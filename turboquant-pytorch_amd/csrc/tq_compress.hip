@@ -2,40 +2,40 @@
 // Replaces MSECompressor.compress (upstream turboquant/compressors_v3.py:46-81) with one kernel.
 //
 // Work decomposition (gfx950, wave64):
-//   * a wave owns a tile of 32 consecutive vectors; waves never synchronise with each other
-//     after the block-wide table load;
+//   * a block is four waves that share tiles of 32 consecutive vectors; wave w keeps the quarter
+//     of the rotation that produces coordinates [32w, 32w+32) resident in registers as MFMA A
+//     operands (all 16-bit terms of the split: 64 registers), so the matrix pipe never waits for
+//     operand loads and several waves fit on a SIMD;
 //   * the tile is fetched with fully coalesced 16-byte loads (one instruction = 1 KiB of
-//     consecutive memory), parked in a wave-private LDS buffer with an XOR swizzle, and read
-//     back as the B operand of v_mfma_f32_32x32x16 (vector n on MFMA column n);
-//   * the A operand is the rotation, pre-split on the host into 16-bit terms whose sum is Pi
-//     to ~2^-22 (fp16 path) / 2^-17 or 2^-25 (bf16 path, 2 or 3 terms); inputs are exact in
-//     the MFMA input type (fp32 inputs are split into three exact bf16 terms), accumulation is
-//     fp32, so the rotated coordinates agree with an fp32 GEMM to ~1e-7 or better;
-//   * the rotation is applied to the raw vector and divided by (norm + 1e-8) afterwards
+//     consecutive memory, a quarter of them by each wave), parked in a double-buffered,
+//     XOR-swizzled LDS buffer (one barrier per tile) and read back as the B operand of
+//     v_mfma_f32_32x32x16 (vector n on MFMA column n);
+//   * the rotation is pre-split on the host into 16-bit terms whose sum is Pi to ~2^-22 (fp16
+//     path) / 2^-17 (bf16 path); inputs are exact in the MFMA input type (fp32 inputs are split
+//     into three exact bf16 terms and use three Pi terms), accumulation is fp32, so the rotated
+//     coordinates agree with an fp32 GEMM to ~1e-6 or better;
+//   * the rotation is applied to the raw vector and scaled by 1 / (norm + 1e-8) afterwards
 //     (linearity), so the norm reduction overlaps the MFMAs;
-//   * every lane ends up with 64 consecutive rotated coordinates of one vector: the code search
-//     is one fused multiply-add, one 8-byte LDS lookup and one compare per coordinate, and the
-//     packed bytes of a lane are contiguous in memory.
+//   * every lane ends up with 16 consecutive rotated coordinates of one vector: the code search
+//     is two fused multiply-adds, one 8-byte LDS lookup and a funnel shift per coordinate, and
+//     the packed bytes of a lane are contiguous in memory;
+//   * tiles whose 32 vectors all exist take a path without per-lane predicates: a fixed number
+//     of loads and stores per iteration lets the compiler wait for the prefetched loads alone
+//     (s_waitcnt vmcnt(n)) instead of draining the previous tile's stores on every iteration.
+#include <type_traits>
+
 #include "tq_device.h"
 
 namespace {
 
 template <int DTYPE> struct InTraits;
-template <> struct InTraits<TQ_F16> {
-    static constexpr int ELEM = 2, WAVES = 8, TERMS = 2;
-};
-template <> struct InTraits<TQ_BF16> {
-    static constexpr int ELEM = 2, WAVES = 8, TERMS = 2;
-};
-template <> struct InTraits<TQ_F32> {
-    static constexpr int ELEM = 4, WAVES = 2, TERMS = 3;
-};
+template <> struct InTraits<TQ_F16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = 3; };
+template <> struct InTraits<TQ_BF16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = 3; };
+// fp32 input keeps three rotation terms resident and stages 16 KiB tiles
+template <> struct InTraits<TQ_F32> { static constexpr int ELEM = 4, TERMS = 3, MIN_WAVES = 2; };
 
-template <int DTYPE>
-constexpr size_t compress_lds_bytes() {
-    using T = InTraits<DTYPE>;
-    return (size_t)T::TERMS * TQ_OPERAND_BYTES + (size_t)T::WAVES * 32 * TQ_HEAD_DIM * T::ELEM;   // dynamic part
-}
+constexpr int CWAVES = TQ_TILES;        // waves per block = MFMA row tiles
+constexpr int CTHREADS = CWAVES * TQ_WAVE;
 
 __device__ __forceinline__ tq_f16v mfma_f16(tq_u4 a, tq_u4 b, tq_f16v c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, a), __builtin_bit_cast(tq_half8, b), c, 0, 0, 0);
@@ -88,31 +88,31 @@ __device__ __forceinline__ void split_f32x8(const float (&x)[8], tq_u4 &t0, tq_u
 }
 
 // ---- packing geometry -------------------------------------------------------------------
-// A lane owns 64 consecutive codes = NB packed bytes = NB/4 dwords.  Inside a dword, code number
-// i (in the order "byte 3 first, most significant code of the byte first") sits at bit
-// shift(i); FIELD is the spacing the sign-collecting funnel shift uses.
+// A lane owns 16 consecutive codes = NB packed bytes, handled as NW words of WB bytes (a full
+// dword, or the lane's 2 bytes for 1-bit codes).  Inside a word, code number i (in the order
+// "highest byte first, most significant code of the byte first") sits at bit shift_of(i);
+// FIELD is the spacing the sign-collecting funnel shift uses.
 template <int BITS> struct Pack {
     static constexpr int IPB = 8 / BITS;                 // codes per byte
-    static constexpr int CPD = 4 * IPB;                  // codes per dword
-    static constexpr int NB = 64 / IPB;                  // bytes per lane
+    static constexpr int NB = 16 / IPB;                  // bytes per lane: 2, 4, 8, 8, 16
+    static constexpr int WB = NB < 4 ? NB : 4;           // bytes per word
+    static constexpr int NW = NB / WB;                   // words per lane
+    static constexpr int CPW = WB * IPB;                 // codes per word
     static constexpr int FIELD = IPB == 1 ? 8 : BITS;    // bits the funnel shift advances per code
     static constexpr int COPIES = TQ_GRID_COPIES(BITS);
     static constexpr int COPY_STRIDE = TQ_GRID_COPY_STRIDE(BITS);
-    // i-th code in descending bit position
-    static constexpr int byte_of(int i) { return 3 - i / IPB; }
+    static constexpr int byte_of(int i) { return WB - 1 - i / IPB; }
     static constexpr int k_of(int i) { return i % IPB; }
     static constexpr int shift_of(int i) { return 8 * byte_of(i) + BITS * (IPB - 1 - k_of(i)); }
-    static constexpr int local_code(int w, int i) { return w * CPD + byte_of(i) * IPB + k_of(i); }
-    // grid copy used for a code at bit position `shift`: its base is pre-shifted by copy_shift
+    static constexpr int local_code(int w, int i) { return w * CPW + byte_of(i) * IPB + k_of(i); }
+    // grid copy used for the i-th code: its base is pre-shifted to the code's bit position
+    // (one-code-per-byte widths use two copies, shifts 0 and 8, and merge halves with one shift)
     static constexpr int copy_of(int i) {
         return IPB == 1 ? (byte_of(i) & 1) : byte_of(i) * IPB + (IPB - 1 - k_of(i));
     }
-    static constexpr int copy_shift(int c) {   // shift baked into copy c
-        return IPB == 1 ? 8 * c : 8 * (c / IPB) + BITS * (c % IPB);
-    }
     static constexpr uint32_t sign_mask() {
         uint32_t m = 0;
-        for (int i = 0; i < CPD; ++i) m |= 1u << (shift_of(i) + FIELD - 1);
+        for (int i = 0; i < CPW; ++i) m |= 1u << (shift_of(i) + FIELD - 1);
         return m;
     }
 };
@@ -124,20 +124,20 @@ __device__ __forceinline__ uint32_t copy_shift_rt(uint32_t c) {
 }
 
 template <int DTYPE, int BITS>
-__global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_kernel(TqDevJob job0, const tq_job *jobs) {
+__global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compress_kernel(TqDevJob job0, const tq_job *jobs) {
     using T = InTraits<DTYPE>;
     using P = Pack<BITS>;
     constexpr int ELEM = T::ELEM;
     constexpr int VEC_BYTES = TQ_HEAD_DIM * ELEM;      // 256 or 512
-    constexpr int STAGE = 32 * VEC_BYTES;              // wave-private tile buffer
-    constexpr int NLOAD = STAGE / 1024;                // 16-byte loads per lane per tile
+    constexpr int STAGE = 32 * VEC_BYTES;              // one tile
+    constexpr int NLOAD = STAGE / 1024 / CWAVES;       // 16-byte loads per lane per tile (this wave's quarter)
     constexpr int PIECES = VEC_BYTES / 16;             // 16-byte pieces per vector
     constexpr int VEC_PER_LOAD = 64 / PIECES;          // vectors covered by one load instruction
-    constexpr int NB = P::NB;
+    constexpr int NB = P::NB, NW = P::NW;
 
-    // grid copies first (static, so that their LDS addresses are compile-time immediates)
+    // grid copies first, so that their LDS addresses are small compile-time immediates
     __shared__ __attribute__((aligned(16))) uint8_t lds_grid[TQ_GRID_LDS_BYTES];
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds_dyn[];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_stage[2][STAGE];
 
     const TqDevJob job = tq_load_job(job0, jobs, blockIdx.y, ELEM);
 
@@ -145,18 +145,27 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
     const uint32_t lane = tid & 63u;
     const uint32_t wave = tid >> 6;
     const uint32_t n_tiles = (job.n_vec + 31u) / 32u;
-    if (blockIdx.x * T::WAVES >= n_tiles) return;  // whole block idle (uniform)
+    uint32_t tile = blockIdx.x;
+    if (tile >= n_tiles) return;  // whole block idle (uniform)
+    const uint32_t tile_stride = gridDim.x;
 
     const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
-    uint8_t *lds_a = lds_dyn;
-    uint8_t *stage = lds_dyn + T::TERMS * TQ_OPERAND_BYTES + wave * STAGE;
 
-    tq_copy_to_lds(lds_a, job.table + (DTYPE == TQ_F16 ? hd->off_a_f16 : hd->off_a_bf16),
-                   T::TERMS * TQ_OPERAND_BYTES, tid, T::WAVES * TQ_WAVE);
+    // ---- this wave's quarter of the rotation, resident for the whole kernel
+    tq_u4 areg[T::TERMS][TQ_STEPS];
+    {
+        const uint8_t *src = job.table + (DTYPE == TQ_F16 ? hd->off_a_f16 : hd->off_a_bf16);
+#pragma unroll
+        for (int term = 0; term < T::TERMS; ++term)
+#pragma unroll
+            for (int s = 0; s < TQ_STEPS; ++s)
+                areg[term][s] = tq_gload16(src + (size_t)term * TQ_OPERAND_BYTES +
+                                           (((size_t)wave * TQ_STEPS + s) * 64 + lane) * 16);
+    }
     {   // one grid copy per code position, base pre-shifted
         const uint32_t cells = hd->grid_cells;
         const uint8_t *src = job.table + hd->off_grid;
-        for (uint32_t i = tid; i < cells * P::COPIES; i += T::WAVES * TQ_WAVE) {
+        for (uint32_t i = tid; i < cells * P::COPIES; i += CTHREADS) {
             const uint32_t c = i / cells, q = i - c * cells;
             tq_u2 e = tq_gload8(src + 8u * q);
             e[1] <<= copy_shift_rt<BITS>(c);
@@ -164,20 +173,25 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
         }
     }
     const float grid_scale = hd->grid_scale, grid_bias = hd->grid_bias;
-    __syncthreads();
-
-    const uint32_t tile_stride = gridDim.x * T::WAVES;
-    uint32_t tile = blockIdx.x * T::WAVES + wave;
 
     const uint32_t ld_vec = lane / PIECES, ld_piece = lane % PIECES;  // role in the coalesced loads
     const uint32_t n = lane & 31u, hk = lane >> 5;                    // role in the MFMA: column, half
     const bool one_row = job.tokens >= job.n_vec;
 
+    // LDS offsets that do not change from tile to tile
+    uint32_t st_off[NLOAD];
+#pragma unroll
+    for (int j = 0; j < NLOAD; ++j) {
+        const uint32_t vl = (wave * NLOAD + j) * VEC_PER_LOAD + ld_vec;
+        const uint32_t swz = (ELEM == 2) ? (vl & 15u) : ((vl & 15u) << 1);
+        st_off[j] = vl * VEC_BYTES + ((ld_piece ^ swz) << 4);
+    }
+
     tq_u4 pre[NLOAD];
-    auto issue_loads = [&](uint32_t tl) {
-        const uint32_t v0 = tl * 32u + ld_vec;
-        if (one_row && tl * 32u + 32u <= job.n_vec) {
-            // full tile of a single row: one 64-bit base, constant steps
+    auto issue_loads = [&](auto full_tag, uint32_t tl) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        const uint32_t v0 = tl * 32u + (wave * NLOAD) * VEC_PER_LOAD + ld_vec;
+        if (FULL && one_row) {
             const uint8_t *p = job.states + (long long)v0 * job.token_stride + ld_piece * 16u;
             const long long step = (long long)VEC_PER_LOAD * job.token_stride;
 #pragma unroll
@@ -186,52 +200,34 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
 #pragma unroll
             for (int j = 0; j < NLOAD; ++j) {
                 uint32_t v = v0 + j * VEC_PER_LOAD;
-                v = v < job.n_vec ? v : job.n_vec - 1u;   // tail: re-read the last vector, never stored
+                if (!FULL) v = v < job.n_vec ? v : job.n_vec - 1u;   // tail: re-read the last vector, never stored
                 pre[j] = tq_gload16(job.states + tq_vec_offset(job, v) + ld_piece * 16u);
             }
         }
     };
-    if (tile < n_tiles) issue_loads(tile);
 
-    // LDS addresses that do not change from tile to tile
-    uint32_t st_off[NLOAD];
-#pragma unroll
-    for (int j = 0; j < NLOAD; ++j) {
-        const uint32_t vl = j * VEC_PER_LOAD + ld_vec;
-        const uint32_t swz = (ELEM == 2) ? (vl & 15u) : ((vl & 15u) << 1);
-        st_off[j] = vl * VEC_BYTES + ((ld_piece ^ swz) << 4);
-    }
-    const tq_u4 *a_lane = reinterpret_cast<const tq_u4 *>(lds_a) + lane;
-
-    while (tile < n_tiles) {
-        // ---- park the tile in LDS (swizzled so that the operand reads below are conflict free)
+    // park this wave's quarter of the prefetched tile in LDS (swizzled: the operand reads are conflict free)
+    auto park = [&](uint8_t *stage) {
 #pragma unroll
         for (int j = 0; j < NLOAD; ++j) *reinterpret_cast<tq_u4 *>(stage + st_off[j]) = pre[j];
-        const uint32_t next = tile + tile_stride;
-        if (next < n_tiles) issue_loads(next);
+    };
 
-        // ---- rotation: acc[t][r] = sum_k Pi[64h + 16t + r][k] * x_n[k]  (raw, unnormalised)
-        tq_f16v acc[TQ_TILES];
-#pragma unroll
-        for (int t = 0; t < TQ_TILES; ++t) acc[t] = tq_zero16();
+    // One tile, already parked in `stage` and published by a barrier: rotate, search, store.
+    auto process = [&](auto full_tag, uint32_t tile, const uint8_t *stage) {
+        constexpr bool FULL = decltype(full_tag)::value;
+
+        // ---- rotation: acc[r] = sum_k Pi[32w + 16h + r][k] * x_n[k]  (raw, unnormalised)
+        tq_f16v acc = tq_zero16();
         float ss0 = 0.f, ss1 = 0.f;
-
 #pragma unroll
         for (int s = 0; s < TQ_STEPS; ++s) {
-            const tq_u4 *a_base = a_lane + (size_t)s * 64;
-            constexpr int TILE_STRIDE = TQ_STEPS * 64;          // tq_u4 units between tiles
-            constexpr int TERM_STRIDE = TQ_OPERAND_BYTES / 16;  // tq_u4 units between terms
             if constexpr (ELEM == 2) {
                 const uint32_t piece = 2u * s + hk;
                 const tq_u4 b = *reinterpret_cast<const tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4));
                 if (s & 1) ss1 = sumsq8<DTYPE>(b, ss1); else ss0 = sumsq8<DTYPE>(b, ss0);
 #pragma unroll
                 for (int term = 0; term < T::TERMS; ++term)
-#pragma unroll
-                    for (int t = 0; t < TQ_TILES; ++t) {
-                        const tq_u4 a = a_base[term * TERM_STRIDE + t * TILE_STRIDE];
-                        acc[t] = (DTYPE == TQ_F16) ? mfma_f16(a, b, acc[t]) : mfma_bf16(a, b, acc[t]);
-                    }
+                    acc = (DTYPE == TQ_F16) ? mfma_f16(areg[term][s], b, acc) : mfma_bf16(areg[term][s], b, acc);
             } else {
                 const uint32_t piece = 2u * (2u * s + hk);
                 const uint32_t swz = (n & 15u) << 1;
@@ -249,12 +245,7 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
 #pragma unroll
                 for (int i = 0; i < 3; ++i)
 #pragma unroll
-                    for (int term = 0; term + i < 3; ++term)
-#pragma unroll
-                        for (int t = 0; t < TQ_TILES; ++t) {
-                            const tq_u4 a = a_base[term * TERM_STRIDE + t * TILE_STRIDE];
-                            acc[t] = mfma_bf16(a, xt[i], acc[t]);
-                        }
+                    for (int term = 0; term + i < 3; ++term) acc = mfma_bf16(areg[term][s], xt[i], acc);
             }
         }
 
@@ -267,26 +258,24 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
         if (DTYPE == TQ_F16) inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
         const float inv_cell = inv * grid_scale;   // grid_scale is a power of two: exact
 
-        // ---- code search + packing.  Lane (n, hk) holds coordinates 64*hk + 16*t + r.
-        // Per coordinate: cell address (fma, and), one 8-byte LDS lookup from the copy whose base
+        // ---- code search + packing.  Lane (n, hk) of wave w holds coordinates 32w + 16hk + r.
+        // Per coordinate: cell address (fma, and), one 8-byte LDS lookup from the grid copy whose base
         // is pre-shifted to the code's bit position, exact comparison by fma, sign bit funnelled
         // into `lt`, bases OR-ed together.  code = base + !(rho < threshold).
-        uint32_t words[NB / 4];
+        uint32_t words[NW];
 #pragma unroll
-        for (int w = 0; w < NB / 4; ++w) {
+        for (int w = 0; w < NW; ++w) {
             uint32_t lt = 0u, lo = 0u, hi = 0u;
-            int cursor = 32;
 #pragma unroll
-            for (int i = 0; i < P::CPD; ++i) {
-                const int c = P::local_code(w, i);
-                const float a = acc[c / 16][c % 16];
+            for (int i = 0; i < P::CPW; ++i) {
+                const float a = acc[P::local_code(w, i)];
                 const uint32_t addr = __float_as_uint(fmaf(a, inv_cell, grid_bias)) & TQ_GRID_ADDR_MASK;
                 const tq_u2 cell = *reinterpret_cast<const tq_u2 *>(lds_grid + P::copy_of(i) * P::COPY_STRIDE + addr);
                 const float t = fmaf(a, inv, -__uint_as_float(cell[0]));
+                const int cursor = i == 0 ? 8 * P::WB : P::shift_of(i - 1);
                 const int gap = cursor - (P::shift_of(i) + P::FIELD);
                 if (gap > 0) lt = __builtin_amdgcn_alignbit(lt, 0u, 32 - gap);
                 lt = __builtin_amdgcn_alignbit(lt, __float_as_uint(t), 32 - P::FIELD);
-                cursor = P::shift_of(i);
                 if (P::IPB == 1 && P::byte_of(i) >= 2) hi |= cell[1]; else lo |= cell[1];
             }
             const uint32_t bases = P::IPB == 1 ? (lo | (hi << 16)) : lo;
@@ -295,24 +284,52 @@ __global__ __launch_bounds__(InTraits<DTYPE>::WAVES *TQ_WAVE) void tq_compress_k
         }
 
         const uint32_t v = tile * 32u + n;
-        if (v < job.n_vec) {
-            uint8_t *dst = job.idx_bytes + (size_t)v * (2 * NB) + hk * NB;
-            if constexpr (NB == 8) {
+        if (FULL || v < job.n_vec) {
+            uint8_t *dst = job.idx_bytes + (size_t)v * (8 * NB) + (2u * wave + hk) * NB;
+            if constexpr (NB == 2) {
+                tq_gstore2(reinterpret_cast<uint16_t *>(dst), (uint16_t)words[0]);
+            } else if constexpr (NB == 4) {
+                *reinterpret_cast<TQ_GLOBAL uint32_t *>((TQ_GLOBAL uint8_t *)dst) = words[0];
+            } else if constexpr (NB == 8) {
                 tq_u2 o = {words[0], words[1]};
                 tq_gstore8(dst, o);
             } else {
-#pragma unroll
-                for (int q = 0; q < NB / 16; ++q) {
-                    tq_u4 o = {words[4 * q], words[4 * q + 1], words[4 * q + 2], words[4 * q + 3]};
-                    tq_gstore16(dst + 16 * q, o);
-                }
+                tq_u4 o = {words[0], words[1], words[2], words[3]};
+                tq_gstore16(dst, o);
             }
-            if (hk == 0) {
-                const _Float16 hn = (_Float16)nrm;
-                tq_gstore2(job.vec_norms + v, __builtin_bit_cast(uint16_t, hn));
-            }
+            // every lane of every wave holds the same norm for vector n: all store it (identical
+            // values to one address) rather than predicating the store on a fraction of the lanes
+            const _Float16 hn = (_Float16)nrm;
+            tq_gstore2(job.vec_norms + v, __builtin_bit_cast(uint16_t, hn));
         }
-        tile = next;
+    };
+
+    // Pipeline over the tiles whose 32 vectors all exist.  Iteration k: start the loads of tile k+1,
+    // barrier (publishes buffer k, and everyone has finished reading buffer k-1), compute and store
+    // tile k, then park tile k+1 into the other buffer.  Loads, stores and the wait for the loads sit
+    // in one straight line, in that order, so the wait is s_waitcnt vmcnt(#stores): the stores of
+    // tile k stay in flight across the iteration boundary.
+    const uint32_t n_full = job.n_vec / 32u;
+    uint32_t buf = 0;
+    if (tile < n_full) {
+        issue_loads(std::true_type{}, tile);
+        park(lds_stage[0]);
+        while (tile < n_full) {
+            const uint32_t next = tile + tile_stride;
+            issue_loads(std::true_type{}, next < n_full ? next : tile);   // last iteration: harmless re-read
+            __syncthreads();
+            process(std::true_type{}, tile, lds_stage[buf]);
+            buf ^= 1u;
+            park(lds_stage[buf]);
+            tile = next;
+        }
+    }
+    // the partial last tile of the job, if this block is the one whose turn it is
+    if (tile == n_full && n_full < n_tiles) {
+        issue_loads(std::false_type{}, tile);
+        park(lds_stage[buf]);
+        __syncthreads();
+        process(std::false_type{}, tile, lds_stage[buf]);
     }
 }
 
@@ -343,24 +360,13 @@ int query_device(DeviceInfo &info) {
 
 template <int DTYPE, int BITS>
 int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t stream) {
-    using T = InTraits<DTYPE>;
     DeviceInfo info;
     int rc = query_device(info);
     if (rc) return rc;
-    constexpr size_t lds = compress_lds_bytes<DTYPE>();
-    static bool configured[64] = {};
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if (!configured[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&tq_compress_kernel<DTYPE, BITS>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        configured[dev] = true;
-    }
-    const uint32_t want = (max_tiles + T::WAVES - 1) / T::WAVES;
-    const uint32_t bx = tq_blocks_per_job(want, info.cus, n_jobs);
-    dim3 grid(bx, (unsigned)n_jobs, 1), block(T::WAVES * TQ_WAVE, 1, 1);
-    hipLaunchKernelGGL((tq_compress_kernel<DTYPE, BITS>), grid, block, lds, stream, job, jobs_dev);
+    // Three four-wave blocks fit on a compute unit (registers: three waves per SIMD).
+    const uint32_t bx = tq_blocks_per_job(max_tiles, info.cus * 3, n_jobs);
+    dim3 grid(bx, (unsigned)n_jobs, 1), block(CTHREADS, 1, 1);
+    hipLaunchKernelGGL((tq_compress_kernel<DTYPE, BITS>), grid, block, 0, stream, job, jobs_dev);
     return (int)hipGetLastError();
 }
 

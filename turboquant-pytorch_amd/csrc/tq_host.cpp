@@ -234,14 +234,15 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
         for (int s = 0; s < TQ_STEPS; ++s)
             for (int l = 0; l < 64; ++l) {
                 const int m = l % 32, hk = l / 32;
-                // MFMA row m = 8a + 4h + b  <->  accumulator (h, r = 4a + b)  <->  output 64h + 16t + r
+                // MFMA row m = 8a + 4h + b  <->  accumulator register r = 4a + b of lane-half h
                 const int a = m / 8, h = (m / 4) % 2, b = m % 4;
-                const int out = 64 * h + 16 * t + 4 * a + b;
+                const int out_c = 32 * t + 16 * h + 4 * a + b;                        // compress (see tq_table.h)
+                const int out_d = 64 * h + 16 * t + 4 * a + b;                        // decompress
                 for (int i = 0; i < 8; ++i) {
                     const size_t o = operand_index(t, s, l, i);
                     {   // compress: rotated[out] = sum_k x[k] * Pi[out][k],  k = 16s + 8hk + i
                         const int k = 16 * s + 8 * hk + i;
-                        const float p = Pi[out * D + k];
+                        const float p = Pi[out_c * D + k];
                         const double ps = (double)p * pi_scale;
                         const uint16_t hi = to_f16((float)ps);
                         const uint16_t lo = to_f16((float)(ps - (double)from_f16(hi)));
@@ -257,7 +258,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
                     }
                     {   // decompress: x[out] = sum_j y[j] * Pi[j][out],  j = 64hk + 8s + i
                         const int j = 64 * hk + 8 * s + i;
-                        const float p = Pi[j * D + out];
+                        const float p = Pi[j * D + out_d];
                         const uint16_t hi = to_f16(p);
                         at_f16[o] = hi;
                         at_f16[term + o] = to_f16((float)((double)p - (double)from_f16(hi)));

@@ -6,7 +6,7 @@
 #include <stdint.h>
 
 #define TQ_TABLE_MAGIC 0x54514d49u /* "TQMI" */
-#define TQ_TABLE_VERSION 4u
+#define TQ_TABLE_VERSION 6u
 #define TQ_HEAD_DIM 128
 
 // --- MFMA operand tiling (v_mfma_f32_32x32x16_{f16,bf16}) --------------------------------
@@ -15,11 +15,16 @@
 // (n = l % 32, h = l / 32) holds row  m = 8*(r/4) + 4*h + (r%4)  of column n.
 //
 // Both kernels put the vectors on the MFMA columns (one vector per lane, two lanes per
-// vector) and choose the row order so that lane-half h ends up with 64 consecutive outputs:
-//     output(t, h, r) = 64*h + 16*t + r
-// and the contraction order so that lane-half hk consumes 64 consecutive inputs in 8 steps:
-//     input(s, hk, i) = 16*s + 8*hk + i      (compress:   element of x)
-//     input(s, hk, i) = 64*hk + 8*s + i      (decompress: code index)
+// vector) and keep the rotation resident in registers as the A operand.
+//
+// compress: a tile of 32 vectors is shared by the four waves of a block; wave w owns MFMA tile w
+// and the row order is chosen so that lane-half h of wave w ends up with 16 consecutive rotated
+// coordinates:
+//     output(tile = w, h, r) = 32*w + 16*h + r
+//     input(s, hk, i)        = 16*s + 8*hk + i               (element of x)
+// decompress: one wave owns all four MFMA tiles, lane-half h gets 64 consecutive elements:
+//     output(tile t, h, r)        = 64*h + 16*t + r
+//     input(s, hk, i)             = 64*hk + 8*s + i          (code index)
 #define TQ_TILES 4  /* 128 outputs / 32 rows  */
 #define TQ_STEPS 8  /* 128 inputs  / 16 deep  */
 #define TQ_OPERAND_BYTES (TQ_TILES * TQ_STEPS * 64 * 16) /* one 128x128 16-bit operand set: 32 KiB */
