@@ -138,6 +138,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     // grid copies first, so that their LDS addresses are small compile-time immediates
     __shared__ __attribute__((aligned(16))) uint8_t lds_grid[TQ_GRID_LDS_BYTES];
     __shared__ __attribute__((aligned(16))) uint8_t lds_stage[2][STAGE];
+    __shared__ float lds_ss[2][32];   // sum of squares of the tile's vectors (16-bit inputs)
 
     const TqDevJob job = tq_load_job(job0, jobs, blockIdx.y, ELEM);
 
@@ -188,34 +189,47 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     }
 
     tq_u4 pre[NLOAD];
+    // loads of this wave's quarter of tile `tl`, generic addressing (any strides, tail clamped)
     auto issue_loads = [&](auto full_tag, uint32_t tl) {
         constexpr bool FULL = decltype(full_tag)::value;
         const uint32_t v0 = tl * 32u + (wave * NLOAD) * VEC_PER_LOAD + ld_vec;
-        if (FULL && one_row) {
-            const uint8_t *p = job.states + (long long)v0 * job.token_stride + ld_piece * 16u;
-            const long long step = (long long)VEC_PER_LOAD * job.token_stride;
 #pragma unroll
-            for (int j = 0; j < NLOAD; ++j) pre[j] = tq_gload16(p + j * step);
-        } else {
+        for (int j = 0; j < NLOAD; ++j) {
+            uint32_t v = v0 + j * VEC_PER_LOAD;
+            if (!FULL) v = v < job.n_vec ? v : job.n_vec - 1u;   // tail: re-read the last vector, never stored
+            pre[j] = tq_gload16(job.states + tq_vec_offset(job, v) + ld_piece * 16u);
+        }
+    };
+    // the same for a single-row job, from a running per-lane pointer
+    auto issue_loads_ptr = [&](const uint8_t *p, long long jstep) {
+#pragma unroll
+        for (int j = 0; j < NLOAD; ++j) pre[j] = tq_gload16(p + j * jstep);
+    };
+
+    // Park this wave's quarter of the prefetched tile in LDS (swizzled: the operand reads are conflict
+    // free).  For 16-bit inputs the squares are summed here, where every element is touched once:
+    // 16 lanes hold one vector, an inclusive row scan leaves the total in the last of them.
+    auto park = [&](uint32_t b) {
+        uint8_t *stage = lds_stage[b];
+#pragma unroll
+        for (int j = 0; j < NLOAD; ++j) *reinterpret_cast<tq_u4 *>(stage + st_off[j]) = pre[j];
+        if constexpr (ELEM == 2) {
 #pragma unroll
             for (int j = 0; j < NLOAD; ++j) {
-                uint32_t v = v0 + j * VEC_PER_LOAD;
-                if (!FULL) v = v < job.n_vec ? v : job.n_vec - 1u;   // tail: re-read the last vector, never stored
-                pre[j] = tq_gload16(job.states + tq_vec_offset(job, v) + ld_piece * 16u);
+                float x = sumsq8<DTYPE>(pre[j], 0.f);
+                x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x111, 0xf, 0xf, true));
+                x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x112, 0xf, 0xf, true));
+                x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x114, 0xf, 0xf, true));
+                x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x118, 0xf, 0xf, true));
+                if ((lane & 15u) == 15u) lds_ss[b][(wave * NLOAD + j) * VEC_PER_LOAD + ld_vec] = x;
             }
         }
     };
 
-    // park this wave's quarter of the prefetched tile in LDS (swizzled: the operand reads are conflict free)
-    auto park = [&](uint8_t *stage) {
-#pragma unroll
-        for (int j = 0; j < NLOAD; ++j) *reinterpret_cast<tq_u4 *>(stage + st_off[j]) = pre[j];
-    };
-
-    // One tile, already parked in `stage` and published by a barrier: rotate, search, store.
-    auto process = [&](auto full_tag, uint32_t tile, const uint8_t *stage) {
-        constexpr bool FULL = decltype(full_tag)::value;
-
+    // One tile, parked in buffer `b` and published by a barrier: rotate and search.
+    // Leaves the lane's packed words in `words` and the vector's norm in `nrm`.
+    auto compute = [&](uint32_t b, uint32_t (&words)[NW], float &nrm) {
+        const uint8_t *stage = lds_stage[b];
         // ---- rotation: acc[r] = sum_k Pi[32w + 16h + r][k] * x_n[k]  (raw, unnormalised)
         tq_f16v acc = tq_zero16();
         float ss0 = 0.f, ss1 = 0.f;
@@ -223,11 +237,10 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
         for (int s = 0; s < TQ_STEPS; ++s) {
             if constexpr (ELEM == 2) {
                 const uint32_t piece = 2u * s + hk;
-                const tq_u4 b = *reinterpret_cast<const tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4));
-                if (s & 1) ss1 = sumsq8<DTYPE>(b, ss1); else ss0 = sumsq8<DTYPE>(b, ss0);
+                const tq_u4 bop = *reinterpret_cast<const tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4));
 #pragma unroll
                 for (int term = 0; term < T::TERMS; ++term)
-                    acc = (DTYPE == TQ_F16) ? mfma_f16(areg[term][s], b, acc) : mfma_bf16(areg[term][s], b, acc);
+                    acc = (DTYPE == TQ_F16) ? mfma_f16(areg[term][s], bop, acc) : mfma_bf16(areg[term][s], bop, acc);
             } else {
                 const uint32_t piece = 2u * (2u * s + hk);
                 const uint32_t swz = (n & 15u) << 1;
@@ -249,10 +262,23 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             }
         }
 
-        // ---- norm: both lanes of a vector hold half of the squares
-        float ss = ss0 + ss1;
-        ss += __shfl_xor(ss, 32);
-        const float nrm = sqrtf(ss);
+        // ---- norm
+        float ss;
+        if constexpr (ELEM == 2) {
+            ss = lds_ss[b][n];
+        } else {
+            ss = ss0 + ss1;                 // both lanes of a vector hold half of the squares
+            ss += __shfl_xor(ss, 32);
+        }
+        // sqrt: reciprocal square root plus one Newton step is correctly rounded except for a
+        // vanishing fraction of inputs; zero, denormal and non-finite sums take the library routine.
+        if (__builtin_expect(__any(!(ss > 1e-30f && ss < 1e30f)), 0)) {
+            nrm = sqrtf(ss);
+        } else {
+            const float r = __builtin_amdgcn_rsqf(ss);
+            const float g = ss * r, h = 0.5f * r;
+            nrm = fmaf(fmaf(-g, g, ss), h, g);
+        }
         // 1 / (norm + 1e-8): the reciprocal only scales the coordinates, one ulp is irrelevant
         float inv = __builtin_amdgcn_rcpf(nrm + 1e-8f);
         if (DTYPE == TQ_F16) inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
@@ -262,7 +288,6 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
         // Per coordinate: cell address (fma, and), one 8-byte LDS lookup from the grid copy whose base
         // is pre-shifted to the code's bit position, exact comparison by fma, sign bit funnelled
         // into `lt`, bases OR-ed together.  code = base + !(rho < threshold).
-        uint32_t words[NW];
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
             uint32_t lt = 0u, lo = 0u, hi = 0u;
@@ -282,54 +307,85 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             const uint32_t ge = (~lt & P::sign_mask()) >> (P::FIELD - 1);
             words[w] = bases + ge;
         }
-
-        const uint32_t v = tile * 32u + n;
-        if (FULL || v < job.n_vec) {
-            uint8_t *dst = job.idx_bytes + (size_t)v * (8 * NB) + (2u * wave + hk) * NB;
-            if constexpr (NB == 2) {
-                tq_gstore2(reinterpret_cast<uint16_t *>(dst), (uint16_t)words[0]);
-            } else if constexpr (NB == 4) {
-                *reinterpret_cast<TQ_GLOBAL uint32_t *>((TQ_GLOBAL uint8_t *)dst) = words[0];
-            } else if constexpr (NB == 8) {
-                tq_u2 o = {words[0], words[1]};
-                tq_gstore8(dst, o);
-            } else {
-                tq_u4 o = {words[0], words[1], words[2], words[3]};
-                tq_gstore16(dst, o);
-            }
-            // every lane of every wave holds the same norm for vector n: all store it (identical
-            // values to one address) rather than predicating the store on a fraction of the lanes
-            const _Float16 hn = (_Float16)nrm;
-            tq_gstore2(job.vec_norms + v, __builtin_bit_cast(uint16_t, hn));
-        }
     };
+
+    // the lane's NB packed bytes and (identical in all lanes of a vector) the fp16 norm
+    auto store = [&](uint8_t *dst, uint16_t *ndst, const uint32_t (&words)[NW], float nrm) {
+        if constexpr (NB == 2) {
+            tq_gstore2(reinterpret_cast<uint16_t *>(dst), (uint16_t)words[0]);
+        } else if constexpr (NB == 4) {
+            *reinterpret_cast<TQ_GLOBAL uint32_t *>((TQ_GLOBAL uint8_t *)dst) = words[0];
+        } else if constexpr (NB == 8) {
+            tq_u2 o = {words[0], words[1]};
+            tq_gstore8(dst, o);
+        } else {
+            tq_u4 o = {words[0], words[1], words[2], words[3]};
+            tq_gstore16(dst, o);
+        }
+        // every lane of every wave holds the same norm for vector n: all store it (identical values
+        // to one address) rather than predicating the store on a fraction of the lanes
+        const _Float16 hn = (_Float16)nrm;
+        tq_gstore2(ndst, __builtin_bit_cast(uint16_t, hn));
+    };
+    const uint32_t lane_slot = (2u * wave + hk) * NB;   // this lane's bytes inside a vector's G = 8 * NB
 
     // Pipeline over the tiles whose 32 vectors all exist.  Iteration k: start the loads of tile k+1,
     // barrier (publishes buffer k, and everyone has finished reading buffer k-1), compute and store
     // tile k, then park tile k+1 into the other buffer.  Loads, stores and the wait for the loads sit
-    // in one straight line, in that order, so the wait is s_waitcnt vmcnt(#stores): the stores of
-    // tile k stay in flight across the iteration boundary.
+    // in one straight line, in that order, and none of them is predicated, so the wait is
+    // s_waitcnt vmcnt(#stores): the stores of tile k stay in flight across the iteration boundary.
     const uint32_t n_full = job.n_vec / 32u;
     uint32_t buf = 0;
+    uint32_t words[NW];
+    float nrm;
     if (tile < n_full) {
-        issue_loads(std::true_type{}, tile);
-        park(lds_stage[0]);
-        while (tile < n_full) {
-            const uint32_t next = tile + tile_stride;
-            issue_loads(std::true_type{}, next < n_full ? next : tile);   // last iteration: harmless re-read
-            __syncthreads();
-            process(std::true_type{}, tile, lds_stage[buf]);
-            buf ^= 1u;
-            park(lds_stage[buf]);
-            tile = next;
+        if (one_row) {
+            // running per-lane pointers: a handful of 64-bit adds per tile instead of index arithmetic
+            const long long jstep = (long long)VEC_PER_LOAD * job.token_stride;
+            const long long in_step = (long long)tile_stride * 32 * job.token_stride;
+            const uint8_t *ld = job.states + (long long)(tile * 32u + (wave * NLOAD) * VEC_PER_LOAD + ld_vec) * job.token_stride + ld_piece * 16u;
+            uint8_t *cd = job.idx_bytes + (size_t)(tile * 32u + n) * (8 * NB) + lane_slot;
+            uint16_t *nd = job.vec_norms + (size_t)tile * 32u + n;
+            const size_t cd_step = (size_t)tile_stride * 32u * (8 * NB), nd_step = (size_t)tile_stride * 32u;
+            issue_loads_ptr(ld, jstep);
+            park(0);
+            while (tile < n_full) {
+                const uint32_t next = tile + tile_stride;
+                ld += next < n_full ? in_step : 0;                       // last iteration: harmless re-read
+                issue_loads_ptr(ld, jstep);
+                __syncthreads();
+                compute(buf, words, nrm);
+                store(cd, nd, words, nrm);
+                cd += cd_step;
+                nd += nd_step;
+                buf ^= 1u;
+                park(buf);
+                tile = next;
+            }
+        } else {
+            issue_loads(std::true_type{}, tile);
+            park(0);
+            while (tile < n_full) {
+                const uint32_t next = tile + tile_stride;
+                issue_loads(std::true_type{}, next < n_full ? next : tile);
+                __syncthreads();
+                compute(buf, words, nrm);
+                const uint32_t v = tile * 32u + n;
+                store(job.idx_bytes + (size_t)v * (8 * NB) + lane_slot, job.vec_norms + v, words, nrm);
+                buf ^= 1u;
+                park(buf);
+                tile = next;
+            }
         }
     }
     // the partial last tile of the job, if this block is the one whose turn it is
     if (tile == n_full && n_full < n_tiles) {
         issue_loads(std::false_type{}, tile);
-        park(lds_stage[buf]);
+        park(buf);
         __syncthreads();
-        process(std::false_type{}, tile, lds_stage[buf]);
+        compute(buf, words, nrm);
+        const uint32_t v = tile * 32u + n;
+        if (v < job.n_vec) store(job.idx_bytes + (size_t)v * (8 * NB) + lane_slot, job.vec_norms + v, words, nrm);
     }
 }
 
