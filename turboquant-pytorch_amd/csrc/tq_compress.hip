@@ -28,9 +28,12 @@
 
 namespace {
 
+#ifndef TQ_C16_WAVES
+#define TQ_C16_WAVES 2
+#endif
 template <int DTYPE> struct InTraits;
-template <> struct InTraits<TQ_F16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = 3; };
-template <> struct InTraits<TQ_BF16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = 3; };
+template <> struct InTraits<TQ_F16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = TQ_C16_WAVES; };
+template <> struct InTraits<TQ_BF16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = TQ_C16_WAVES; };
 // fp32 input keeps three rotation terms resident and stages 16 KiB tiles
 template <> struct InTraits<TQ_F32> { static constexpr int ELEM = 4, TERMS = 3, MIN_WAVES = 2; };
 
@@ -200,23 +203,18 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             pre[j] = tq_gload16(job.states + tq_vec_offset(job, v) + ld_piece * 16u);
         }
     };
-    // the same for a single-row job, from a running per-lane pointer
-    auto issue_loads_ptr = [&](const uint8_t *p, long long jstep) {
-#pragma unroll
-        for (int j = 0; j < NLOAD; ++j) pre[j] = tq_gload16(p + j * jstep);
-    };
 
     // Park this wave's quarter of the prefetched tile in LDS (swizzled: the operand reads are conflict
     // free).  For 16-bit inputs the squares are summed here, where every element is touched once:
     // 16 lanes hold one vector, an inclusive row scan leaves the total in the last of them.
-    auto park = [&](uint32_t b) {
+    auto park = [&](uint32_t b, const tq_u4 (&src)[NLOAD]) {
         uint8_t *stage = lds_stage[b];
 #pragma unroll
-        for (int j = 0; j < NLOAD; ++j) *reinterpret_cast<tq_u4 *>(stage + st_off[j]) = pre[j];
+        for (int j = 0; j < NLOAD; ++j) *reinterpret_cast<tq_u4 *>(stage + st_off[j]) = src[j];
         if constexpr (ELEM == 2) {
 #pragma unroll
             for (int j = 0; j < NLOAD; ++j) {
-                float x = sumsq8<DTYPE>(pre[j], 0.f);
+                float x = sumsq8<DTYPE>(src[j], 0.f);
                 x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x111, 0xf, 0xf, true));
                 x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x112, 0xf, 0xf, true));
                 x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x114, 0xf, 0xf, true));
@@ -226,43 +224,40 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
         }
     };
 
-    // One tile, parked in buffer `b` and published by a barrier: rotate and search.
-    // Leaves the lane's packed words in `words` and the vector's norm in `nrm`.
-    auto compute = [&](uint32_t b, uint32_t (&words)[NW], float &nrm) {
-        const uint8_t *stage = lds_stage[b];
-        // ---- rotation: acc[r] = sum_k Pi[32w + 16h + r][k] * x_n[k]  (raw, unnormalised)
-        tq_f16v acc = tq_zero16();
-        float ss0 = 0.f, ss1 = 0.f;
+    // ---- the three stages of a tile ---------------------------------------------------------
+    // (1) rotation step s of the tile parked in `stage`: acc[r] += sum over 16 inputs of
+    //     Pi[32w + 16h + r][k] * x_n[k]  (raw, unnormalised); fp32 inputs also sum their squares here
+    auto rotate_step = [&](const uint8_t *stage, int s, tq_f16v &acc, float &ss0, float &ss1) {
+        if constexpr (ELEM == 2) {
+            const uint32_t piece = 2u * s + hk;
+            const tq_u4 bop = *reinterpret_cast<const tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4));
 #pragma unroll
-        for (int s = 0; s < TQ_STEPS; ++s) {
-            if constexpr (ELEM == 2) {
-                const uint32_t piece = 2u * s + hk;
-                const tq_u4 bop = *reinterpret_cast<const tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4));
+            for (int term = 0; term < T::TERMS; ++term)
+                acc = (DTYPE == TQ_F16) ? mfma_f16(areg[term][s], bop, acc) : mfma_bf16(areg[term][s], bop, acc);
+        } else {
+            const uint32_t piece = 2u * (2u * s + hk);
+            const uint32_t swz = (n & 15u) << 1;
+            const uint8_t *row = stage + n * VEC_BYTES;
+            const tq_u4 q0 = *reinterpret_cast<const tq_u4 *>(row + ((piece ^ swz) << 4));
+            const tq_u4 q1 = *reinterpret_cast<const tq_u4 *>(row + (((piece + 1u) ^ swz) << 4));
+            float x[8];
 #pragma unroll
-                for (int term = 0; term < T::TERMS; ++term)
-                    acc = (DTYPE == TQ_F16) ? mfma_f16(areg[term][s], bop, acc) : mfma_bf16(areg[term][s], bop, acc);
-            } else {
-                const uint32_t piece = 2u * (2u * s + hk);
-                const uint32_t swz = (n & 15u) << 1;
-                const uint8_t *row = stage + n * VEC_BYTES;
-                const tq_u4 q0 = *reinterpret_cast<const tq_u4 *>(row + ((piece ^ swz) << 4));
-                const tq_u4 q1 = *reinterpret_cast<const tq_u4 *>(row + (((piece + 1u) ^ swz) << 4));
-                float x[8];
+            for (int i = 0; i < 4; ++i) { x[i] = __uint_as_float(q0[i]); x[4 + i] = __uint_as_float(q1[i]); }
 #pragma unroll
-                for (int i = 0; i < 4; ++i) { x[i] = __uint_as_float(q0[i]); x[4 + i] = __uint_as_float(q1[i]); }
+            for (int i = 0; i < 8; ++i) { if (i & 1) ss1 = fmaf(x[i], x[i], ss1); else ss0 = fmaf(x[i], x[i], ss0); }
+            tq_u4 xt[3];
+            split_f32x8(x, xt[0], xt[1], xt[2]);
+            // all products whose weight is >= 2^-24 of the leading one: (x term i, Pi term j), i + j <= 2
 #pragma unroll
-                for (int i = 0; i < 8; ++i) { if (i & 1) ss1 = fmaf(x[i], x[i], ss1); else ss0 = fmaf(x[i], x[i], ss0); }
-                tq_u4 xt[3];
-                split_f32x8(x, xt[0], xt[1], xt[2]);
-                // all products whose weight is >= 2^-24 of the leading one: (x term i, Pi term j), i + j <= 2
+            for (int i = 0; i < 3; ++i)
 #pragma unroll
-                for (int i = 0; i < 3; ++i)
-#pragma unroll
-                    for (int term = 0; term + i < 3; ++term) acc = mfma_bf16(areg[term][s], xt[i], acc);
-            }
+                for (int term = 0; term + i < 3; ++term) acc = mfma_bf16(areg[term][s], xt[i], acc);
         }
+    };
 
-        // ---- norm
+    // (2) norm of the lane's vector and the two scale factors of the code search
+    struct Scale { float nrm, inv, inv_cell; };
+    auto scale_of = [&](uint32_t b, float ss0, float ss1) {
         float ss;
         if constexpr (ELEM == 2) {
             ss = lds_ss[b][n];
@@ -270,43 +265,76 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             ss = ss0 + ss1;                 // both lanes of a vector hold half of the squares
             ss += __shfl_xor(ss, 32);
         }
+        Scale sc;
         // sqrt: reciprocal square root plus one Newton step is correctly rounded except for a
-        // vanishing fraction of inputs; zero, denormal and non-finite sums take the library routine.
-        if (__builtin_expect(__any(!(ss > 1e-30f && ss < 1e30f)), 0)) {
-            nrm = sqrtf(ss);
-        } else {
+        // vanishing fraction of inputs.  Sums below 1e-35 (norm < 1e-17: it vanishes both in
+        // norm + 1e-8 and in fp16) count as zero; infinite and NaN sums pass through.
+        {
             const float r = __builtin_amdgcn_rsqf(ss);
             const float g = ss * r, h = 0.5f * r;
-            nrm = fmaf(fmaf(-g, g, ss), h, g);
+            sc.nrm = fmaf(fmaf(-g, g, ss), h, g);
+            sc.nrm = ss < 1e-35f ? 0.f : sc.nrm;
+            sc.nrm = ss < __builtin_inff() ? sc.nrm : ss;
         }
         // 1 / (norm + 1e-8): the reciprocal only scales the coordinates, one ulp is irrelevant
-        float inv = __builtin_amdgcn_rcpf(nrm + 1e-8f);
-        if (DTYPE == TQ_F16) inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
-        const float inv_cell = inv * grid_scale;   // grid_scale is a power of two: exact
+        sc.inv = __builtin_amdgcn_rcpf(sc.nrm + 1e-8f);
+        if (DTYPE == TQ_F16) sc.inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
+        sc.inv_cell = sc.inv * grid_scale;   // grid_scale is a power of two: exact
+        return sc;
+    };
 
-        // ---- code search + packing.  Lane (n, hk) of wave w holds coordinates 32w + 16hk + r.
-        // Per coordinate: cell address (fma, and), one 8-byte LDS lookup from the grid copy whose base
-        // is pre-shifted to the code's bit position, exact comparison by fma, sign bit funnelled
-        // into `lt`, bases OR-ed together.  code = base + !(rho < threshold).
+    // (3) code search + packing.  Lane (n, hk) of wave w holds coordinates 32w + 16hk + r.
+    // Per coordinate: cell address (fma, and), one 8-byte LDS lookup from the grid copy whose base
+    // is pre-shifted to the code's bit position, exact comparison by fma, sign bit funnelled
+    // into `lt`, bases OR-ed together.  code = base + !(rho < threshold).
+    // The 16 coordinates of a lane are visited in the order q = 0..15 = (word, position in word).
+    struct Search { uint32_t lt[NW], lo[NW], hi[NW]; };
+    auto search_begin = [&](Search &z) {
+#pragma unroll
+        for (int w = 0; w < NW; ++w) z.lt[w] = z.lo[w] = z.hi[w] = 0u;
+    };
+    auto search_lookup = [&](int q, const tq_f16v &acc, const Scale &sc) {
+        const int w = q / P::CPW, i = q % P::CPW;
+        const float a = acc[P::local_code(w, i)];
+        const uint32_t addr = __float_as_uint(fmaf(a, sc.inv_cell, grid_bias)) & TQ_GRID_ADDR_MASK;
+        return *reinterpret_cast<const tq_u2 *>(lds_grid + P::copy_of(i) * P::COPY_STRIDE + addr);
+    };
+    auto search_apply = [&](Search &z, int q, const tq_f16v &acc, const Scale &sc, tq_u2 cell) {
+        const int w = q / P::CPW, i = q % P::CPW;
+        const float a = acc[P::local_code(w, i)];
+        const float t = fmaf(a, sc.inv, -__uint_as_float(cell[0]));
+        const int cursor = i == 0 ? 8 * P::WB : P::shift_of(i - 1);
+        const int gap = cursor - (P::shift_of(i) + P::FIELD);
+        if (gap > 0) z.lt[w] = __builtin_amdgcn_alignbit(z.lt[w], 0u, 32 - gap);
+        z.lt[w] = __builtin_amdgcn_alignbit(z.lt[w], __float_as_uint(t), 32 - P::FIELD);
+        if (P::IPB == 1 && P::byte_of(i) >= 2) z.hi[w] |= cell[1]; else z.lo[w] |= cell[1];
+    };
+    auto search_coord = [&](Search &z, int q, const tq_f16v &acc, const Scale &sc) {
+        search_apply(z, q, acc, sc, search_lookup(q, acc, sc));
+    };
+    auto search_end = [&](const Search &z, uint32_t (&words)[NW]) {
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
-            uint32_t lt = 0u, lo = 0u, hi = 0u;
-#pragma unroll
-            for (int i = 0; i < P::CPW; ++i) {
-                const float a = acc[P::local_code(w, i)];
-                const uint32_t addr = __float_as_uint(fmaf(a, inv_cell, grid_bias)) & TQ_GRID_ADDR_MASK;
-                const tq_u2 cell = *reinterpret_cast<const tq_u2 *>(lds_grid + P::copy_of(i) * P::COPY_STRIDE + addr);
-                const float t = fmaf(a, inv, -__uint_as_float(cell[0]));
-                const int cursor = i == 0 ? 8 * P::WB : P::shift_of(i - 1);
-                const int gap = cursor - (P::shift_of(i) + P::FIELD);
-                if (gap > 0) lt = __builtin_amdgcn_alignbit(lt, 0u, 32 - gap);
-                lt = __builtin_amdgcn_alignbit(lt, __float_as_uint(t), 32 - P::FIELD);
-                if (P::IPB == 1 && P::byte_of(i) >= 2) hi |= cell[1]; else lo |= cell[1];
-            }
-            const uint32_t bases = P::IPB == 1 ? (lo | (hi << 16)) : lo;
-            const uint32_t ge = (~lt & P::sign_mask()) >> (P::FIELD - 1);
+            const uint32_t bases = P::IPB == 1 ? (z.lo[w] | (z.hi[w] << 16)) : z.lo[w];
+            const uint32_t ge = (~z.lt[w] & P::sign_mask()) >> (P::FIELD - 1);
             words[w] = bases + ge;
         }
+    };
+
+    // One tile, parked in buffer `b` and published by a barrier: rotate, then search.
+    // Leaves the lane's packed words in `words` and the vector's norm in `nrm`.
+    auto compute = [&](uint32_t b, uint32_t (&words)[NW], float &nrm) {
+        tq_f16v acc = tq_zero16();
+        float ss0 = 0.f, ss1 = 0.f;
+#pragma unroll
+        for (int s = 0; s < TQ_STEPS; ++s) rotate_step(lds_stage[b], s, acc, ss0, ss1);
+        const Scale sc = scale_of(b, ss0, ss1);
+        Search z;
+        search_begin(z);
+#pragma unroll
+        for (int q = 0; q < 16; ++q) search_coord(z, q, acc, sc);
+        search_end(z, words);
+        nrm = sc.nrm;
     };
 
     // the lane's NB packed bytes and (identical in all lanes of a vector) the fp16 norm
@@ -329,59 +357,154 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     };
     const uint32_t lane_slot = (2u * wave + hk) * NB;   // this lane's bytes inside a vector's G = 8 * NB
 
-    // Pipeline over the tiles whose 32 vectors all exist.  Iteration k: start the loads of tile k+1,
-    // barrier (publishes buffer k, and everyone has finished reading buffer k-1), compute and store
-    // tile k, then park tile k+1 into the other buffer.  Loads, stores and the wait for the loads sit
-    // in one straight line, in that order, and none of them is predicated, so the wait is
-    // s_waitcnt vmcnt(#stores): the stores of tile k stay in flight across the iteration boundary.
     const uint32_t n_full = job.n_vec / 32u;
     uint32_t buf = 0;
     uint32_t words[NW];
     float nrm;
-    if (tile < n_full) {
-        if (one_row) {
-            // running per-lane pointers: a handful of 64-bit adds per tile instead of index arithmetic
+    if (tile < n_full && ELEM == 2 && one_row) {
+        if constexpr (ELEM == 2) {
+            // Single-row jobs with 16-bit elements (the KV-cache case).  Software pipeline inside the
+            // wave, over this block's full tiles t_0 .. t_{m-1}: iteration j
+            //   starts the loads of t_{j+2} into the register set that t_j has just left,
+            //   passes the barrier that publishes t_j in LDS buffer j % 2,
+            //   rotates t_j on the matrix cores while searching and packing the codes of t_{j-1},
+            //   whose rotated coordinates wait in the other accumulator set: the two instruction
+            //   streams are independent, so the VALU work fills the issue slots under the MFMAs,
+            //   stores t_{j-1} and parks t_{j+1} (loaded an iteration ago) in the other LDS buffer.
+            // Loads, stores and the wait for the older loads sit in one straight line and none is
+            // predicated, so the wait is s_waitcnt vmcnt(n > 0): stores and the newer loads stay in
+            // flight.  Two tiles per wave are on their way from memory at any time.  Per-lane
+            // pointers run along the job: a handful of 64-bit adds per tile, no index arithmetic.
             const long long jstep = (long long)VEC_PER_LOAD * job.token_stride;
             const long long in_step = (long long)tile_stride * 32 * job.token_stride;
             const uint8_t *ld = job.states + (long long)(tile * 32u + (wave * NLOAD) * VEC_PER_LOAD + ld_vec) * job.token_stride + ld_piece * 16u;
             uint8_t *cd = job.idx_bytes + (size_t)(tile * 32u + n) * (8 * NB) + lane_slot;
             uint16_t *nd = job.vec_norms + (size_t)tile * 32u + n;
             const size_t cd_step = (size_t)tile_stride * 32u * (8 * NB), nd_step = (size_t)tile_stride * 32u;
-            issue_loads_ptr(ld, jstep);
-            park(0);
-            while (tile < n_full) {
-                const uint32_t next = tile + tile_stride;
-                ld += next < n_full ? in_step : 0;                       // last iteration: harmless re-read
-                issue_loads_ptr(ld, jstep);
+            const uint32_t m = (n_full - tile + tile_stride - 1u) / tile_stride;   // this block's full tiles
+            uint32_t ahead = m - 1u;      // tiles beyond the one `ld` points at
+            uint32_t to_rotate = m;
+
+            tq_u4 set0[NLOAD], set1[NLOAD];
+            // past the block's last tile the pointer stays where it is: a harmless re-read, never used
+            auto load_next = [&](tq_u4 (&dst)[NLOAD]) {
+#pragma unroll
+                for (int j = 0; j < NLOAD; ++j) dst[j] = tq_gload16(ld + j * jstep);
+                ld += ahead ? in_step : 0;
+                ahead -= ahead ? 1u : 0u;
+            };
+            // iteration j: `fresh` receives t_{j+2}, `ready` holds t_{j+1}; `acc_new` receives t_j,
+            // (`acc_old`, `sc_old`) belong to t_{j-1}
+            auto iteration = [&](auto with_search, uint32_t b, tq_u4 (&fresh)[NLOAD], const tq_u4 (&ready)[NLOAD],
+                                 tq_f16v &acc_new, Scale &sc_new, const tq_f16v &acc_old, const Scale &sc_old) {
+                constexpr bool SEARCH = decltype(with_search)::value;
+                load_next(fresh);
                 __syncthreads();
-                compute(buf, words, nrm);
-                store(cd, nd, words, nrm);
-                cd += cd_step;
-                nd += nd_step;
-                buf ^= 1u;
-                park(buf);
-                tile = next;
+                acc_new = tq_zero16();
+                Search z;
+                search_begin(z);
+                const uint8_t *stage = lds_stage[b];
+                auto operand = [&](int s) {
+                    const uint32_t piece = 2u * s + hk;
+                    return *reinterpret_cast<const tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4));
+                };
+                auto mfma = [&](int term, int s, tq_u4 bop) {
+                    acc_new = (DTYPE == TQ_F16) ? mfma_f16(areg[term][s], bop, acc_new) : mfma_bf16(areg[term][s], bop, acc_new);
+                };
+                // LDS reads run one step ahead of their use: the operand of step s + 1 and the grid
+                // cells of coordinates 2s + 2, 2s + 3 are requested before the MFMAs of step s
+                tq_u4 bop = operand(0);
+                tq_u2 c0 = {0u, 0u}, c1 = {0u, 0u};
+                if constexpr (SEARCH) {
+                    c0 = search_lookup(0, acc_old, sc_old);
+                    c1 = search_lookup(1, acc_old, sc_old);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+                }
+#pragma unroll
+                for (int s = 0; s < TQ_STEPS; ++s) {
+                    tq_u4 bop_next = bop;
+                    tq_u2 n0 = c0, n1 = c1;
+                    if (s + 1 < TQ_STEPS) {
+                        bop_next = operand(s + 1);
+                        if constexpr (SEARCH) { n0 = search_lookup(2 * s + 2, acc_old, sc_old); n1 = search_lookup(2 * s + 3, acc_old, sc_old); }
+                    }
+                    mfma(0, s, bop);
+                    if constexpr (SEARCH) search_apply(z, 2 * s, acc_old, sc_old, c0);
+                    mfma(1, s, bop);
+                    if constexpr (SEARCH) search_apply(z, 2 * s + 1, acc_old, sc_old, c1);
+                    if constexpr (SEARCH) {
+                        // pin the order: address arithmetic, the step's LDS reads, then each MFMA
+                        // followed by the VALU work that fills its shadow
+                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);   // VALU
+                        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);   // DS read
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                    }
+                    bop = bop_next; c0 = n0; c1 = n1;
+                }
+                const float ss0 = 0.f, ss1 = 0.f;
+                sc_new = scale_of(b, ss0, ss1);
+                if constexpr (SEARCH) {
+                    search_end(z, words);
+                    store(cd, nd, words, sc_old.nrm);
+                    cd += cd_step;
+                    nd += nd_step;
+                }
+                park(b ^ 1u, ready);
+            };
+            auto drain = [&](const tq_f16v &acc_old, const Scale &sc_old) {
+                Search z;
+                search_begin(z);
+#pragma unroll
+                for (int q = 0; q < 16; ++q) search_coord(z, q, acc_old, sc_old);
+                search_end(z, words);
+                store(cd, nd, words, sc_old.nrm);
+            };
+
+            load_next(set0);
+            load_next(set1);
+            park(0u, set0);
+            tq_f16v acc_a, acc_b;
+            Scale sc_a, sc_b;
+            iteration(std::false_type{}, 0u, set0, set1, acc_a, sc_a, acc_a, sc_a);
+            --to_rotate;
+            while (true) {
+                if (to_rotate == 0u) { drain(acc_a, sc_a); break; }
+                iteration(std::true_type{}, 1u, set1, set0, acc_b, sc_b, acc_a, sc_a);
+                --to_rotate;
+                if (to_rotate == 0u) { drain(acc_b, sc_b); break; }
+                iteration(std::true_type{}, 0u, set0, set1, acc_a, sc_a, acc_b, sc_b);
+                --to_rotate;
             }
-        } else {
-            issue_loads(std::true_type{}, tile);
-            park(0);
-            while (tile < n_full) {
-                const uint32_t next = tile + tile_stride;
-                issue_loads(std::true_type{}, next < n_full ? next : tile);
-                __syncthreads();
-                compute(buf, words, nrm);
-                const uint32_t v = tile * 32u + n;
-                store(job.idx_bytes + (size_t)v * (8 * NB) + lane_slot, job.vec_norms + v, words, nrm);
-                buf ^= 1u;
-                park(buf);
-                tile = next;
-            }
+            tile += m * tile_stride;
+            buf = m & 1u;   // the buffer nobody reads while slower waves finish the last iteration
+        }
+    } else if (tile < n_full) {
+        // General case (several rows with their own stride, fp32 elements).  Iteration k: start the
+        // loads of tile k+1, barrier (publishes buffer k, and everyone has finished reading buffer
+        // k-1), compute and store tile k, then park tile k+1 into the other buffer.  Loads, stores
+        // and the wait for the loads sit in one straight line, unpredicated: s_waitcnt vmcnt(#stores).
+        issue_loads(std::true_type{}, tile);
+        park(0, pre);
+        while (tile < n_full) {
+            const uint32_t next = tile + tile_stride;
+            issue_loads(std::true_type{}, next < n_full ? next : tile);
+            __syncthreads();
+            compute(buf, words, nrm);
+            const uint32_t v = tile * 32u + n;
+            store(job.idx_bytes + (size_t)v * (8 * NB) + lane_slot, job.vec_norms + v, words, nrm);
+            buf ^= 1u;
+            park(buf, pre);
+            tile = next;
         }
     }
     // the partial last tile of the job, if this block is the one whose turn it is
     if (tile == n_full && n_full < n_tiles) {
         issue_loads(std::false_type{}, tile);
-        park(buf);
+        park(buf, pre);
         __syncthreads();
         compute(buf, words, nrm);
         const uint32_t v = tile * 32u + n;
@@ -419,8 +542,16 @@ int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uin
     DeviceInfo info;
     int rc = query_device(info);
     if (rc) return rc;
-    // Three four-wave blocks fit on a compute unit (registers: three waves per SIMD).
-    const uint32_t bx = tq_blocks_per_job(max_tiles, info.cus * 3, n_jobs);
+    // blocks resident per compute unit for this instantiation (registers and LDS decide): the grid
+    // is that many blocks per unit, each walking its share of the tiles
+    static int resident = 0;
+    if (resident == 0) {
+        int nb = 0;
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, tq_compress_kernel<DTYPE, BITS>, CTHREADS, 0);
+        if (e != hipSuccess) return (int)e;
+        resident = nb > 0 ? nb : 1;
+    }
+    const uint32_t bx = tq_blocks_per_job(max_tiles, info.cus * resident, n_jobs);
     dim3 grid(bx, (unsigned)n_jobs, 1), block(CTHREADS, 1, 1);
     hipLaunchKernelGGL((tq_compress_kernel<DTYPE, BITS>), grid, block, 0, stream, job, jobs_dev);
     return (int)hipGetLastError();
