@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define TQ_ABI_VERSION 1
+#define TQ_ABI_VERSION 2
 
 /* element types of K/V tensors */
 enum { TQ_F32 = 0, TQ_F16 = 1, TQ_BF16 = 2 };
@@ -96,23 +96,32 @@ int tq_table_quantize_host(const void *table_host, const float *r, long long n, 
  *               [:, :, :s, :] of one is rows=B*H, tokens=s, row_stride=S*128.
  *               Base address and strides must keep every vector 16-byte aligned.
  *   table_dev   device copy of the blob from tq_table_build
- *   idx_bytes   device, [rows*tokens, bytes_per_vector] uint8, contiguous
- *   vec_norms   device, [rows*tokens] IEEE fp16 bit patterns (norm of the fp32-widened vector)
+ *   idx_bytes   device, uint8, bytes_per_vector per packed slot
+ *   vec_norms   device, one IEEE fp16 bit pattern per packed slot (norm of the fp32-widened vector)
+ *   packed_row_stride
+ *               vector n uses packed slot  (n / tokens) * packed_row_stride + (n % tokens)  of
+ *               idx_bytes and vec_norms.  0 means `tokens`: the dense [rows*tokens] layout the
+ *               reference returns.  A larger value appends to a preallocated per-row store
+ *               [rows, capacity]: pass pointers already advanced to the first free token and
+ *               packed_row_stride = capacity (the chunk list of generation_test_v2.py:109-126
+ *               kept as one buffer).
  *   stream      hipStream_t (NULL = the default stream)
  */
 int tq_compress(const void *states, int dtype, long long rows, long long tokens,
                 long long row_stride, long long token_stride,
                 const void *table_dev, int head_dim, int bits,
-                uint8_t *idx_bytes, uint16_t *vec_norms, void *stream);
+                uint8_t *idx_bytes, uint16_t *vec_norms, long long packed_row_stride, void *stream);
 
 /*
  * decompress: packed codes + fp16 norms -> vectors of `out_dtype`.
  * Replaces MSECompressor.decompress, compressors_v3.py:84-105 (out_dtype = TQ_F32), and with
  * TQ_F16 / TQ_BF16 the fused `.to(dtype)` + torch.cat into the full-length K/V buffer of
  * TurboQuantV3.decompress_kv, compressors_v3.py:226-232: vector n is written at element
- *   (n / tokens) * row_stride + (n % tokens) * token_stride   of `out`.
+ *   (n / tokens) * row_stride + (n % tokens) * token_stride   of `out`
+ * and read from packed slot (n / tokens) * packed_row_stride + (n % tokens) (0 = dense), which
+ * also covers the loop over stored chunks of generation_test_v2.py:131-135.
  */
-int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms,
+int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long packed_row_stride,
                   long long rows, long long tokens,
                   const void *table_dev, int head_dim, int bits,
                   void *out, int out_dtype, long long row_stride, long long token_stride,
@@ -137,6 +146,7 @@ typedef struct tq_job {
     long long token_stride;    /* elements, for `states`                                  */
     int bits;                  /* 1..8, must match the table                              */
     int dtype;                 /* element type of `states`                                */
+    long long packed_row_stride; /* packed slots per row of idx_bytes / vec_norms; 0 = tokens */
 } tq_job;
 
 #define TQ_MAX_JOBS 4096

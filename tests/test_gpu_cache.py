@@ -1,0 +1,151 @@
+"""GPU tests of the append-in-place packed store (packed_row_stride of the C ABI) and of the
+streaming cache built on it, against the dense kernels, the CPU oracle and the bookkeeping of
+the reference's generation-time cache (generation_test_v2.py:80-165)."""
+import numpy as np
+import pytest
+import torch
+
+from test_gpu_parity import DEV, bits16, outlier_kv, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.fail("these tests need a HIP device; there is no CPU fallback to test")
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_append_to_packed_store_equals_dense(pkg, bits):
+    """Chunks compressed into consecutive token slots of a [B,H,capacity,G] store give the bytes of
+    one dense call over the concatenated tokens; de-quantising a slice of the store gives the dense
+    result; slots outside the written range stay untouched."""
+    B, H, cap, D = 2, 3, 192, 128
+    comp = pkg.MSECompressor(D, bits, seed=5, device=DEV)
+    G = D // (8 // bits)
+    x = outlier_kv((B, H, 150, D), seed=bits, dtype=torch.bfloat16).to(DEV)
+    store = torch.full((B, H, cap, G), 0xEE, dtype=torch.uint8, device=DEV)
+    norms = torch.full((B, H, cap), -7.0, dtype=torch.float16, device=DEV)
+    pos = 3                                   # start away from slot 0: pointers are advanced, not rows
+    for lo, hi in ((0, 70), (70, 71), (71, 150)):          # many tokens, a single one, a ragged rest
+        n = hi - lo
+        comp.compress_into(x[:, :, lo:hi], store[:, :, pos:pos + n], norms[:, :, pos:pos + n])
+        pos += n
+    dense = comp.compress(x)
+    assert torch.equal(store[:, :, 3:153], dense["idx_bytes"])
+    assert torch.equal(norms[:, :, 3:153], dense["vec_norms"])
+    assert bool((store[:, :, :3] == 0xEE).all()) and bool((store[:, :, 153:] == 0xEE).all())
+    assert bool((norms[:, :, :3] == -7).all()) and bool((norms[:, :, 153:] == -7).all())
+    want = torch.empty(B, H, 150, D, dtype=torch.bfloat16, device=DEV)
+    comp.decompress_into(dense, want)
+    out = torch.zeros(B, H, 160, D, dtype=torch.bfloat16, device=DEV)
+    comp.decompress_packed(store[:, :, 3:153], norms[:, :, 3:153], out[:, :, :150])
+    assert torch.equal(out[:, :, :150], want) and not bool(out[:, :, 150:].any())
+    # one row, one token: the smallest append
+    one = torch.zeros(1, 1, 8, G, dtype=torch.uint8, device=DEV)
+    onen = torch.zeros(1, 1, 8, dtype=torch.float16, device=DEV)
+    comp.compress_into(x[:1, :1, 4:5], one[:, :, 6:7], onen[:, :, 6:7])
+    assert torch.equal(one[0, 0, 6], dense["idx_bytes"][0, 0, 4]) and not bool(one[0, 0, :6].any())
+
+
+def test_batched_jobs_with_packed_row_stride(pkg):
+    native = pkg._native
+    comps = [pkg.MSECompressor(128, 4, seed=100 + l, device=DEV) for l in range(3)]
+    xs = [outlier_kv((2, 2, 90 + l, 128), seed=40 + l, dtype=torch.float16).to(DEV) for l in range(3)]
+    stores = [torch.zeros(2, 2, 128, 64, dtype=torch.uint8, device=DEV) for _ in range(3)]
+    norms = [torch.zeros(2, 2, 128, dtype=torch.float16, device=DEV) for _ in range(3)]
+    jobs = [{"states": x, "idx_bytes": s[:, :, 10:10 + x.shape[2]], "vec_norms": n[:, :, 10:10 + x.shape[2]],
+             "table": c.table(), "bits": 4} for x, s, n, c in zip(xs, stores, norms, comps)]
+    native.JobList(jobs, DEV).compress()
+    torch.cuda.synchronize()
+    for x, s, n, c in zip(xs, stores, norms, comps):
+        d = c.compress(x)
+        assert torch.equal(s[:, :, 10:10 + x.shape[2]], d["idx_bytes"]) and torch.equal(n[:, :, 10:10 + x.shape[2]], d["vec_norms"])
+        assert not bool(s[:, :, :10].any()) and not bool(s[:, :, 10 + x.shape[2]:].any())
+    outs = [torch.zeros_like(x) for x in xs]
+    native.JobList([dict(j, states=o) for j, o in zip(jobs, outs)], DEV).decompress()
+    torch.cuda.synchronize()
+    for x, o, c in zip(xs, outs, comps):
+        want = torch.empty_like(x)
+        c.decompress_into(c.compress(x), want)
+        assert torch.equal(o, want)
+
+
+@pytest.mark.parametrize("rw", [0, 16, 128])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_v3cache_stream_equals_one_shot_codec(pkg, oracle, rw, dtype):
+    """Prefill, single-token decode steps and a multi-token step through V3Cache.update.  After every
+    call: length and bookkeeping as the reference's cache computes them, the uncompressed tail
+    bit-identical to the incoming tokens, the de-quantised part bit-identical to one dense
+    compress + decompress over the same tokens (codes do not depend on the chunking), and within
+    tolerance of the CPU oracle's decode of the stored bytes."""
+    B, H, D, L = 2, 2, 128, 2
+    cache = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=rw, protected_layers=0, n_layers=L)
+    steps = [150, 1, 1, 1, 7, 1, 40, 1]
+    keys = [outlier_kv((B, H, sum(steps), D), seed=300 + l, dtype=dtype).to(DEV) for l in range(L)]
+    vals = [outlier_kv((B, H, sum(steps), D), seed=400 + l, dtype=dtype).to(DEV) for l in range(L)]
+    seen = 0
+    for n_new in steps:
+        for l in range(L):
+            fk, fv = cache.update(keys[l][:, :, seen:seen + n_new], vals[l][:, :, seen:seen + n_new], l)
+            total = seen + n_new
+            n_c = total if rw == 0 else max(total - rw, 0)
+            assert fk.shape == (B, H, total, D) and fv.shape == fk.shape and fk.dtype == dtype
+            assert cache.get_seq_length(l) == total
+            assert torch.equal(fk[:, :, n_c:], keys[l][:, :, n_c:total]), (rw, total)
+            assert torch.equal(fv[:, :, n_c:], vals[l][:, :, n_c:total])
+            if n_c:
+                tq = cache._get_compressor(l, D, DEV)
+                assert tq.residual_window == 0
+                ck, cv = tq.compress_kv(keys[l][:, :, :n_c], vals[l][:, :, :n_c])
+                dk, dv = tq.decompress_kv(ck, cv)
+                assert torch.equal(fk[:, :, :n_c], dk) and torch.equal(fv[:, :, :n_c], dv), (rw, total)
+        seen += n_new
+    total = sum(steps)
+    n_c = total if rw == 0 else total - rw
+    assert cache.get_compression_info() == f"{n_c} compressed, {total - n_c} fp16, {total} total"
+    # stored bytes decoded by the oracle
+    st = cache._stores[1]
+    tq = cache._get_compressor(1, D, DEV)
+    for comp, idx, nrm, full in ((tq.key_compressor, st.k_idx, st.k_nrm, fk), (tq.val_compressor, st.v_idx, st.v_nrm, fv)):
+        orc = oracle.COracle(comp.Pi.cpu().numpy(), comp.centroids.cpu().numpy(), comp.bits, True)
+        packed = idx[:, :, :n_c].contiguous().cpu().numpy().reshape(-1, idx.shape[-1])
+        ref = orc.decompress(packed, bits16(nrm[:, :, :n_c].contiguous()).reshape(-1))
+        err, _ = rel_l2(full[:, :, :n_c].float().cpu().numpy().reshape(-1, D), ref)
+        assert err < 5e-3, err               # bf16 / fp16 rounding of the output on top of the 1e-3 bar
+    assert cache.stored_bytes() == L * B * H * (n_c * (64 + 32 + 4) + 2 * (total - n_c) * D * 2)
+
+
+def test_v3cache_grows_and_protects_layers(pkg):
+    """Capacity doubles without losing history; protected layers store 8-bit codes for K and V."""
+    cache = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=8, protected_layers=1, n_layers=3)
+    x = outlier_kv((1, 2, 700, 128), seed=9, dtype=torch.bfloat16).to(DEV)
+    out = None
+    for lo in range(0, 700, 100):
+        for l in range(3):
+            out = cache.update(x[:, :, lo:lo + 100], x[:, :, lo:lo + 100], l)
+    assert cache._stores[0].k_idx.shape[-1] == 128 and cache._stores[0].v_idx.shape[-1] == 128
+    assert cache._stores[1].k_idx.shape[-1] == 64 and cache._stores[1].v_idx.shape[-1] == 32
+    assert cache._stores[2].k_idx.shape[-1] == 128
+    assert cache._stores[1].capacity >= 692 and cache._stores[1].n_compressed == 692
+    tq = cache._get_compressor(2, 128, DEV)
+    ck, cv = tq.compress_kv(x[:, :, :692], x[:, :, :692])
+    dk, _ = tq.decompress_kv(ck, cv)
+    assert torch.equal(out[0][:, :, :692], dk) and torch.equal(out[0][:, :, 692:], x[:, :, 692:])
+    with pytest.raises(ValueError):
+        cache.update(x[:, :1, :1], x[:, :1, :1], 0)          # head count changed
+
+
+def test_hf_dynamic_cache_subclass(pkg):
+    """The transformers-facing subclass keeps DynamicCache's interface alive around update()."""
+    transformers = pytest.importorskip("transformers")
+    cls = pkg.hf_cache_class()
+    cache = cls(key_bits=4, value_bits=2, residual_window=4, n_layers=2)
+    assert isinstance(cache, transformers.DynamicCache) and isinstance(cache, pkg.V3Cache)
+    x = outlier_kv((1, 2, 12, 128), seed=1, dtype=torch.float16).to(DEV)
+    for l in range(2):
+        k, v = cache.update(x, x, l)
+        assert k.shape == (1, 2, 12, 128)
+    assert cache.get_seq_length() == 12 and cache.get_seq_length(1) == 12
+    assert cache.get_compression_info() == "8 compressed, 4 fp16, 12 total"

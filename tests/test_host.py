@@ -7,6 +7,8 @@ behaviour of the C entry points, and that the library exports what include/tqamd
 import ctypes
 import os
 import re
+import shutil
+import subprocess
 
 import numpy as np
 import pytest
@@ -23,14 +25,30 @@ def test_library_exports_every_declared_symbol(pkg):
     for name in declared:
         assert hasattr(lib, name), name
     assert sorted(pkg._native.EXPORTS) == declared
-    assert lib.tq_abi_version() == 1
+    assert lib.tq_abi_version() == 2
     assert lib.tq_status_string(0) == b"ok"
     assert b"bits" in lib.tq_status_string(-2)
 
 
-def test_job_struct_layout_matches_header(pkg):
-    # 4 pointers + 4 int64 + 2 int32 = 72 bytes, no padding surprises
-    assert ctypes.sizeof(pkg._native.TqJob) == 72
+def test_job_struct_layout_matches_header(pkg, tmp_path):
+    # 4 pointers + 4 int64 + 2 int32 + 1 int64 = 80 bytes
+    J = pkg._native.TqJob
+    assert ctypes.sizeof(J) == 80
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler to read the header with")
+    fields = [f[0] for f in J._fields_]
+    src = tmp_path / "layout.c"
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "tqamd.h"\nint main(void) {\n'
+                   '  printf("%zu", sizeof(tq_job));\n'
+                   + "".join(f'  printf(" %zu", offsetof(tq_job, {f}));\n' for f in fields)
+                   + '  printf(" %d\\n", TQ_ABI_VERSION);\n  return 0;\n}\n')
+    exe = tmp_path / "layout"
+    subprocess.run([gcc, "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert int(out[0]) == ctypes.sizeof(J)
+    assert [int(x) for x in out[1:-1]] == [getattr(J, f).offset for f in fields]
+    assert int(out[-1]) == pkg._native.lib().tq_abi_version()
 
 
 def test_codebooks_match_reference_bits(pkg, golden):
@@ -253,7 +271,7 @@ def test_c_abi_argument_errors(pkg):
     args = dict(rows=1, tokens=4, rs=0, ts=128)
     call = lambda states, dtype, bits, hd, idx=p, norms=p, table=p, **kw: lib.tq_compress(
         states, dtype, kw.get("rows", 1), kw.get("tokens", 4), kw.get("rs", 0), kw.get("ts", 128), table, hd, bits,
-        idx, norms, None)
+        idx, norms, kw.get("prs", 0), None)
     assert call(p, 1, 0, 128) == E["BITS"]
     assert call(p, 1, 4, 64) == E["HEAD_DIM"]
     assert call(p, 7, 4, 128) == E["DTYPE"]
@@ -263,9 +281,12 @@ def test_c_abi_argument_errors(pkg):
     assert call(p, 1, 4, 128, tokens=-1) == E["SIZE"]
     assert call(p, 1, 4, 128, ts=132) == E["ALIGN"]
     assert call(None, 1, 4, 128, tokens=0) == 0          # empty input: nothing to do, not an error
-    assert lib.tq_decompress(p, p, 1, 4, p, 128, 9, p, 0, 0, 128, None) == E["BITS"]
-    assert lib.tq_decompress(p, p, 1, 4, p, 128, 4, None, 0, 0, 128, None) == E["NULL"]
-    assert lib.tq_decompress(p, p, 1, 0, p, 128, 4, None, 0, 0, 128, None) == 0
+    assert call(p, 1, 4, 128, rows=2, rs=1024, prs=3) == E["SIZE"]   # packed rows shorter than the token count
+    assert call(p, 1, 4, 128, rows=2, rs=1024, prs=1 << 31) == E["SIZE"]
+    assert lib.tq_decompress(p, p, 0, 1, 4, p, 128, 9, p, 0, 0, 128, None) == E["BITS"]
+    assert lib.tq_decompress(p, p, 0, 1, 4, p, 128, 4, None, 0, 0, 128, None) == E["NULL"]
+    assert lib.tq_decompress(p, p, 0, 1, 0, p, 128, 4, None, 0, 0, 128, None) == 0
+    assert lib.tq_decompress(p, p, 2, 2, 4, p, 128, 4, p, 1, 1024, 128, None) == E["SIZE"]
     assert lib.tq_compress_batched(None, None, 0, 128, None) == 0
     assert lib.tq_compress_batched(None, None, 3, 128, None) == E["NULL"]
 
@@ -282,3 +303,51 @@ def test_vector_layout_reduction(pkg):
     assert vl(torch.zeros(2, 40, 3, 128).transpose(1, 2)) is None            # three stride levels
     assert vl(torch.zeros(1, 1, 0, 128)) == (0, 0, 0, 128)
     assert vl(torch.zeros(2, 3, 40, 130, dtype=torch.float16)[..., :128]) is None   # rows not 16-byte aligned
+
+
+def test_row_layout_and_packed_row_stride(pkg):
+    nat = pkg._native
+    store = torch.zeros(2, 3, 64, 32, dtype=torch.uint8)
+    norms = torch.zeros(2, 3, 64, dtype=torch.float16)
+    assert nat.packed_row_stride(store, norms) == 0
+    assert nat.packed_row_stride(store[:, :, 8:24], norms[:, :, 8:24]) == 64
+    assert nat.packed_row_stride(store[:, :, :64], norms[:, :, :64]) == 0
+    assert nat.packed_row_stride(store[:, :, 8:24], norms[:, :, 8:25]) is None       # shapes differ
+    assert nat.packed_row_stride(store[:, :, ::2], norms[:, :, ::2]) is None         # not a slice
+    assert nat.packed_row_stride(store[:, :, 8:24], torch.zeros(2, 3, 32, dtype=torch.float16)[:, :, 8:24]) is None
+    x = torch.zeros(2, 3, 40, 128, dtype=torch.float16)
+    assert nat.row_layout(x) == (6, 40, 40 * 128, 128)
+    assert nat.row_layout(x[:, :, 5:6]) == (6, 1, 40 * 128, 128)
+    assert nat.row_layout(x[:1, :1]) == (1, 40, 0, 128)
+    assert nat.row_layout(torch.zeros(2, 40, 3, 128).transpose(1, 2)) is None        # batch and head do not merge
+    assert nat.row_layout(torch.zeros(1, 40, 3, 128, dtype=torch.float16).transpose(1, 2)) == (3, 40, 128, 384)
+
+
+def test_compute_metrics_definition(pkg):
+    """The batched metric equals the per-head loop it replaces, on batch element 0 only."""
+    g = torch.Generator().manual_seed(3)
+    real = torch.randn(2, 6, 50, generator=g)
+    tq = real + 0.3 * torch.randn(2, 6, 50, generator=g)
+    tq[0, 2] = -real[0, 2]                                  # one head that disagrees completely
+    m = pkg.compute_metrics(real, tq, 6)
+    cos, t1, t5 = [], 0, 0
+    for h in range(6):
+        rs, ts = real[0, h], tq[0, h]
+        cos.append(torch.nn.functional.cosine_similarity(rs.unsqueeze(0), ts.unsqueeze(0)).item())
+        t1 += int(rs.argmax().item() == ts.argmax().item())
+        t5 += int(rs.argmax().item() in ts.topk(5).indices.tolist())
+    assert abs(m["cosine_sim"] - sum(cos) / 6) < 1e-6
+    assert (m["top1_matches"], m["top5_matches"], m["n_checks"]) == (t1, t5, 6)
+    assert m["top1_pct"] == 100 * t1 / 6 and m["top5_pct"] == 100 * t5 / 6 and t1 < 6
+    same = pkg.compute_metrics(real, real.clone(), 6)
+    assert abs(same["cosine_sim"] - 1) < 1e-6 and same["top1_pct"] == 100 and same["top5_pct"] == 100
+    q = torch.randn(1, 2, 1, 8, generator=g)
+    k = torch.randn(1, 2, 5, 8, generator=g)
+    assert torch.allclose(pkg.attention_scores(q, k), torch.einsum("bhqd,bhsd->bhs", q, k), atol=1e-6)
+
+
+def test_v3cache_refuses_cpu_tensors_and_reports_state(pkg):
+    cache = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=4, n_layers=2)
+    assert cache.get_seq_length() == 0 and cache.get_compression_info() == "no compression"
+    with pytest.raises(Exception):                          # no CPU path: the codec tables live on HIP devices
+        cache.update(torch.zeros(1, 1, 8, 128), torch.zeros(1, 1, 8, 128), 0)

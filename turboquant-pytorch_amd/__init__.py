@@ -9,9 +9,12 @@ alias module at the repository root (or `importlib.import_module("turboquant-pyt
 from .lloyd_max import LloydMaxCodebook, solve_lloyd_max
 from .rotation import generate_rotation_matrix
 from .compressors_v3 import MSECompressor, TurboQuantV3
+from .kv_cache import V3Cache, hf_cache_class
+from .metrics import attention_scores, compute_metrics
 from . import _native
 
 __all__ = [
-    "MSECompressor", "TurboQuantV3", "LloydMaxCodebook", "solve_lloyd_max",
+    "MSECompressor", "TurboQuantV3", "V3Cache", "hf_cache_class", "attention_scores", "compute_metrics",
+    "LloydMaxCodebook", "solve_lloyd_max",
     "generate_rotation_matrix", "_native",
 ]

@@ -79,6 +79,7 @@ class TqJob(ctypes.Structure):
         ("token_stride", ctypes.c_longlong),
         ("bits", ctypes.c_int),
         ("dtype", ctypes.c_int),
+        ("packed_row_stride", ctypes.c_longlong),
     ]
 
 
@@ -112,8 +113,8 @@ def lib() -> ctypes.CDLL:
     L.tq_table_bytes.argtypes = [ci, ci]
     L.tq_table_build.argtypes = [vp, vp, ci, ci, vp, ctypes.c_size_t]
     L.tq_table_quantize_host.argtypes = [vp, vp, ll, vp]
-    L.tq_compress.argtypes = [vp, ci, ll, ll, ll, ll, vp, ci, ci, vp, vp, vp]
-    L.tq_decompress.argtypes = [vp, vp, ll, ll, vp, ci, ci, vp, ci, ll, ll, vp]
+    L.tq_compress.argtypes = [vp, ci, ll, ll, ll, ll, vp, ci, ci, vp, vp, ll, vp]
+    L.tq_decompress.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, ll, ll, vp]
     L.tq_compress_batched.argtypes = [vp, vp, ci, ci, vp]
     L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp]
     for name in EXPORTS:
@@ -210,39 +211,81 @@ def vector_layout(t: torch.Tensor) -> Optional[Tuple[int, int, int, int]]:
     return None
 
 
+def row_layout(t: torch.Tensor) -> Optional[Tuple[int, int, int, int]]:
+    """Like vector_layout, but always rows = B*H and tokens = S (the form a per-row packed store
+    needs); None if the batch and head dimensions do not merge."""
+    B, H, S, D = t.shape
+    sb, sh, ss, sd = t.stride()
+    if D != 1 and sd != 1:
+        return None
+    esz = t.element_size()
+    if (t.data_ptr() % 16) or any((st * esz) % 16 for st in (sb, sh, ss)):
+        return None
+    if B != 1 and H != 1 and sb != H * sh:
+        return None
+    row_stride = sh if H != 1 else sb
+    return (B * H, S, row_stride if B * H > 1 else 0, ss if S > 1 else D)
+
+
+def packed_row_stride(idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> Optional[int]:
+    """Packed slots per (batch, head) row of a [B,H,S,G] / [B,H,S] pair of packed buffers: 0 when
+    both are contiguous, the row capacity when they are token-axis slices of a [B,H,capacity,..]
+    store, None when they are neither."""
+    if idx_bytes.is_contiguous() and vec_norms.is_contiguous():
+        return 0
+    B, H, S, G = idx_bytes.shape
+    if tuple(vec_norms.shape) != (B, H, S):
+        return None
+    sb, sh, ss, sg = idx_bytes.stride()
+    nb, nh, ns = vec_norms.stride()
+    if sg != 1 or ss != G or ns != 1 or sh % G or sh // G != nh or sh // G < S:
+        return None
+    if B != 1 and (sb != H * sh or nb != H * nh):
+        return None
+    return sh // G
+
+
 def _stream_handle(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
 def compress_into(states: torch.Tensor, table: torch.Tensor, bits: int,
                   idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> None:
-    """Launch tq_compress on `states` ([B,H,S,128], any supported float type, last dim dense)."""
+    """Launch tq_compress on `states` ([B,H,S,128], any supported float type, last dim dense).
+    The packed buffers are contiguous, or token-axis slices of a [B,H,capacity,..] store."""
     _require_gpu(states, "states")
     _require_gpu(table, "codec table")
-    lay = vector_layout(states)
+    prs = packed_row_stride(idx_bytes, vec_norms)
+    if prs is None:
+        raise TqError("packed buffers must be contiguous or token-axis slices of one [B,H,capacity,..] store")
+    lay = row_layout(states) if prs else vector_layout(states)
     if lay is None:
         states = states.contiguous()
-        lay = vector_layout(states)
+        lay = row_layout(states) if prs else vector_layout(states)
     rows, tokens, row_stride, token_stride = lay
     with torch.cuda.device(states.device):
         rc = lib().tq_compress(states.data_ptr(), dtype_code(states.dtype), rows, tokens, row_stride, token_stride,
                                table.data_ptr(), states.shape[-1], bits,
-                               idx_bytes.data_ptr(), vec_norms.data_ptr(), _stream_handle(states.device))
+                               idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, _stream_handle(states.device))
     check(rc, "tq_compress")
 
 
 def decompress_into(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
                     out: torch.Tensor) -> None:
-    """Launch tq_decompress, writing vector n of the packed stream to `out` ([B,H,S,128] view)."""
+    """Launch tq_decompress, writing vector n of the packed stream to `out` ([B,H,S,128] view).
+    The packed buffers are contiguous, or token-axis slices of a [B,H,capacity,..] store."""
     _require_gpu(idx_bytes, "idx_bytes")
     _require_gpu(out, "output")
-    lay = vector_layout(out)
+    prs = packed_row_stride(idx_bytes, vec_norms)
+    if prs is None:
+        idx_bytes, vec_norms, prs = idx_bytes.contiguous(), vec_norms.contiguous(), 0
+    lay = row_layout(out) if prs else vector_layout(out)
     if lay is None:
         raise TqError("decompress output must have a dense last dimension, 16-byte aligned rows and at most "
                       "two stride levels")
     rows, tokens, row_stride, token_stride = lay
     with torch.cuda.device(out.device):
-        rc = lib().tq_decompress(idx_bytes.data_ptr(), vec_norms.data_ptr(), rows, tokens, table.data_ptr(),
+        rc = lib().tq_decompress(idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, rows, tokens, table.data_ptr(),
                                  out.shape[-1], bits, out.data_ptr(), dtype_code(out.dtype), row_stride,
                                  token_stride, _stream_handle(out.device))
     check(rc, "tq_decompress")
@@ -273,12 +316,18 @@ def _(states, table, bits):
             states.new_empty((B, H, S), dtype=torch.float16))
 
 
+@torch.library.custom_op("tqamd::compress_into", mutates_args=("idx_bytes", "vec_norms"), device_types="cuda")
+def compress_into_op(states: torch.Tensor, table: torch.Tensor, bits: int,
+                     idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> None:
+    compress_into(states, table, bits, idx_bytes, vec_norms)
+
+
 @torch.library.custom_op("tqamd::decompress", mutates_args=(), device_types="cuda")
 def decompress_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
                   head_dim: int, out_dtype: torch.dtype) -> torch.Tensor:
     B, H, S, _ = idx_bytes.shape
     out = torch.empty((B, H, S, head_dim), dtype=out_dtype, device=idx_bytes.device)
-    decompress_into(idx_bytes.contiguous(), vec_norms.contiguous(), table, bits, out)
+    decompress_into(idx_bytes, vec_norms, table, bits, out)
     return out
 
 
@@ -291,7 +340,7 @@ def _(idx_bytes, vec_norms, table, bits, head_dim, out_dtype):
 @torch.library.custom_op("tqamd::decompress_into", mutates_args=("out",), device_types="cuda")
 def decompress_into_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
                        out: torch.Tensor) -> None:
-    decompress_into(idx_bytes.contiguous(), vec_norms.contiguous(), table, bits, out)
+    decompress_into(idx_bytes, vec_norms, table, bits, out)
 
 
 # ------------------------------------------------------------------------------------
@@ -311,13 +360,15 @@ class JobList:
         for i, j in enumerate(jobs):
             t = j["states"]
             _require_gpu(t, "states")
-            lay = vector_layout(t)
+            prs = packed_row_stride(j["idx_bytes"], j["vec_norms"])
+            lay = None if prs is None else (row_layout(t) if prs else vector_layout(t))
             if lay is None:
-                raise TqError("batched jobs need tensors with a dense last dimension and at most two stride levels")
+                raise TqError("batched jobs need tensors with a dense last dimension and at most two stride "
+                              "levels, and packed buffers that are contiguous or slices of a per-row store")
             rows, tokens, row_stride, token_stride = lay
             self.host[i] = TqJob(t.data_ptr(), j["idx_bytes"].data_ptr(), j["vec_norms"].data_ptr(),
                                  j["table"].data_ptr(), rows, tokens, row_stride, token_stride,
-                                 int(j["bits"]), dtype_code(t.dtype))
+                                 int(j["bits"]), dtype_code(t.dtype), prs)
             self._keep.append((t, j["idx_bytes"], j["vec_norms"], j["table"]))
         raw = np.frombuffer(bytes(self.host), dtype=np.uint8).copy()
         self.dev = torch.from_numpy(raw).to(self.device)

@@ -97,6 +97,32 @@ class MSECompressor:
         }
 
     @torch.no_grad()
+    def compress_into(self, states: torch.Tensor, idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> None:
+        """Compress (B, H, S, D) states into caller-owned packed buffers u8 [B,H,S,G] / f16 [B,H,S]:
+        contiguous tensors, or token-axis slices of a preallocated [B,H,capacity,..] store (appending
+        to a cache without reallocating it)."""
+        B, H, S, D = states.shape
+        width = math.ceil(D / (8 // self.bits))
+        if tuple(idx_bytes.shape) != (B, H, S, width) or tuple(vec_norms.shape) != (B, H, S):
+            raise ValueError(f"packed buffers {tuple(idx_bytes.shape)} / {tuple(vec_norms.shape)} do not match "
+                             f"states {tuple(states.shape)} at {self.bits} bits")
+        if idx_bytes.dtype != torch.uint8 or vec_norms.dtype != torch.float16:
+            raise ValueError("packed buffers must be uint8 codes and float16 norms")
+        if S * B * H:
+            torch.ops.tqamd.compress_into(states, self.table(), self.bits, idx_bytes, vec_norms)
+
+    @torch.no_grad()
+    def decompress_packed(self, idx_bytes: torch.Tensor, vec_norms: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """De-quantise packed buffers (as accepted by compress_into) into `out` [B,H,S,D]."""
+        B, H, S, D = out.shape
+        if tuple(idx_bytes.shape[:3]) != (B, H, S) or tuple(vec_norms.shape) != (B, H, S):
+            raise ValueError(f"packed buffers {tuple(idx_bytes.shape)} / {tuple(vec_norms.shape)} do not match "
+                             f"output {tuple(out.shape)}")
+        if S * B * H:
+            torch.ops.tqamd.decompress_into(idx_bytes, vec_norms, self.table(), self.bits, out)
+        return out
+
+    @torch.no_grad()
     def decompress(self, compressed: dict) -> torch.Tensor:
         """Back to a float32 (B, H, S, D) tensor."""
         B, H, S, D = compressed["shape"]

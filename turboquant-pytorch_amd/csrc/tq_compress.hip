@@ -494,8 +494,8 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             issue_loads(std::true_type{}, next < n_full ? next : tile);
             __syncthreads();
             compute(buf, words, nrm);
-            const uint32_t v = tile * 32u + n;
-            store(job.idx_bytes + (size_t)v * (8 * NB) + lane_slot, job.vec_norms + v, words, nrm);
+            const uint32_t slot = tq_packed_slot(job, tile * 32u + n);
+            store(job.idx_bytes + (size_t)slot * (8 * NB) + lane_slot, job.vec_norms + slot, words, nrm);
             buf ^= 1u;
             park(buf, pre);
             tile = next;
@@ -508,7 +508,10 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
         __syncthreads();
         compute(buf, words, nrm);
         const uint32_t v = tile * 32u + n;
-        if (v < job.n_vec) store(job.idx_bytes + (size_t)v * (8 * NB) + lane_slot, job.vec_norms + v, words, nrm);
+        if (v < job.n_vec) {
+            const uint32_t slot = tq_packed_slot(job, v);
+            store(job.idx_bytes + (size_t)slot * (8 * NB) + lane_slot, job.vec_norms + slot, words, nrm);
+        }
     }
 }
 
@@ -584,7 +587,7 @@ int elem_bytes(int dtype) { return dtype == TQ_F32 ? 4 : (dtype == TQ_F16 || dty
 // Shared argument checks of one job; fills n_vec.
 int check_job(const void *states, int dtype, long long rows, long long tokens, long long row_stride,
               long long token_stride, const void *table, int head_dim, int bits, const void *idx_bytes,
-              const void *vec_norms, long long *n_vec) {
+              const void *vec_norms, long long packed_row_stride, long long *n_vec) {
     if (bits < 1 || bits > 8) return TQ_ERR_BITS;
     if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
     const int eb = elem_bytes(dtype);
@@ -596,6 +599,7 @@ int check_job(const void *states, int dtype, long long rows, long long tokens, l
     if (!states || !table || !idx_bytes || !vec_norms) return TQ_ERR_NULL;
     if (token_stride < TQ_HEAD_DIM && tokens > 1) return TQ_ERR_SIZE;
     if (rows > 1 && row_stride < 0) return TQ_ERR_SIZE;
+    if (packed_row_stride != 0 && (packed_row_stride < tokens || packed_row_stride > (long long)0x7fffffff / rows)) return TQ_ERR_SIZE;
     if (((uintptr_t)states & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & 15u) || ((uintptr_t)vec_norms & 1u))
         return TQ_ERR_ALIGN;
     if (((token_stride * eb) & 15) || (rows > 1 && ((row_stride * eb) & 15))) return TQ_ERR_ALIGN;
@@ -606,10 +610,11 @@ int check_job(const void *states, int dtype, long long rows, long long tokens, l
 
 extern "C" int tq_compress(const void *states, int dtype, long long rows, long long tokens,
                            long long row_stride, long long token_stride, const void *table_dev,
-                           int head_dim, int bits, uint8_t *idx_bytes, uint16_t *vec_norms, void *stream) {
+                           int head_dim, int bits, uint8_t *idx_bytes, uint16_t *vec_norms,
+                           long long packed_row_stride, void *stream) {
     long long n_vec = 0;
     const int rc = check_job(states, dtype, rows, tokens, row_stride, token_stride, table_dev, head_dim, bits,
-                             idx_bytes, vec_norms, &n_vec);
+                             idx_bytes, vec_norms, packed_row_stride, &n_vec);
     if (rc || n_vec == 0) return rc;
     TqDevJob job;
     job.states = static_cast<const uint8_t *>(states);
@@ -618,6 +623,7 @@ extern "C" int tq_compress(const void *states, int dtype, long long rows, long l
     job.table = static_cast<const uint8_t *>(table_dev);
     job.n_vec = (uint32_t)n_vec;
     job.tokens = (uint32_t)tokens;
+    job.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     job.row_stride = row_stride * elem_bytes(dtype);
     job.token_stride = token_stride * elem_bytes(dtype);
     return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), static_cast<hipStream_t>(stream));
@@ -635,7 +641,7 @@ extern "C" int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_d
         if (j.dtype != jobs_host[0].dtype) return TQ_ERR_DTYPE;
         long long n_vec = 0;
         const int rc = check_job(j.states, j.dtype, j.rows, j.tokens, j.row_stride, j.token_stride, j.table_dev,
-                                 head_dim, j.bits, j.idx_bytes, j.vec_norms, &n_vec);
+                                 head_dim, j.bits, j.idx_bytes, j.vec_norms, j.packed_row_stride, &n_vec);
         if (rc) return rc;
         if (n_vec > max_vec) max_vec = n_vec;
     }

@@ -109,7 +109,8 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     auto issue_loads = [&](uint32_t tl) {
         const uint32_t v = tl * 32u + n;
         const bool ok = v < job.n_vec;
-        const uint8_t *src = job.idx_bytes + (size_t)(ok ? v : 0u) * (2 * NB) + hk * NB;
+        const uint32_t slot = ok ? tq_packed_slot(job, v) : 0u;
+        const uint8_t *src = job.idx_bytes + (size_t)slot * (2 * NB) + hk * NB;
         if constexpr (NW == 2) {
             tq_u2 t = {0u, 0u};
             if (ok) t = tq_gload8(src);
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
                 for (int i = 0; i < 4; ++i) raw[4 * q + i] = t[i];
             }
         }
-        norm_bits = ok ? tq_gload2(job.vec_norms + v) : (uint16_t)0;
+        norm_bits = ok ? tq_gload2(job.vec_norms + slot) : (uint16_t)0;
     };
     if (tile < n_tiles) issue_loads(tile);
 
@@ -262,7 +263,7 @@ int elem_bytes(int dtype) { return dtype == TQ_F32 ? 4 : (dtype == TQ_F16 || dty
 
 int check_job(const void *out, int dtype, long long rows, long long tokens, long long row_stride,
               long long token_stride, const void *table, int head_dim, int bits, const void *idx_bytes,
-              const void *vec_norms, long long *n_vec) {
+              const void *vec_norms, long long packed_row_stride, long long *n_vec) {
     if (bits < 1 || bits > 8) return TQ_ERR_BITS;
     if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
     const int eb = elem_bytes(dtype);
@@ -274,6 +275,7 @@ int check_job(const void *out, int dtype, long long rows, long long tokens, long
     if (!out || !table || !idx_bytes || !vec_norms) return TQ_ERR_NULL;
     if (token_stride < TQ_HEAD_DIM && tokens > 1) return TQ_ERR_SIZE;
     if (rows > 1 && row_stride < 0) return TQ_ERR_SIZE;
+    if (packed_row_stride != 0 && (packed_row_stride < tokens || packed_row_stride > (long long)0x7fffffff / rows)) return TQ_ERR_SIZE;
     if (((uintptr_t)out & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & 15u) || ((uintptr_t)vec_norms & 1u))
         return TQ_ERR_ALIGN;
     if (((token_stride * eb) & 15) || (rows > 1 && ((row_stride * eb) & 15))) return TQ_ERR_ALIGN;
@@ -282,12 +284,13 @@ int check_job(const void *out, int dtype, long long rows, long long tokens, long
 
 }  // namespace
 
-extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long rows, long long tokens,
+extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long packed_row_stride,
+                             long long rows, long long tokens,
                              const void *table_dev, int head_dim, int bits, void *out, int out_dtype,
                              long long row_stride, long long token_stride, void *stream) {
     long long n_vec = 0;
     const int rc = check_job(out, out_dtype, rows, tokens, row_stride, token_stride, table_dev, head_dim, bits,
-                             idx_bytes, vec_norms, &n_vec);
+                             idx_bytes, vec_norms, packed_row_stride, &n_vec);
     if (rc || n_vec == 0) return rc;
     TqDevJob job;
     job.states = static_cast<const uint8_t *>(out);
@@ -296,6 +299,7 @@ extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms
     job.table = static_cast<const uint8_t *>(table_dev);
     job.n_vec = (uint32_t)n_vec;
     job.tokens = (uint32_t)tokens;
+    job.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     job.row_stride = row_stride * elem_bytes(out_dtype);
     job.token_stride = token_stride * elem_bytes(out_dtype);
     return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), static_cast<hipStream_t>(stream));
@@ -314,7 +318,7 @@ extern "C" int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs
         if (j.dtype != jobs_host[0].dtype) return TQ_ERR_DTYPE;
         long long n_vec = 0;
         const int rc = check_job(j.states, j.dtype, j.rows, j.tokens, j.row_stride, j.token_stride, j.table_dev,
-                                 head_dim, j.bits, j.idx_bytes, j.vec_norms, &n_vec);
+                                 head_dim, j.bits, j.idx_bytes, j.vec_norms, j.packed_row_stride, &n_vec);
         if (rc) return rc;
         if (n_vec > max_vec) max_vec = n_vec;
     }

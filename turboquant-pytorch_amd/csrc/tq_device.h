@@ -25,6 +25,7 @@ struct TqDevJob {
     const uint8_t *table;
     uint32_t n_vec;          // rows * tokens  (< 2^31)
     uint32_t tokens;
+    uint32_t packed_row_stride;  // packed slots per row (>= tokens)
     long long row_stride;    // bytes
     long long token_stride;  // bytes
 };
@@ -39,6 +40,7 @@ __device__ __forceinline__ TqDevJob tq_load_job(const TqDevJob &single, const tq
     job.table = static_cast<const uint8_t *>(j.table_dev);
     job.n_vec = (uint32_t)(j.rows * j.tokens);
     job.tokens = (uint32_t)j.tokens;
+    job.packed_row_stride = (uint32_t)(j.packed_row_stride ? j.packed_row_stride : j.tokens);
     job.row_stride = j.row_stride * elem_bytes;
     job.token_stride = j.token_stride * elem_bytes;
     return job;
@@ -50,6 +52,13 @@ __device__ __forceinline__ long long tq_vec_offset(const TqDevJob &job, uint32_t
     const uint32_t row = v / job.tokens;
     const uint32_t tok = v - row * job.tokens;
     return (long long)row * job.row_stride + (long long)tok * job.token_stride;
+}
+
+// Packed slot (index into idx_bytes rows and vec_norms) of vector v.
+__device__ __forceinline__ uint32_t tq_packed_slot(const TqDevJob &job, uint32_t v) {
+    if (job.tokens >= job.n_vec) return v;  // one row
+    const uint32_t row = v / job.tokens;
+    return row * job.packed_row_stride + (v - row * job.tokens);
 }
 
 // Global-memory accessors (explicit address space: plain pointers read from a descriptor

@@ -1,0 +1,206 @@
+"""
+Streaming KV cache over the TurboQuant V3 codec.
+
+`V3Cache.update(key_states, value_states, layer_idx)` has the contract of the reference's
+generation-time cache (turboquant/generation_test_v2.py:48-165): new tokens join an uncompressed
+window of the most recent `residual_window` tokens, tokens pushed out of the window are
+compressed for good, and every call returns the full-length keys and values of the layer --
+de-quantised old tokens followed by the window -- in the dtype of the incoming states.
+
+What is different underneath:
+  * the reference keeps a Python list of compressed chunks per layer and de-quantises them one
+    by one on every step (O(steps) small launches, then a concatenation).  Here each layer owns
+    one preallocated packed store [B, H, capacity, G] (+ fp16 norms); tokens leaving the window are
+    appended in place (`packed_row_stride` of the C ABI), and a step is one compress launch per
+    tensor for the leaving tokens plus one decompress launch per tensor that writes the whole
+    history straight into the output buffer;
+  * codes depend on the vector alone, so the stored bytes are the same whatever the chunking.
+The class does not derive from transformers' DynamicCache; `hf_cache_class()` builds that
+subclass when transformers is importable.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from .compressors_v3 import TurboQuantV3
+
+
+class _LayerStore:
+    """Packed history and uncompressed window of one layer."""
+
+    def __init__(self, comp: TurboQuantV3, B: int, H: int, D: int, dtype: torch.dtype, device: torch.device,
+                 capacity: int, window: int):
+        self.comp = comp
+        self.B, self.H, self.D = B, H, D
+        self.dtype, self.device = dtype, device
+        self.capacity = 0
+        self.k_idx = self.k_nrm = self.v_idx = self.v_nrm = None
+        self.n_compressed = 0
+        self.window = window
+        # the window store holds the uncompressed tail between calls
+        self.k_win = torch.empty((B, H, max(window, 1), D), dtype=dtype, device=device)
+        self.v_win = torch.empty_like(self.k_win)
+        self.n_recent = 0
+        self.total_seq = 0
+        self.reserve(capacity)
+
+    @staticmethod
+    def _width(D: int, bits: int) -> int:
+        ipb = 8 // bits
+        return -(-D // ipb)
+
+    def reserve(self, tokens: int) -> None:
+        """Make room for `tokens` compressed tokens per (batch, head) row (amortised doubling)."""
+        if tokens <= self.capacity:
+            return
+        cap = max(tokens, 2 * self.capacity, 256)
+        cap = -(-cap // 64) * 64
+        new = []
+        for old, width in ((self.k_idx, self._width(self.D, self.comp.key_bits)), (self.k_nrm, None),
+                           (self.v_idx, self._width(self.D, self.comp.value_bits)), (self.v_nrm, None)):
+            if width is None:
+                buf = torch.empty((self.B, self.H, cap), dtype=torch.float16, device=self.device)
+            else:
+                buf = torch.empty((self.B, self.H, cap, width), dtype=torch.uint8, device=self.device)
+            if old is not None and self.n_compressed:
+                buf[:, :, :self.n_compressed].copy_(old[:, :, :self.n_compressed])
+            new.append(buf)
+        self.k_idx, self.k_nrm, self.v_idx, self.v_nrm = new
+        self.capacity = cap
+
+    def append_compressed(self, keys: torch.Tensor, values: torch.Tensor) -> None:
+        """Compress [B,H,n,D] views of keys / values into packed slots [n_compressed, n_compressed + n)."""
+        n = keys.shape[2]
+        if n == 0:
+            return
+        self.reserve(self.n_compressed + n)
+        lo, hi = self.n_compressed, self.n_compressed + n
+        kc, vc = self.comp.key_compressor, self.comp.val_compressor
+        kc.compress_into(keys, self.k_idx[:, :, lo:hi], self.k_nrm[:, :, lo:hi])
+        vc.compress_into(values, self.v_idx[:, :, lo:hi], self.v_nrm[:, :, lo:hi])
+        self.n_compressed = hi
+
+
+class V3Cache:
+    """Streaming compressed KV cache; `update` follows generation_test_v2.py:80-153."""
+
+    def __init__(self, key_bits: int = 4, value_bits: int = 2, residual_window: int = 128,
+                 protected_layers: int = 0, n_layers: int = 36, *, capacity: int = 0):
+        self.key_bits = key_bits
+        self.value_bits = value_bits
+        self.residual_window = residual_window
+        self.protected_layers = protected_layers
+        self.n_layers = n_layers
+        self.capacity = capacity          # expected compressed tokens per sequence (0: grow on demand)
+        self._compressors: Dict[int, TurboQuantV3] = {}
+        self._stores: Dict[int, _LayerStore] = {}
+
+    def _get_compressor(self, layer_idx: int, head_dim: int, device) -> TurboQuantV3:
+        # generation_test_v2.py:65-78: per-layer codec, residual_window=0 (the cache owns the window)
+        if layer_idx not in self._compressors:
+            self._compressors[layer_idx] = TurboQuantV3(
+                head_dim=head_dim,
+                key_bits=self.key_bits,
+                value_bits=self.value_bits,
+                residual_window=0,
+                layer_idx=layer_idx,
+                n_layers=self.n_layers,
+                protected_layers=self.protected_layers,
+                seed=42,
+                device=str(device),
+            )
+        return self._compressors[layer_idx]
+
+    @torch.no_grad()
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
+               cache_kwargs: Optional[dict] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        B, H, S_new, D = key_states.shape
+        device = key_states.device
+        comp = self._get_compressor(layer_idx, D, device)
+        st = self._stores.get(layer_idx)
+        if st is None:
+            st = _LayerStore(comp, B, H, D, key_states.dtype, device, self.capacity, self.residual_window)
+            self._stores[layer_idx] = st
+        elif (st.B, st.H, st.D) != (B, H, D):
+            raise ValueError(f"layer {layer_idx}: states {tuple(key_states.shape)} do not match the cached "
+                             f"batch/head/dim {(st.B, st.H, st.D)}")
+        st.total_seq += S_new
+
+        # the uncompressed tokens are (window ++ new); everything beyond the last `rw` of them leaves
+        rw = self.residual_window
+        recent = st.n_recent + S_new
+        overflow = recent if rw == 0 else max(recent - rw, 0)
+        from_window = min(overflow, st.n_recent)
+        from_new = overflow - from_window
+        st.append_compressed(st.k_win[:, :, :from_window], st.v_win[:, :, :from_window])
+        st.append_compressed(key_states[:, :, :from_new], value_states[:, :, :from_new])
+
+        keep_old = st.n_recent - from_window
+        keep_new = S_new - from_new
+        n_c = st.n_compressed
+        total = n_c + keep_old + keep_new
+        full_k = torch.empty((B, H, total, D), dtype=key_states.dtype, device=device)
+        full_v = torch.empty((B, H, total, D), dtype=value_states.dtype, device=device)
+        if n_c:
+            comp.key_compressor.decompress_packed(st.k_idx[:, :, :n_c], st.k_nrm[:, :, :n_c], full_k[:, :, :n_c])
+            comp.val_compressor.decompress_packed(st.v_idx[:, :, :n_c], st.v_nrm[:, :, :n_c], full_v[:, :, :n_c])
+        if keep_old:
+            full_k[:, :, n_c:n_c + keep_old].copy_(st.k_win[:, :, from_window:st.n_recent])
+            full_v[:, :, n_c:n_c + keep_old].copy_(st.v_win[:, :, from_window:st.n_recent])
+        if keep_new:
+            full_k[:, :, n_c + keep_old:].copy_(key_states[:, :, from_new:])
+            full_v[:, :, n_c + keep_old:].copy_(value_states[:, :, from_new:])
+        # the tail of the output is the next window
+        st.n_recent = keep_old + keep_new
+        if st.n_recent:
+            st.k_win[:, :, :st.n_recent].copy_(full_k[:, :, n_c:])
+            st.v_win[:, :, :st.n_recent].copy_(full_v[:, :, n_c:])
+        return full_k, full_v
+
+    def get_seq_length(self, layer_idx: int = 0) -> int:
+        st = self._stores.get(layer_idx)
+        return st.total_seq if st is not None else 0
+
+    def get_compression_info(self) -> str:
+        if not self._stores:
+            return "no compression"
+        st = self._stores.get(0)
+        comp = st.n_compressed if st is not None else 0
+        total = st.total_seq if st is not None else 0
+        return f"{comp} compressed, {total - comp} fp16, {total} total"
+
+    def stored_bytes(self) -> int:
+        """Bytes held for the tokens seen so far (packed codes, norms, window), over all layers."""
+        n = 0
+        for st in self._stores.values():
+            rows = st.B * st.H
+            n += rows * st.n_compressed * (st.k_idx.shape[-1] + st.v_idx.shape[-1] + 4)
+            n += 2 * rows * st.n_recent * st.D * st.k_win.element_size()
+        return n
+
+
+def hf_cache_class():
+    """A `V3Cache` that also derives from transformers.DynamicCache, so that it can be passed as
+    `past_key_values` to `model.generate` the way generation_test_v2.py:178-201 does."""
+    from transformers import DynamicCache
+
+    class HFV3Cache(V3Cache, DynamicCache):
+        def __init__(self, *args, **kwargs):
+            DynamicCache.__init__(self)
+            V3Cache.__init__(self, *args, **kwargs)
+
+        def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
+            out = V3Cache.update(self, key_states, value_states, layer_idx, cache_kwargs)
+            layers = getattr(self, "layers", None)
+            if layers is not None:
+                from transformers.cache_utils import DynamicLayer
+                while len(layers) <= layer_idx:
+                    layers.append(DynamicLayer())
+            return out
+
+        def get_seq_length(self, layer_idx=0):
+            return V3Cache.get_seq_length(self, layer_idx)
+
+    return HFV3Cache
