@@ -10,7 +10,8 @@ Default workload (the one BASELINE.json quotes its target on): Llama-3-8B-shaped
 32 layers x [1, 8, 32768, 128] bf16, K4/V2, protected_layers=4 with the reference's semantics
 (the first and last 4 layers use 8-bit keys AND values, compressors_v3.py:158-160), no residual
 window.  `--workload llama3-8b-32k-k4v2` runs the same shape with every layer at K4/V2;
-`--workload qwen2.5-3b-8k` is BASELINE config 2 (fp16).
+`--workload qwen2.5-3b-8k` is BASELINE config 2 (fp16); `--workload decode-64x16k` is the streaming
+decode case (config 5): a step is one generated token through `V3Cache.update` on every layer.
 
 Prints ONE JSON line (see README / DESIGN.md for the fields).
 """
@@ -33,6 +34,10 @@ WORKLOADS = {
     "llama3-8b-32k": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2, protected=4),
     "llama3-8b-32k-k4v2": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2, protected=0),
     "qwen2.5-3b-8k": dict(layers=36, batch=1, heads=2, tokens=8192, dtype="f16", key_bits=4, value_bits=2, protected=0),
+    # streaming decode (BASELINE config 5): 64 sequences with 16384 compressed + 128 window tokens; a step is
+    # one new token through V3Cache.update on all 32 layers (compress what leaves the window, de-quantise all)
+    "decode-64x16k": dict(layers=32, batch=64, heads=8, tokens=16384, dtype="bf16", key_bits=4, value_bits=2,
+                          protected=0, window=128, decode=True),
 }
 
 
@@ -94,6 +99,67 @@ def cpu_baseline(pkg, widths, budget_s=20.0):
     }
 
 
+def run_decode(args, torch, pkg, w, dev):
+    """One decode token per step through the streaming cache: per layer, the token leaving the window
+    is compressed and appended, the whole history is de-quantised into fresh K / V tensors."""
+    L, B, H, S0, rw = w["layers"], w["batch"], w["heads"], w["tokens"], w["window"]
+    dtype = torch.bfloat16
+    cache = pkg.V3Cache(key_bits=w["key_bits"], value_bits=w["value_bits"], residual_window=rw,
+                        protected_layers=w["protected"], n_layers=L, capacity=S0 + args.steps + args.warmup + 8)
+    # prefill: the same synthetic K / V tensors for every layer (each layer has its own rotation)
+    k0 = synth_kv(torch, (B, H, S0 + rw, 128), seed=5_000_000, dtype=dtype, device=dev)
+    v0 = synth_kv(torch, (B, H, S0 + rw, 128), seed=5_000_001, dtype=dtype, device=dev)
+    for l in range(L):
+        cache.update(k0, v0, l)
+    del k0, v0
+    torch.cuda.synchronize()
+    kn = synth_kv(torch, (B, H, 1, 128), seed=5_000_002, dtype=dtype, device=dev)
+    vn = synth_kv(torch, (B, H, 1, 128), seed=5_000_003, dtype=dtype, device=dev)
+
+    def step():
+        out = None
+        for l in range(L):
+            out = cache.update(kn, vn, l)
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fk, fv = step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    total = cache.get_seq_length(0)
+    n_c = total - rw
+    if fk.shape != (B, H, total, 128) or not torch.equal(fk[:, :, -1:], kn):
+        sys.exit("bench.py: decode step returned the wrong tensors")
+    # per step and layer: K and V de-quantise ~n_c tokens per row, compress one, copy the window
+    rows = B * H
+    deq_vec = 2 * L * rows * (n_c - (args.steps - 1) / 2.0)
+    cmp_vec = 2 * L * rows
+    step_bytes = L * rows * ((n_c - (args.steps - 1) / 2.0) * (algorithmic_bytes(w["key_bits"], 2, "d") + algorithmic_bytes(w["value_bits"], 2, "d"))
+                             + (algorithmic_bytes(w["key_bits"], 2, "c") + algorithmic_bytes(w["value_bits"], 2, "c"))
+                             + 2 * rw * 512)
+    sec = wall / args.steps
+    result = {
+        "metric": "KV vectors/sec (compress+decompress)", "value": (deq_vec + cmp_vec) / sec, "unit": "vectors/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "layers": L, "batch": B, "kv_heads": H, "compressed_tokens": n_c,
+                   "window_tokens": rw, "head_dim": 128, "key_bits": w["key_bits"], "value_bits": w["value_bits"],
+                   "new_tokens_per_step": 1},
+        "decode_steps_per_s": 1.0 / sec,
+        "step_algorithmic_GB": step_bytes / 1e9, "step_GBps": step_bytes / sec / 1e9,
+        "roofline": {"bound": "hbm", "kernel": "whole step (decompress dominates)", "achieved": step_bytes / sec / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": step_bytes / sec / 1e9 / HBM_PEAK_GBS, "traffic": None},
+        "stored_GB": cache.stored_bytes() / 1e9,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(pkg, {w["key_bits"]: 0.5, w["value_bits"]: 0.5}, args.cpu_seconds)
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -116,6 +182,8 @@ def main():
     torch.cuda.set_device(dev)
 
     w = WORKLOADS[args.workload]
+    if w.get("decode"):
+        return run_decode(args, torch, pkg, w, dev)
     L, B, H, S = w["layers"], w["batch"], w["heads"], w["tokens"]
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16}[w["dtype"]]
     n_vec = B * H * S
