@@ -38,6 +38,10 @@ WORKLOADS = {
     # one new token through V3Cache.update on all 32 layers (compress what leaves the window, de-quantise all)
     "decode-64x16k": dict(layers=32, batch=64, heads=8, tokens=16384, dtype="bf16", key_bits=4, value_bits=2,
                           protected=0, window=128, decode=True),
+    # the same cache read through V3Cache.append + V3Cache.attend: attention of one query token per sequence
+    # (32 query heads over 8 kv heads) computed from the packed store, nothing de-quantised to memory
+    "decode-attend-64x16k": dict(layers=32, batch=64, heads=8, tokens=16384, dtype="bf16", key_bits=4, value_bits=2,
+                                 protected=0, window=128, decode=True, attend=True, q_heads=32),
 }
 
 
@@ -116,10 +120,17 @@ def run_decode(args, torch, pkg, w, dev):
     kn = synth_kv(torch, (B, H, 1, 128), seed=5_000_002, dtype=dtype, device=dev)
     vn = synth_kv(torch, (B, H, 1, 128), seed=5_000_003, dtype=dtype, device=dev)
 
+    attend = bool(w.get("attend"))
+    qn = synth_kv(torch, (B, w.get("q_heads", H), 1, 128), seed=5_000_004, dtype=dtype, device=dev) if attend else None
+
     def step():
         out = None
         for l in range(L):
-            out = cache.update(kn, vn, l)
+            if attend:
+                cache.append(kn, vn, l)
+                out = cache.attend(qn, l)
+            else:
+                out = cache.update(kn, vn, l)
         return out
 
     for _ in range(args.warmup):
@@ -127,12 +138,15 @@ def run_decode(args, torch, pkg, w, dev):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        fk, fv = step()
+        res = step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     total = cache.get_seq_length(0)
     n_c = total - rw
-    if fk.shape != (B, H, total, 128) or not torch.equal(fk[:, :, -1:], kn):
+    if attend:
+        if res.shape != qn.shape or not bool(torch.isfinite(res.float()).all()):
+            sys.exit("bench.py: attend returned the wrong tensor")
+    elif res[0].shape != (B, H, total, 128) or not torch.equal(res[0][:, :, -1:], kn):
         sys.exit("bench.py: decode step returned the wrong tensors")
     # per step and layer: K and V de-quantise ~n_c tokens per row, compress one, copy the window
     rows = B * H
@@ -142,6 +156,12 @@ def run_decode(args, torch, pkg, w, dev):
                              + (algorithmic_bytes(w["key_bits"], 2, "c") + algorithmic_bytes(w["value_bits"], 2, "c"))
                              + 2 * rw * 512)
     sec = wall / args.steps
+    if attend:
+        # packed codes and norms are read once; nothing de-quantised is written.  (Scores and probabilities,
+        # 4 bytes per query head and token, cross HBM between the three kernels; they are not algorithmic.)
+        step_bytes = L * rows * ((n_c - (args.steps - 1) / 2.0) * (packed_bytes(w["key_bits"]) + packed_bytes(w["value_bits"]) + 4)
+                                 + (algorithmic_bytes(w["key_bits"], 2, "c") + algorithmic_bytes(w["value_bits"], 2, "c"))
+                                 + 2 * rw * 256)
     result = {
         "metric": "KV vectors/sec (compress+decompress)", "value": (deq_vec + cmp_vec) / sec, "unit": "vectors/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
@@ -151,7 +171,7 @@ def run_decode(args, torch, pkg, w, dev):
                    "new_tokens_per_step": 1},
         "decode_steps_per_s": 1.0 / sec,
         "step_algorithmic_GB": step_bytes / 1e9, "step_GBps": step_bytes / sec / 1e9,
-        "roofline": {"bound": "hbm", "kernel": "whole step (decompress dominates)", "achieved": step_bytes / sec / 1e9,
+        "roofline": {"bound": "hbm", "kernel": "whole step (scores + weighted values from packed codes)" if attend else "whole step (decompress dominates)", "achieved": step_bytes / sec / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": step_bytes / sec / 1e9 / HBM_PEAK_GBS, "traffic": None},
         "stored_GB": cache.stored_bytes() / 1e9,
     }

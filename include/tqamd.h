@@ -156,6 +156,31 @@ int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_j
 int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
                           int head_dim, void *stream);
 
+/*
+ * Decode-time attention on the packed cache, without de-quantising it.  Replaces, for single-token
+ * decode steps, "de-quantise every stored chunk (generation_test_v2.py:131-135, compressors_v3.py:84-105)
+ * and let the model multiply by the result" (score definition: validate_v3.py:87).
+ * `rows` = batch * kv_heads packed rows of `tokens` tokens (slot of token t of row r:
+ * r * packed_row_stride + t; 0 = tokens); query head (r * group + g) belongs to row r.
+ *
+ * tq_scores:   scores[(r*group + g) * scores_stride + t] = norm_t * sum_j q_rot[r][g][j] * centroid[code(t, j)]
+ *              = q . k_hat_t  when  q_rot = Pi q  (times any softmax scale folded into q_rot).
+ *              q_rot: device, float32 [rows, group, head_dim] contiguous; group <= 32.
+ * tq_weighted_values:
+ *              out_rot[r][g][j] = sum_t weights[(r*group + g) * weights_stride + t] * norm_t * centroid[code(t, j)],
+ *              so that  sum_t w_t v_hat_t = out_rot[r][g] @ Pi.  group <= 8 per call.  The token range is
+ *              cut into `splits` pieces summed in a fixed order; `partial` is caller-provided scratch of
+ *              rows * splits * group * head_dim floats.  tq_weighted_values_splits suggests a split count.
+ */
+int tq_scores(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long packed_row_stride,
+              long long rows, long long tokens, const void *table_dev, int head_dim, int bits,
+              const float *q_rot, int group, float *scores, long long scores_stride, void *stream);
+int tq_weighted_values_splits(long long rows, long long tokens);
+int tq_weighted_values(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long packed_row_stride,
+                       long long rows, long long tokens, const void *table_dev, int head_dim, int bits,
+                       const float *weights, long long weights_stride, int group,
+                       float *partial, int splits, float *out_rot, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

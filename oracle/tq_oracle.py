@@ -15,6 +15,11 @@ upstream algorithm live here and check each other:
 Only tests/, the repository's smoke check and the benchmark's cpu_baseline leg
 may import this module; the shipped package never does.
 
+  * `attention_decode` -- one-query attention over explicit K / V in float64: the score definition of
+    turboquant/validate_v3.py:87 followed by the textbook softmax-weighted sum the model applies to the
+    tensors generation_test_v2.py:131-153 returns.  Pinned in tests/test_oracle.py against
+    torch.nn.functional.scaled_dot_product_attention and against a brute-force loop.
+
 What pins it: tests/golden/*.npz hold outputs of the real reference on seeded
 inputs (tests/golden/make_fixtures.py wrote them); tests/test_oracle.py checks
 both restatements against those, against each other, against exhaustive
@@ -278,3 +283,21 @@ def fp16_ulp_distance(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
         u = u.astype(np.int32)
         return np.where(u & 0x8000, -(u & 0x7FFF), u & 0x7FFF)
     return np.abs(key(a_bits) - key(b_bits))
+
+
+# --------------------------------------------------------------------------
+# one-query attention (checker for the packed-cache attention kernels)
+# --------------------------------------------------------------------------
+def attention_decode(q: np.ndarray, K: np.ndarray, V: np.ndarray, scale: float):
+    """q [B,Hq,D], K and V [B,H,S,D] (query head j reads kv head j // (Hq/H)) ->
+    (scores [B,Hq,S] = scale * q.k as in validate_v3.py:87, out [B,Hq,D] = softmax(scores) @ V), float64."""
+    B, Hq, D = q.shape
+    H = K.shape[1]
+    G = Hq // H
+    q4 = q.astype(np.float64).reshape(B, H, G, D)
+    scores = np.einsum("bhgd,bhsd->bhgs", q4, K.astype(np.float64)) * scale
+    m = scores.max(-1, keepdims=True) if scores.shape[-1] else scores
+    p = np.exp(scores - m)
+    p /= p.sum(-1, keepdims=True)
+    out = np.einsum("bhgs,bhsd->bhgd", p, V.astype(np.float64))
+    return scores.reshape(B, Hq, -1), out.reshape(B, Hq, D)

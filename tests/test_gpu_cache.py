@@ -149,3 +149,119 @@ def test_hf_dynamic_cache_subclass(pkg):
         assert k.shape == (1, 2, 12, 128)
     assert cache.get_seq_length() == 12 and cache.get_seq_length(1) == 12
     assert cache.get_compression_info() == "8 compressed, 4 fp16, 12 total"
+
+
+# ---------------------------------------------------------------------------------------------
+# attention straight from the packed store
+# ---------------------------------------------------------------------------------------------
+def _oracle_decode(oracle, comp, idx, nrm, shape):
+    orc = oracle.COracle(comp.Pi.cpu().numpy(), comp.centroids.cpu().numpy(), comp.bits, True)
+    flat = orc.decompress(idx.contiguous().cpu().numpy().reshape(-1, idx.shape[-1]), bits16(nrm.contiguous()).reshape(-1))
+    return flat.reshape(shape)
+
+
+@pytest.mark.parametrize("bits,group,S", [(4, 4, 1000), (2, 8, 333), (8, 1, 64), (3, 2, 31), (1, 16, 257), (6, 32, 96)])
+def test_packed_scores_against_oracle(pkg, oracle, bits, group, S):
+    """scale * q . k_hat from packed keys (query rotated once, codes never expanded to vectors) equals the
+    float64 scores over the oracle's de-quantised keys; tolerance: the fp16 rounding of the centroid
+    table the decode kernels share (2^-11 relative per coordinate), i.e. 1e-3 of scale*|q|*|k|."""
+    B, H, D = 2, 3, 128
+    comp = pkg.MSECompressor(D, bits, seed=77 + bits, device=DEV)
+    keys = outlier_kv((B, H, S, D), seed=bits * 10 + group, dtype=torch.bfloat16).to(DEV)
+    store = torch.zeros(B, H, S + 40, D // (8 // bits), dtype=torch.uint8, device=DEV)
+    norms = torch.zeros(B, H, S + 40, dtype=torch.float16, device=DEV)
+    comp.compress_into(keys, store[:, :, 7:7 + S], norms[:, :, 7:7 + S])
+    g = torch.Generator(device="cpu")
+    g.manual_seed(group)
+    q = (torch.randn(B, H * group, 1, D, generator=g) * torch.exp(torch.randn(B, H * group, 1, 1, generator=g))).to(DEV)
+    scale = D ** -0.5
+    out = torch.full((B, H * group, S + 5), 123.0, dtype=torch.float32, device=DEV)
+    got = comp.packed_scores(store[:, :, 7:7 + S], norms[:, :, 7:7 + S], q, scale, out=out[:, :, :S])
+    assert got.data_ptr() == out.data_ptr() and bool((out[:, :, S:] == 123.0).all())
+    k_hat = _oracle_decode(oracle, comp, store[:, :, 7:7 + S], norms[:, :, 7:7 + S], (B, H, S, D))
+    ref, _ = oracle.attention_decode(q.squeeze(2).cpu().numpy(), k_hat, k_hat, scale)
+    bound = scale * np.linalg.norm(q.squeeze(2).cpu().numpy().astype(np.float64), axis=-1)[:, :, None] \
+        * np.repeat(np.linalg.norm(k_hat.astype(np.float64), axis=-1), group, axis=1)
+    err = np.abs(got.cpu().numpy() - ref) / np.maximum(bound, 1e-30)
+    print(f"[scores] b{bits} G{group} S{S}: max error {err.max():.2e} of scale*|q|*|k|")
+    assert err.max() < 1e-3
+    # and the definition the reference uses: scores over the product's own de-quantised keys
+    deq = torch.empty(B, H, S, D, dtype=torch.float32, device=DEV)
+    comp.decompress_packed(store[:, :, 7:7 + S], norms[:, :, 7:7 + S], deq)
+    same = pkg.attention_scores(q, deq.repeat_interleave(group, dim=1)) * scale
+    assert float((got - same).abs().max()) < 1e-3 * float(bound.max())
+    dense = comp.packed_scores(store[:, :, 7:7 + S].contiguous(), norms[:, :, 7:7 + S].contiguous(), q.squeeze(2), scale)
+    assert torch.equal(dense, got)
+
+
+@pytest.mark.parametrize("bits,group,S", [(2, 4, 1000), (4, 8, 333), (8, 1, 64), (3, 2, 31), (1, 16, 257)])
+def test_packed_weighted_values_against_oracle(pkg, oracle, bits, group, S):
+    B, H, D = 2, 3, 128
+    comp = pkg.MSECompressor(D, bits, seed=177 + bits, device=DEV)
+    vals = outlier_kv((B, H, S, D), seed=bits * 10 + group + 1, dtype=torch.float16).to(DEV)
+    store = torch.zeros(B, H, S + 9, D // (8 // bits), dtype=torch.uint8, device=DEV)
+    norms = torch.zeros(B, H, S + 9, dtype=torch.float16, device=DEV)
+    comp.compress_into(vals, store[:, :, 2:2 + S], norms[:, :, 2:2 + S])
+    g = torch.Generator(device="cpu")
+    g.manual_seed(S)
+    w_full = torch.softmax(3 * torch.randn(B, H * group, S + 16, generator=g), dim=-1).to(DEV)
+    w = w_full[:, :, :S]                                         # a strided slice, as the cache passes it
+    got = comp.packed_weighted_values(store[:, :, 2:2 + S], norms[:, :, 2:2 + S], w)
+    v_hat = _oracle_decode(oracle, comp, store[:, :, 2:2 + S], norms[:, :, 2:2 + S], (B, H, S, D)).astype(np.float64)
+    ref = np.einsum("bhgs,bhsd->bhgd", w.cpu().numpy().astype(np.float64).reshape(B, H, group, S), v_hat).reshape(B, H * group, D)
+    err = np.linalg.norm(got.cpu().numpy() - ref) / np.linalg.norm(ref)
+    print(f"[weighted values] b{bits} G{group} S{S}: relative L2 error {err:.2e}")
+    assert got.shape == (B, H * group, D) and err < 1e-3
+    again = comp.packed_weighted_values(store[:, :, 2:2 + S], norms[:, :, 2:2 + S], w)
+    assert torch.equal(again, got)                               # fixed summation order
+
+
+@pytest.mark.parametrize("rw,dtype", [(128, torch.bfloat16), (0, torch.float16), (16, torch.bfloat16)])
+def test_v3cache_attend_equals_attention_over_the_cache(pkg, oracle, rw, dtype):
+    """append() leaves the cache in the state update() leaves it in, and attend() equals one-query
+    attention over (oracle-decoded packed tokens ++ window) in float64; it also agrees with attention
+    over the bf16 / fp16 tensors update() hands to the model within their rounding."""
+    B, H, G, D, L = 2, 2, 4, 128, 2
+    a = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=rw, n_layers=L)
+    b = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=rw, n_layers=L)
+    steps = [300, 1, 1, 5, 1] + [1] * 20
+    total = sum(steps)
+    keys = [outlier_kv((B, H, total, D), seed=600 + l, dtype=dtype).to(DEV) for l in range(L)]
+    vals = [outlier_kv((B, H, total, D), seed=700 + l, dtype=dtype).to(DEV) for l in range(L)]
+    g = torch.Generator(device="cpu")
+    g.manual_seed(9)
+    seen = 0
+    for i, n_new in enumerate(steps):
+        for l in range(L):
+            fk, fv = a.update(keys[l][:, :, seen:seen + n_new], vals[l][:, :, seen:seen + n_new], l)
+            b.append(keys[l][:, :, seen:seen + n_new], vals[l][:, :, seen:seen + n_new], l)
+            sa, sb = a._stores[l], b._stores[l]
+            assert (sa.n_compressed, sa.n_recent, sa.total_seq) == (sb.n_compressed, sb.n_recent, sb.total_seq)
+            if i in (0, 3, len(steps) - 1):
+                n_c = sb.n_compressed
+                assert torch.equal(sa.k_idx[:, :, :n_c], sb.k_idx[:, :, :n_c]) and torch.equal(sa.v_nrm[:, :, :n_c], sb.v_nrm[:, :, :n_c])
+                assert all(torch.equal(x, y) for x, y in zip(sa.window(), sb.window()))
+                q = (4 * torch.randn(B, H * G, 1, D, generator=g)).to(dtype).to(DEV)
+                out = b.attend(q, l)
+                assert out.shape == (B, H * G, 1, D) and out.dtype == dtype
+                tq = b._get_compressor(l, D, DEV)
+                kw, vw = sb.window()
+                parts_k, parts_v = [], []
+                if n_c:
+                    parts_k.append(_oracle_decode(oracle, tq.key_compressor, sb.k_idx[:, :, :n_c], sb.k_nrm[:, :, :n_c], (B, H, n_c, D)))
+                    parts_v.append(_oracle_decode(oracle, tq.val_compressor, sb.v_idx[:, :, :n_c], sb.v_nrm[:, :, :n_c], (B, H, n_c, D)))
+                parts_k.append(kw.float().cpu().numpy())
+                parts_v.append(vw.float().cpu().numpy())
+                _, ref = oracle.attention_decode(q.squeeze(2).float().cpu().numpy(), np.concatenate(parts_k, 2),
+                                                 np.concatenate(parts_v, 2), D ** -0.5)
+                got = out.squeeze(2).float().cpu().numpy()
+                err = np.linalg.norm(got - ref) / np.linalg.norm(ref)
+                # what the model would compute from update()'s tensors
+                model = torch.nn.functional.scaled_dot_product_attention(
+                    q.float(), fk.float().repeat_interleave(G, dim=1), fv.float().repeat_interleave(G, dim=1)).squeeze(2)
+                err_model = float((out.squeeze(2).float() - model).norm() / model.norm())
+                print(f"[attend] rw={rw} step {i} layer {l}: vs oracle {err:.2e}, vs attention over update() tensors {err_model:.2e}")
+                assert err < 6e-3 and err_model < 2e-2           # output rounded to bf16 / fp16: 2^-9 / 2^-11
+        seen += n_new
+    with pytest.raises(ValueError):
+        b.attend(torch.zeros(B, H * G, 2, D, device=DEV), 0)

@@ -229,3 +229,25 @@ def test_decompress_inverts_rotation(golden, oracle):
         assert np.abs(rec - ref).max() < 2e-6
         back = (rec.astype(np.float64) / 3.0) @ Pi.astype(np.float64).T
         assert np.abs(back - cent[codes]).max() < 2e-6
+
+
+def test_attention_decode_oracle_is_textbook_attention(oracle):
+    """The float64 checker equals torch's scaled_dot_product_attention (grouped heads expanded) and a
+    brute-force loop over heads and tokens."""
+    rng = np.random.default_rng(5)
+    B, H, G, S, D = 2, 3, 4, 37, 16
+    q = rng.standard_normal((B, H * G, D)).astype(np.float32)
+    K = rng.standard_normal((B, H, S, D)).astype(np.float32)
+    V = rng.standard_normal((B, H, S, D)).astype(np.float32)
+    scale = 0.3
+    scores, out = oracle.attention_decode(q, K, V, scale)
+    tq, tK, tV = (torch.from_numpy(a).double() for a in (q, K, V))
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        tq.unsqueeze(2), tK.repeat_interleave(G, dim=1), tV.repeat_interleave(G, dim=1), scale=scale).squeeze(2)
+    assert np.abs(out - ref.numpy()).max() < 1e-12
+    for b, hq in ((0, 0), (1, 5), (1, 11)):
+        h = hq // G
+        s = np.array([scale * float(np.dot(q[b, hq].astype(np.float64), K[b, h, t].astype(np.float64))) for t in range(S)])
+        assert np.abs(scores[b, hq] - s).max() < 1e-12
+        p = np.exp(s - s.max()); p /= p.sum()
+        assert np.abs(out[b, hq] - (p[:, None] * V[b, h].astype(np.float64)).sum(0)).max() < 1e-12

@@ -20,7 +20,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(CSRC, "libtqamd.so")
-SOURCES = ("tq_host.cpp", "tq_compress.hip", "tq_decompress.hip")
+SOURCES = ("tq_host.cpp", "tq_compress.hip", "tq_decompress.hip", "tq_attend.hip")
 HEADERS = ("tq_table.h", "tq_device.h", os.path.join("..", "..", "include", "tqamd.h"))
 GPU_ARCH = "gfx950"
 
@@ -87,6 +87,7 @@ EXPORTS = (
     "tq_abi_version", "tq_status_string", "tq_device_count", "tq_bytes_per_vector",
     "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_quantize_host",
     "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched",
+    "tq_scores", "tq_weighted_values", "tq_weighted_values_splits",
 )
 
 _lib = None
@@ -116,6 +117,9 @@ def lib() -> ctypes.CDLL:
     L.tq_compress.argtypes = [vp, ci, ll, ll, ll, ll, vp, ci, ci, vp, vp, ll, vp]
     L.tq_decompress.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, ll, ll, vp]
     L.tq_compress_batched.argtypes = [vp, vp, ci, ci, vp]
+    L.tq_scores.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, vp, ll, vp]
+    L.tq_weighted_values_splits.argtypes = [ll, ll]
+    L.tq_weighted_values.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ll, ci, vp, ci, vp, vp]
     L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp]
     for name in EXPORTS:
         if name not in ("tq_status_string", "tq_table_bytes"):
@@ -341,6 +345,82 @@ def _(idx_bytes, vec_norms, table, bits, head_dim, out_dtype):
 def decompress_into_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
                        out: torch.Tensor) -> None:
     decompress_into(idx_bytes, vec_norms, table, bits, out)
+
+
+def _packed_rows(idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, int, int, int]:
+    """(idx_bytes, vec_norms, packed_row_stride, rows, tokens) of a [B,H,S,G] / [B,H,S] packed pair for
+    the row-wise entry points (copies only if the pair is not a slice of one per-row store)."""
+    prs = packed_row_stride(idx_bytes, vec_norms)
+    if prs is None:
+        idx_bytes, vec_norms, prs = idx_bytes.contiguous(), vec_norms.contiguous(), 0
+    B, H, S, _ = idx_bytes.shape
+    return idx_bytes, vec_norms, prs, B * H, S
+
+
+@torch.library.custom_op("tqamd::scores_into", mutates_args=("scores",), device_types="cuda")
+def scores_into_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
+                   q_rot: torch.Tensor, scores: torch.Tensor) -> None:
+    """scores[b, h*G + g, t] = q_rot[b, h*G + g] . centroids[codes(b, h, t)] * norm(b, h, t), written into
+    `scores` ([B, Hq, S] float32 view whose last dimension is dense and whose heads are equally spaced)."""
+    _require_gpu(idx_bytes, "idx_bytes")
+    idx_bytes, vec_norms, prs, rows, tokens = _packed_rows(idx_bytes, vec_norms)
+    B, Hq, D = q_rot.shape
+    group = Hq // idx_bytes.shape[1]
+    if scores.dtype != torch.float32 or tuple(scores.shape) != (B, Hq, tokens) or (tokens > 1 and scores.stride(2) != 1) \
+            or (Hq > 1 and B > 1 and scores.stride(0) != Hq * scores.stride(1)):
+        raise TqError("scores must be a float32 [B, Hq, S] view with a dense last dimension and evenly spaced heads")
+    q_rot = q_rot.to(torch.float32).contiguous()
+    stride = scores.stride(1) if Hq > 1 else (scores.stride(0) if B > 1 else max(tokens, 1))
+    with torch.cuda.device(idx_bytes.device):
+        rc = lib().tq_scores(idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, rows, tokens, table.data_ptr(), D, bits,
+                             q_rot.data_ptr(), group, scores.data_ptr(), stride, _stream_handle(idx_bytes.device))
+    check(rc, "tq_scores")
+
+
+@torch.library.custom_op("tqamd::weighted_values", mutates_args=(), device_types="cuda")
+def weighted_values_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
+                       weights: torch.Tensor, head_dim: int) -> torch.Tensor:
+    """out[b, h*G + g] = sum_t weights[b, h*G + g, t] * norm(b, h, t) * centroids[codes(b, h, t)]  (rotated space)."""
+    _require_gpu(idx_bytes, "idx_bytes")
+    idx_bytes, vec_norms, prs, rows, tokens = _packed_rows(idx_bytes, vec_norms)
+    B, Hq, S = weights.shape
+    Hkv = idx_bytes.shape[1]
+    group = Hq // Hkv
+    if weights.dtype != torch.float32 or S != tokens or (S > 1 and weights.stride(2) != 1) \
+            or (Hq > 1 and B > 1 and weights.stride(0) != Hq * weights.stride(1)):
+        weights = weights.to(torch.float32).contiguous()
+    stride = weights.stride(1) if Hq > 1 else (weights.stride(0) if B > 1 else max(tokens, 1))
+    out = torch.empty((B, Hq, head_dim), dtype=torch.float32, device=idx_bytes.device)
+    L = lib()
+    splits = L.tq_weighted_values_splits(rows, tokens)
+    step = 8                                             # query heads per kv head and launch
+    with torch.cuda.device(idx_bytes.device):
+        if group <= step:
+            partial = torch.empty((rows, splits, group, head_dim), dtype=torch.float32, device=idx_bytes.device)
+            rc = L.tq_weighted_values(idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, rows, tokens, table.data_ptr(),
+                                      head_dim, bits, weights.data_ptr(), stride, group, partial.data_ptr(), splits,
+                                      out.data_ptr(), _stream_handle(idx_bytes.device))
+            check(rc, "tq_weighted_values")
+        else:
+            # wide groups: one launch per slice of 8 query heads, gathered through a [rows, g, D] buffer
+            w4 = weights.reshape(B, Hkv, group, S) if weights.is_contiguous() else weights.contiguous().reshape(B, Hkv, group, S)
+            o4 = out.view(B, Hkv, group, head_dim)
+            for g0 in range(0, group, step):
+                g1 = min(group, g0 + step)
+                wpart = w4[:, :, g0:g1].contiguous()
+                opart = torch.empty((rows, g1 - g0, head_dim), dtype=torch.float32, device=idx_bytes.device)
+                partial = torch.empty((rows, splits, g1 - g0, head_dim), dtype=torch.float32, device=idx_bytes.device)
+                rc = L.tq_weighted_values(idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, rows, tokens, table.data_ptr(),
+                                          head_dim, bits, wpart.data_ptr(), S, g1 - g0, partial.data_ptr(), splits,
+                                          opart.data_ptr(), _stream_handle(idx_bytes.device))
+                check(rc, "tq_weighted_values")
+                o4[:, :, g0:g1].copy_(opart.view(B, Hkv, g1 - g0, head_dim))
+    return out
+
+
+@weighted_values_op.register_fake
+def _(idx_bytes, vec_norms, table, bits, weights, head_dim):
+    return weights.new_empty((weights.shape[0], weights.shape[1], head_dim), dtype=torch.float32)
 
 
 # ------------------------------------------------------------------------------------

@@ -123,6 +123,36 @@ class MSECompressor:
         return out
 
     @torch.no_grad()
+    def packed_scores(self, idx_bytes: torch.Tensor, vec_norms: torch.Tensor, queries: torch.Tensor,
+                      scale: float = 1.0, out: torch.Tensor = None) -> torch.Tensor:
+        """scale * q . k_hat for every packed key, without de-quantising: queries [B,Hq,1,D] or [B,Hq,D]
+        (Hq a multiple of the packed H: query head j reads kv head j // (Hq/H)), packed keys as accepted
+        by decompress_packed -> float32 scores [B,Hq,S] (written into `out` when given).  Equals
+        attention_scores(queries, decompress(...)) * scale (validate_v3.py:87) up to rounding."""
+        B, H, S, _ = idx_bytes.shape
+        q = queries.reshape(B, -1, self.head_dim)
+        Hq = q.shape[1]
+        if Hq % H:
+            raise ValueError(f"{Hq} query heads do not divide over {H} kv heads")
+        q_rot = torch.matmul(q.to(torch.float32), self.Pi.T) * scale        # (Pi q): rotate once per step
+        if out is None:
+            out = torch.empty((B, Hq, S), dtype=torch.float32, device=idx_bytes.device)
+        if B * Hq * S:
+            torch.ops.tqamd.scores_into(idx_bytes, vec_norms, self.table(), self.bits, q_rot, out)
+        return out
+
+    @torch.no_grad()
+    def packed_weighted_values(self, idx_bytes: torch.Tensor, vec_norms: torch.Tensor,
+                               weights: torch.Tensor) -> torch.Tensor:
+        """sum_t weights[b, hq, t] * v_hat[b, hq // group, t] over the packed values -> float32 [B,Hq,D],
+        accumulated in the rotated space and rotated back once."""
+        B, H, S, _ = idx_bytes.shape
+        if S == 0:
+            return torch.zeros((B, weights.shape[1], self.head_dim), dtype=torch.float32, device=idx_bytes.device)
+        out_rot = torch.ops.tqamd.weighted_values(idx_bytes, vec_norms, self.table(), self.bits, weights, self.head_dim)
+        return torch.matmul(out_rot, self.Pi)
+
+    @torch.no_grad()
     def decompress(self, compressed: dict) -> torch.Tensor:
         """Back to a float32 (B, H, S, D) tensor."""
         B, H, S, D = compressed["shape"]

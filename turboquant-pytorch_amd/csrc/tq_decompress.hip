@@ -32,41 +32,6 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
-// Decode the eight codes of MFMA step s held by this lane into a packed fp16x8 operand.
-// raw[] holds the lane's 64/IPB packed bytes, little-endian dwords.
-template <int IPB, int NW>
-__device__ __forceinline__ tq_u4 decode_step(const uint32_t (&raw)[NW], int s, const uint8_t *lut) {
-    tq_u4 out;
-    if constexpr (IPB == 1) {  // 8 bytes, one code each -> 8 two-byte lookups
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const uint32_t b0 = (raw[2 * s + (2 * d) / 4] >> (8 * ((2 * d) % 4))) & 0xffu;
-            const uint32_t b1 = (raw[2 * s + (2 * d + 1) / 4] >> (8 * ((2 * d + 1) % 4))) & 0xffu;
-            const uint32_t lo = *reinterpret_cast<const uint16_t *>(lut + b0 * 2u);
-            const uint32_t hi = *reinterpret_cast<const uint16_t *>(lut + b1 * 2u);
-            out[d] = lo | (hi << 16);
-        }
-    } else if constexpr (IPB == 2) {  // 4 bytes, two codes each -> 4 four-byte lookups
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const uint32_t b = (raw[s] >> (8 * d)) & 0xffu;
-            out[d] = *reinterpret_cast<const uint32_t *>(lut + b * 4u);
-        }
-    } else if constexpr (IPB == 4) {  // 2 bytes, four codes each -> 2 eight-byte lookups
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            const uint32_t b = (raw[s / 2] >> (16 * (s % 2) + 8 * q)) & 0xffu;
-            const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lut + b * 8u);
-            out[2 * q] = v[0];
-            out[2 * q + 1] = v[1];
-        }
-    } else {  // IPB == 8: 1 byte, eight codes -> 1 sixteen-byte lookup
-        const uint32_t b = (raw[s / 4] >> (8 * (s % 4))) & 0xffu;
-        out = *reinterpret_cast<const tq_u4 *>(lut + b * 16u);
-    }
-    return out;
-}
-
 template <int DTYPE, int IPB>
 __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompress_kernel(TqDevJob job0, const tq_job *jobs) {
     using T = OutTraits<DTYPE>;

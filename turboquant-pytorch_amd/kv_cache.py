@@ -38,10 +38,13 @@ class _LayerStore:
         self.capacity = 0
         self.k_idx = self.k_nrm = self.v_idx = self.v_nrm = None
         self.n_compressed = 0
-        self.window = window
-        # the window store holds the uncompressed tail between calls
-        self.k_win = torch.empty((B, H, max(window, 1), D), dtype=dtype, device=device)
+        self.window_tokens = window
+        # the window store holds the uncompressed tail between calls: tokens [w0, w0 + n_recent) of a
+        # buffer twice the window long, so that it is moved back to the front once per `window` steps
+        self.win_cap = max(2 * window, 1)
+        self.k_win = torch.empty((B, H, self.win_cap, D), dtype=dtype, device=device)
         self.v_win = torch.empty_like(self.k_win)
+        self.w0 = 0
         self.n_recent = 0
         self.total_seq = 0
         self.reserve(capacity)
@@ -82,6 +85,26 @@ class _LayerStore:
         vc.compress_into(values, self.v_idx[:, :, lo:hi], self.v_nrm[:, :, lo:hi])
         self.n_compressed = hi
 
+    def window(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Views [B,H,n_recent,D] of the uncompressed keys and values, oldest first."""
+        return (self.k_win[:, :, self.w0:self.w0 + self.n_recent], self.v_win[:, :, self.w0:self.w0 + self.n_recent])
+
+    def extend_window(self, keys: torch.Tensor, values: torch.Tensor) -> None:
+        n = keys.shape[2]
+        if n == 0:
+            return
+        if self.w0 + self.n_recent + n > self.win_cap:
+            if self.n_recent:
+                k, v = self.window()
+                k, v = k.clone(), v.clone()
+                self.k_win[:, :, :self.n_recent].copy_(k)
+                self.v_win[:, :, :self.n_recent].copy_(v)
+            self.w0 = 0
+        lo = self.w0 + self.n_recent
+        self.k_win[:, :, lo:lo + n].copy_(keys)
+        self.v_win[:, :, lo:lo + n].copy_(values)
+        self.n_recent += n
+
 
 class V3Cache:
     """Streaming compressed KV cache; `update` follows generation_test_v2.py:80-153."""
@@ -113,10 +136,8 @@ class V3Cache:
             )
         return self._compressors[layer_idx]
 
-    @torch.no_grad()
-    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
-               cache_kwargs: Optional[dict] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-        B, H, S_new, D = key_states.shape
+    def _store(self, key_states: torch.Tensor, layer_idx: int) -> _LayerStore:
+        B, H, _, D = key_states.shape
         device = key_states.device
         comp = self._get_compressor(layer_idx, D, device)
         st = self._stores.get(layer_idx)
@@ -126,38 +147,83 @@ class V3Cache:
         elif (st.B, st.H, st.D) != (B, H, D):
             raise ValueError(f"layer {layer_idx}: states {tuple(key_states.shape)} do not match the cached "
                              f"batch/head/dim {(st.B, st.H, st.D)}")
-        st.total_seq += S_new
+        return st
 
-        # the uncompressed tokens are (window ++ new); everything beyond the last `rw` of them leaves
+    def _push(self, st: _LayerStore, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
+        """Bookkeeping of generation_test_v2.py:96-126: the uncompressed tokens are (window ++ new); all but
+        the last `residual_window` of them are compressed for good, the rest is the new window."""
+        S_new = key_states.shape[2]
+        st.total_seq += S_new
         rw = self.residual_window
         recent = st.n_recent + S_new
         overflow = recent if rw == 0 else max(recent - rw, 0)
         from_window = min(overflow, st.n_recent)
         from_new = overflow - from_window
-        st.append_compressed(st.k_win[:, :, :from_window], st.v_win[:, :, :from_window])
+        kw, vw = st.window()
+        st.append_compressed(kw[:, :, :from_window], vw[:, :, :from_window])
         st.append_compressed(key_states[:, :, :from_new], value_states[:, :, :from_new])
+        st.w0 += from_window
+        st.n_recent -= from_window
+        if st.n_recent == 0:
+            st.w0 = 0
+        st.extend_window(key_states[:, :, from_new:], value_states[:, :, from_new:])
 
-        keep_old = st.n_recent - from_window
-        keep_new = S_new - from_new
+    @torch.no_grad()
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
+               cache_kwargs: Optional[dict] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        B, H, S_new, D = key_states.shape
+        device = key_states.device
+        st = self._store(key_states, layer_idx)
+        comp = st.comp
+        self._push(st, key_states, value_states)
         n_c = st.n_compressed
-        total = n_c + keep_old + keep_new
+        total = n_c + st.n_recent
         full_k = torch.empty((B, H, total, D), dtype=key_states.dtype, device=device)
         full_v = torch.empty((B, H, total, D), dtype=value_states.dtype, device=device)
         if n_c:
             comp.key_compressor.decompress_packed(st.k_idx[:, :, :n_c], st.k_nrm[:, :, :n_c], full_k[:, :, :n_c])
             comp.val_compressor.decompress_packed(st.v_idx[:, :, :n_c], st.v_nrm[:, :, :n_c], full_v[:, :, :n_c])
-        if keep_old:
-            full_k[:, :, n_c:n_c + keep_old].copy_(st.k_win[:, :, from_window:st.n_recent])
-            full_v[:, :, n_c:n_c + keep_old].copy_(st.v_win[:, :, from_window:st.n_recent])
-        if keep_new:
-            full_k[:, :, n_c + keep_old:].copy_(key_states[:, :, from_new:])
-            full_v[:, :, n_c + keep_old:].copy_(value_states[:, :, from_new:])
-        # the tail of the output is the next window
-        st.n_recent = keep_old + keep_new
         if st.n_recent:
-            st.k_win[:, :, :st.n_recent].copy_(full_k[:, :, n_c:])
-            st.v_win[:, :, :st.n_recent].copy_(full_v[:, :, n_c:])
+            kw, vw = st.window()
+            full_k[:, :, n_c:].copy_(kw)
+            full_v[:, :, n_c:].copy_(vw)
         return full_k, full_v
+
+    @torch.no_grad()
+    def append(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int) -> None:
+        """`update` without building the full-length tensors: the state afterwards is the same.  For decode
+        loops that read the cache through `attend`."""
+        self._push(self._store(key_states, layer_idx), key_states, value_states)
+
+    @torch.no_grad()
+    def attend(self, query_states: torch.Tensor, layer_idx: int, scale: Optional[float] = None) -> torch.Tensor:
+        """softmax(scale * q K^T) V of one query token per sequence, [B,Hq,1,D] -> [B,Hq,1,D], over everything
+        cached for the layer -- what the model computes from the tensors `update` returns -- read
+        straight from the packed store: scores from the packed keys (query rotated once), softmax in
+        float32, the weighted sum of the packed values in the rotated space, window tokens as they are.
+        Query head j uses kv head j // (Hq / H)."""
+        st = self._stores[layer_idx]
+        B, Hq, Sq, D = query_states.shape
+        if Sq != 1 or B != st.B or Hq % st.H:
+            raise ValueError(f"attend needs one query token per sequence, [B={st.B}, k*{st.H}, 1, {st.D}]; got {tuple(query_states.shape)}")
+        G = Hq // st.H
+        scale = D ** -0.5 if scale is None else scale
+        n_c, n_w = st.n_compressed, st.n_recent
+        kc, vc = st.comp.key_compressor, st.comp.val_compressor
+        scores = torch.empty((B, Hq, n_c + n_w), dtype=torch.float32, device=query_states.device)
+        if n_c:
+            kc.packed_scores(st.k_idx[:, :, :n_c], st.k_nrm[:, :, :n_c], query_states, scale, out=scores[:, :, :n_c])
+        q4 = query_states.reshape(B, st.H, G, D).to(torch.float32)
+        kw, vw = st.window()
+        if n_w:
+            kw = kw.to(torch.float32)
+            scores[:, :, n_c:] = (torch.matmul(q4, kw.transpose(-2, -1)) * scale).reshape(B, Hq, n_w)
+        probs = torch.softmax(scores, dim=-1)
+        out = vc.packed_weighted_values(st.v_idx[:, :, :n_c], st.v_nrm[:, :, :n_c], probs[:, :, :n_c])
+        if n_w:
+            vw = vw.to(torch.float32)
+            out = out + torch.matmul(probs[:, :, n_c:].reshape(B, st.H, G, n_w), vw).reshape(B, Hq, D)
+        return out.to(query_states.dtype).reshape(B, Hq, 1, D)
 
     def get_seq_length(self, layer_idx: int = 0) -> int:
         st = self._stores.get(layer_idx)
