@@ -143,21 +143,39 @@ struct WvArgs {
 };
 
 // Block (split, row): sum over the split's tokens of  weight[g][t] * norm_t * centroids[codes_t]  for the
-// row's `group` query heads, in the rotated space.  A wave takes tiles of 32 tokens: the packed bytes and
-// the norm-scaled weights go through a wave-private LDS area, then lane l accumulates coordinates 2l, 2l+1
-// of every query head over the tile's tokens (the contraction runs over tokens, a few rows only: VALU work).
+// row's `group` query heads, in the rotated space: a [group x tokens] x [tokens x 128] product whose
+// contraction runs over tokens, on v_mfma_f32_32x32x16_f16.  A wave takes runs of up to 128 tokens (4 KiB of
+// packed bytes, so that enough memory traffic is in flight per wave; loads run one run ahead):
+//   * the run's packed bytes (contiguous in memory), norms and weights are staged in a wave-private LDS area;
+//   * per tile of 32 tokens, lane (n, hk) owns coordinates 4n .. 4n+3 and, per MFMA step ks, tokens
+//     16ks + 8hk + i (i < 8): for each of those tokens it reads the byte(s) holding its four codes and looks them
+//     up in the byte -> centroids table, so every lookup is used in full; a token-pair byte permute inside the
+//     lane turns the 8 x 4 values into four B operands (one per coordinate: MFMA column n of column tile c is
+//     coordinate 4n + c), scaled by the tokens' norms in packed fp16;
+//   * the A operand holds the weights (rows = query heads, zero above `group`) as fp16 hi + lo of
+//     w * 2^14: weights are probabilities, so everything down to 2^-38 keeps at least a denormal.
+// Accumulators (4 column tiles) live in registers across the split; the four waves' sums meet in LDS.
 template <int IPB>
 __global__ __launch_bounds__(WV_WAVES *TQ_WAVE) void tq_weighted_values_kernel(WvArgs a) {
-    constexpr int GB = TQ_HEAD_DIM / IPB;            // packed bytes per vector
-    constexpr int TILE_BYTES = 32 * GB;              // 512 .. 4096
-    constexpr int PIECES = TILE_BYTES / 16;          // 16-byte pieces per tile: 32 .. 256
+    constexpr int GB = TQ_HEAD_DIM / IPB;                    // packed bytes per vector: 16 .. 128
+    constexpr int SUB = GB >= 128 ? 1 : GB >= 64 ? 2 : 4;    // 32-token tiles per run
+    constexpr int RUN = 32 * SUB;                            // tokens per run: 32, 64, 128
+    constexpr int CODE_BYTES = RUN * GB;                     // <= 4096
+    constexpr int CPIECES = CODE_BYTES / 16;                 // 16-byte pieces of packed bytes per run
+    constexpr int NCP = (CPIECES + 63) / 64;
+    constexpr int WROW = RUN / 4;                            // 16-byte pieces per weight row and run
+    constexpr int WPIECES = WV_MAX_GROUP * WROW;
+    constexpr int NWP = (WPIECES + 63) / 64;
+    constexpr int W_SHIFT = 14;
+    constexpr int AREA = 4096 + WV_MAX_GROUP * RUN * 4;      // per wave: staged codes + weights, later the wave's sums
+    static_assert(CODE_BYTES <= 4096 && WV_MAX_GROUP * TQ_HEAD_DIM * 4 <= AREA, "wave area too small");
     __shared__ __attribute__((aligned(16))) uint8_t lds_lut[4096];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_codes[WV_WAVES][TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) float lds_w[WV_WAVES][32][WV_MAX_GROUP];
-    __shared__ float lds_red[WV_WAVES][WV_MAX_GROUP][TQ_HEAD_DIM];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_area[WV_WAVES][AREA];
+    __shared__ __attribute__((aligned(16))) uint16_t lds_norm[WV_WAVES][RUN];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t row = blockIdx.y, split = blockIdx.x;
+    const uint32_t n = lane & 31u, hk = lane >> 5;
     const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(a.table);
     tq_copy_to_lds(lds_lut, a.table + hd->off_lut, 256u * 2u * IPB, tid, WV_WAVES * TQ_WAVE);
     __syncthreads();
@@ -166,72 +184,160 @@ __global__ __launch_bounds__(WV_WAVES *TQ_WAVE) void tq_weighted_values_kernel(W
     const uint32_t t_end = min(a.tokens, t_begin + a.chunk);
     const size_t slot0 = (size_t)row * a.packed_row_stride;
     const uint32_t G = a.group;
+    const bool live = n < G;                                   // this lane's MFMA row is a query head
+    const TQ_GLOBAL float *wbase = (const TQ_GLOBAL float *)a.weights + (size_t)row * G * a.stride;
+    uint8_t *codes = lds_area[wave];
+    float *wst = reinterpret_cast<float *>(lds_area[wave] + 4096);      // [query head][token of the run]
+    // rows of the weight matrix start 16-byte aligned: four weights are one vector load
+    const bool aligned_rows = (a.stride % 4 == 0) && (((uintptr_t)a.weights & 15u) == 0);
 
-    // where this lane's two codes (coordinates 2l, 2l+1) sit: byte inside a vector, fp16 pair inside the table entry
-    const uint32_t byte_in_vec = (2u * lane) / IPB;
-    const uint32_t pair_off = ((2u * lane) % IPB) * 2u;
-
-    float acc[WV_MAX_GROUP][2];
+    tq_f16v acc[TQ_TILES];
 #pragma unroll
-    for (int g = 0; g < WV_MAX_GROUP; ++g) acc[g][0] = acc[g][1] = 0.f;
+    for (int c = 0; c < TQ_TILES; ++c) acc[c] = tq_zero16();
 
-    for (uint32_t t0 = t_begin + 32u * wave; t0 < t_end; t0 += 32u * WV_WAVES) {
-        const uint32_t n_tok = min(32u, t_end - t0);
-        // packed bytes of the tile: contiguous in memory (tokens of one row follow each other)
+    // loads of a run, issued one run ahead of their use
+    tq_u4 code_next[NCP];
+    tq_u4 w_next[NWP];
+    uint16_t norm_next[(RUN + 63) / 64];
+    auto issue_loads = [&](uint32_t t0) {
+        const uint32_t n_tok = min((uint32_t)RUN, t_end - t0);
         const uint8_t *src = a.idx_bytes + (slot0 + t0) * GB;
 #pragma unroll
-        for (int p = 0; p < (PIECES + 63) / 64; ++p) {
+        for (int p = 0; p < NCP; ++p) {
             const uint32_t piece = p * 64u + lane;
-            if (piece < PIECES && piece * 16u < n_tok * GB)
-                *reinterpret_cast<tq_u4 *>(&lds_codes[wave][piece * 16u]) = tq_gload16(src + piece * 16u);
+            const bool ok = piece < CPIECES && piece * 16u < n_tok * GB;
+            code_next[p] = tq_gload16(src + (ok ? piece : 0u) * 16u);
         }
-        // weights times norms, [token][head]
-        {
-            const uint32_t tl = lane & 31u;
-            const bool ok = tl < n_tok;
-            const float nrm = ok ? (float)__builtin_bit_cast(_Float16, tq_gload2(a.vec_norms + slot0 + t0 + tl)) : 0.f;
-            for (uint32_t g = lane >> 5; g < WV_MAX_GROUP; g += 2u) {
-                float w = 0.f;
-                if (ok && g < G) w = ((const TQ_GLOBAL float *)a.weights)[((size_t)row * G + g) * a.stride + t0 + tl] * nrm;
-                lds_w[wave][tl][g] = w;
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-        for (uint32_t tl = 0; tl < n_tok; ++tl) {
-            float c0, c1;
-            if constexpr (IPB == 1) {
-                const uint32_t two = *reinterpret_cast<const uint16_t *>(&lds_codes[wave][tl * GB + 2u * lane]);
-                c0 = (float)__builtin_bit_cast(_Float16, *reinterpret_cast<const uint16_t *>(lds_lut + (two & 0xffu) * 2u));
-                c1 = (float)__builtin_bit_cast(_Float16, *reinterpret_cast<const uint16_t *>(lds_lut + (two >> 8) * 2u));
-            } else {
-                const uint32_t b = lds_codes[wave][tl * GB + byte_in_vec];
-                const tq_half2 c = __builtin_bit_cast(tq_half2, *reinterpret_cast<const uint32_t *>(lds_lut + b * (2u * IPB) + pair_off));
-                c0 = (float)c[0];
-                c1 = (float)c[1];
-            }
-            const float4 w03 = *reinterpret_cast<const float4 *>(&lds_w[wave][tl][0]);
-            const float4 w47 = *reinterpret_cast<const float4 *>(&lds_w[wave][tl][4]);
-            const float w[8] = {w03.x, w03.y, w03.z, w03.w, w47.x, w47.y, w47.z, w47.w};
 #pragma unroll
-            for (int g = 0; g < WV_MAX_GROUP; ++g) {
-                acc[g][0] = fmaf(w[g], c0, acc[g][0]);
-                acc[g][1] = fmaf(w[g], c1, acc[g][1]);
+        for (int p = 0; p < (RUN + 63) / 64; ++p) {
+            const uint32_t tl = p * 64u + lane;
+            norm_next[p] = (tl < n_tok) ? tq_gload2(a.vec_norms + slot0 + t0 + tl) : (uint16_t)0;   // tokens past the end weigh nothing
+        }
+#pragma unroll
+        for (int p = 0; p < NWP; ++p) {
+            const uint32_t piece = p * 64u + lane;
+            const uint32_t g = piece / WROW, tl = (piece % WROW) * 4u;
+            tq_u4 v = {0u, 0u, 0u, 0u};
+            if (piece < WPIECES && g < G && tl < n_tok) {
+                const TQ_GLOBAL float *wp = wbase + (size_t)g * a.stride + t0 + tl;
+                if (aligned_rows && tl + 4u <= n_tok) {
+                    v = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>(wp);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = (tl + i < n_tok) ? __float_as_uint(wp[i]) : 0u;
+                }
+            }
+            w_next[p] = v;
+        }
+    };
+    uint32_t t0 = t_begin + RUN * wave;
+    if (t0 < t_end) issue_loads(t0);
+    while (t0 < t_end) {
+        // ---- stage the run: packed bytes [token][GB], norms [token], weights [head][token]
+#pragma unroll
+        for (int p = 0; p < NCP; ++p) {
+            const uint32_t piece = p * 64u + lane;
+            if (piece < CPIECES) *reinterpret_cast<tq_u4 *>(codes + piece * 16u) = code_next[p];
+        }
+#pragma unroll
+        for (int p = 0; p < (RUN + 63) / 64; ++p) {
+            const uint32_t tl = p * 64u + lane;
+            if (tl < RUN) lds_norm[wave][tl] = norm_next[p];
+        }
+#pragma unroll
+        for (int p = 0; p < NWP; ++p) {
+            const uint32_t piece = p * 64u + lane;
+            if (piece < WPIECES) *reinterpret_cast<tq_u4 *>(wst + piece * 4u) = w_next[p];
+        }
+        const uint32_t t_next = t0 + RUN * WV_WAVES;
+        if (t_next < t_end) issue_loads(t_next);
+        // staged as 16-byte vectors, read back in other units: no compiler reordering across this point
+        // (the LDS itself serves a wave in order)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const uint32_t tl0 = 32u * u + 16u * ks + 8u * hk;          // this lane's eight tokens of the step
+                // weights of this lane's query head, fp16 hi + lo of w * 2^W_SHIFT
+                tq_u4 whi = {0u, 0u, 0u, 0u}, wlo = {0u, 0u, 0u, 0u};
+                if (live) {
+                    const float4 w0 = *reinterpret_cast<const float4 *>(wst + n * RUN + tl0);
+                    const float4 w1 = *reinterpret_cast<const float4 *>(wst + n * RUN + tl0 + 4);
+                    const float x[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+                    tq_half8 h, l;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const float xs = x[i] * (float)(1 << W_SHIFT);
+                        const _Float16 xh = (_Float16)xs;
+                        h[i] = xh;
+                        l[i] = (_Float16)(xs - (float)xh);
+                    }
+                    whi = __builtin_bit_cast(tq_u4, h);
+                    wlo = __builtin_bit_cast(tq_u4, l);
+                }
+                const tq_u4 nrm = *reinterpret_cast<const tq_u4 *>(&lds_norm[wave][tl0]);   // fp16 norms of the eight tokens
+                uint32_t lo[8], hi[8];   // per token: centroids of coordinates (4n, 4n+1) and (4n+2, 4n+3)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint8_t *tok = codes + (tl0 + i) * GB;
+                    if constexpr (IPB == 8) {          // half a byte holds the lane's four codes
+                        const uint32_t b = tok[n >> 1];
+                        const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lds_lut + b * 16u + (n & 1u) * 8u);
+                        lo[i] = v[0]; hi[i] = v[1];
+                    } else if constexpr (IPB == 4) {   // one byte
+                        const uint32_t b = tok[n];
+                        const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lds_lut + b * 8u);
+                        lo[i] = v[0]; hi[i] = v[1];
+                    } else if constexpr (IPB == 2) {   // two bytes
+                        const uint32_t two = *reinterpret_cast<const uint16_t *>(tok + 2u * n);
+                        lo[i] = *reinterpret_cast<const uint32_t *>(lds_lut + (two & 0xffu) * 4u);
+                        hi[i] = *reinterpret_cast<const uint32_t *>(lds_lut + (two >> 8) * 4u);
+                    } else {                           // four bytes, one code each
+                        const uint32_t four = *reinterpret_cast<const uint32_t *>(tok + 4u * n);
+                        const uint32_t c0 = *reinterpret_cast<const uint16_t *>(lds_lut + (four & 0xffu) * 2u);
+                        const uint32_t c1 = *reinterpret_cast<const uint16_t *>(lds_lut + ((four >> 8) & 0xffu) * 2u);
+                        const uint32_t c2 = *reinterpret_cast<const uint16_t *>(lds_lut + ((four >> 16) & 0xffu) * 2u);
+                        const uint32_t c3 = *reinterpret_cast<const uint16_t *>(lds_lut + (four >> 24) * 2u);
+                        lo[i] = c0 | (c1 << 16); hi[i] = c2 | (c3 << 16);
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < TQ_TILES; ++c) {
+                    // coordinate 4n + c of the eight tokens: token pairs (2d, 2d+1) side by side, times their norms
+                    tq_u4 bt;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const uint32_t even = c < 2 ? lo[2 * d] : hi[2 * d], odd = c < 2 ? lo[2 * d + 1] : hi[2 * d + 1];
+                        bt[d] = __builtin_amdgcn_perm(odd, even, (c & 1) ? 0x07060302u : 0x05040100u);
+                    }
+                    const tq_half8 y = __builtin_bit_cast(tq_half8, bt) * __builtin_bit_cast(tq_half8, nrm);
+                    acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, whi), y, acc[c], 0, 0, 0);
+                    acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, wlo), y, acc[c], 0, 0, 0);
+                }
             }
         }
+        asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();
+        t0 = t_next;
     }
+    asm volatile("" ::: "memory");
+    // accumulator register r of lane (n, hk), column tile c: query head 8*(r/4) + 4*hk + r%4, coordinate 4n + c
+    float *sums = reinterpret_cast<float *>(lds_area[wave]);
 #pragma unroll
-    for (int g = 0; g < WV_MAX_GROUP; ++g) {
-        lds_red[wave][g][2 * lane] = acc[g][0];
-        lds_red[wave][g][2 * lane + 1] = acc[g][1];
-    }
+    for (int c = 0; c < TQ_TILES; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t m = 8u * (r / 4) + 4u * hk + (r % 4);
+            if (m < WV_MAX_GROUP) sums[m * TQ_HEAD_DIM + 4u * n + c] = acc[c][r] * (1.0f / (float)(1 << W_SHIFT));
+        }
     __syncthreads();
     float *dst = a.partial + ((size_t)row * gridDim.x + split) * G * TQ_HEAD_DIM;
     for (uint32_t i = tid; i < G * TQ_HEAD_DIM; i += WV_WAVES * TQ_WAVE) {
-        const uint32_t g = i / TQ_HEAD_DIM, j = i % TQ_HEAD_DIM;
         float s = 0.f;
 #pragma unroll
-        for (int w = 0; w < WV_WAVES; ++w) s += lds_red[w][g][j];
+        for (int w = 0; w < WV_WAVES; ++w) s += reinterpret_cast<const float *>(lds_area[w])[i];
         ((TQ_GLOBAL float *)dst)[i] = s;
     }
 }
@@ -323,7 +429,7 @@ extern "C" int tq_weighted_values_splits(long long rows, long long tokens) {
     int cus = 0;
     if (device_cus(cus)) cus = 256;
     long long splits = ((long long)cus * 8 + rows - 1) / rows;       // ~8 four-wave blocks per compute unit
-    const long long most = (tokens + 32 * WV_WAVES - 1) / (32 * WV_WAVES);
+    const long long most = (tokens + 128 * WV_WAVES - 1) / (128 * WV_WAVES);
     if (splits > most) splits = most;
     if (splits > 4096) splits = 4096;
     return splits < 1 ? 1 : (int)splits;
@@ -359,7 +465,7 @@ extern "C" int tq_weighted_values(const uint8_t *idx_bytes, const uint16_t *vec_
     a.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     a.group = (uint32_t)group;
     const long long per_split = (tokens + splits - 1) / splits;
-    a.chunk = (uint32_t)((per_split + 31) / 32 * 32);
+    a.chunk = (uint32_t)((per_split + 127) / 128 * 128);
     dim3 grid((unsigned)splits, (unsigned)rows, 1), block(WV_WAVES * TQ_WAVE, 1, 1);
     switch (8 / bits) {
         case 8: hipLaunchKernelGGL(tq_weighted_values_kernel<8>, grid, block, 0, s, a); break;

@@ -210,19 +210,25 @@ class V3Cache:
         scale = D ** -0.5 if scale is None else scale
         n_c, n_w = st.n_compressed, st.n_recent
         kc, vc = st.comp.key_compressor, st.comp.val_compressor
-        scores = torch.empty((B, Hq, n_c + n_w), dtype=torch.float32, device=query_states.device)
+        # rows padded to a multiple of 8 floats (the kernels read weights with 16-byte loads); the padding
+        # scores are -inf, so the softmax runs over the whole contiguous buffer
+        total = n_c + n_w
+        width = -(-total // 8) * 8
+        scores = torch.empty((B, Hq, width), dtype=torch.float32, device=query_states.device)
+        if width > total:
+            scores[:, :, total:] = float("-inf")
         if n_c:
             kc.packed_scores(st.k_idx[:, :, :n_c], st.k_nrm[:, :, :n_c], query_states, scale, out=scores[:, :, :n_c])
         q4 = query_states.reshape(B, st.H, G, D).to(torch.float32)
         kw, vw = st.window()
         if n_w:
             kw = kw.to(torch.float32)
-            scores[:, :, n_c:] = (torch.matmul(q4, kw.transpose(-2, -1)) * scale).reshape(B, Hq, n_w)
+            scores[:, :, n_c:total] = (torch.matmul(q4, kw.transpose(-2, -1)) * scale).reshape(B, Hq, n_w)
         probs = torch.softmax(scores, dim=-1)
         out = vc.packed_weighted_values(st.v_idx[:, :, :n_c], st.v_nrm[:, :, :n_c], probs[:, :, :n_c])
         if n_w:
             vw = vw.to(torch.float32)
-            out = out + torch.matmul(probs[:, :, n_c:].reshape(B, st.H, G, n_w), vw).reshape(B, Hq, D)
+            out = out + torch.matmul(probs[:, :, n_c:total].reshape(B, st.H, G, n_w), vw).reshape(B, Hq, D)
         return out.to(query_states.dtype).reshape(B, Hq, 1, D)
 
     def get_seq_length(self, layer_idx: int = 0) -> int:
