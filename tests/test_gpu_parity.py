@@ -399,3 +399,78 @@ def test_round_trip_properties_at_scale(pkg):
     assert float(same) > 0.995
     rel = (rec - x.float()).norm() / x.float().norm()
     assert 0.09 < float(rel) < 0.105          # sqrt(0.0095): the 4-bit Lloyd-Max distortion
+
+
+# ---------------------------------------------------------------------------------------------
+# the other published configurations at their real tensor shapes (one layer each against the oracle)
+# ---------------------------------------------------------------------------------------------
+def test_config2_shape_qwen_8k(pkg, oracle):
+    """Qwen2.5-3B-shaped layer: [1,2,8192,128] fp16 with per-channel outliers, K4/V2, no window, layer 17 of
+    36: packed bytes against the oracle (boundary window), norms, de-quantised tensors; then all 36 layers
+    in one batched launch give the bytes of per-layer calls."""
+    L, shape = 36, (1, 2, 8192, 128)
+    tq = pkg.TurboQuantV3(128, key_bits=4, value_bits=2, residual_window=0, layer_idx=17, n_layers=L,
+                          protected_layers=0, device=DEV)
+    keys = outlier_kv(shape, seed=2_000_170, dtype=torch.float16)
+    vals = outlier_kv(shape, seed=2_000_171, dtype=torch.float16)
+    ck, cv = tq.compress_kv(keys.to(DEV), vals.to(DEV))
+    assert ck["split_at"] == 8192 and ck["fp16"].shape[2] == 0
+    rk, rv = tq.decompress_kv(ck, cv)
+    for c, x, comp, rec, name in ((ck, keys, tq.key_compressor, rk, "K4"), (cv, vals, tq.val_compressor, rv, "V2")):
+        Pi, cent = comp.Pi.cpu().numpy(), comp.centroids.cpu().numpy()
+        ref, _ = check_codes(oracle, c["compressed"]["idx_bytes"].cpu().numpy(), x.float().numpy().reshape(-1, 128), Pi, cent,
+                             comp.bits, f"config 2 {name}")
+        check_norms(oracle, bits16(c["compressed"]["vec_norms"]), ref["vec_norms"], f"config 2 {name}")
+        want = oracle.COracle(Pi, cent, comp.bits, True).decompress(ref["idx_bytes"], ref["vec_norms"])
+        err, _ = rel_l2(rec.float().cpu().numpy().reshape(-1, 128), want)
+        assert rec.dtype == torch.float16 and err < 2e-3, (name, err)      # fp16 output rounding on top of 1e-3
+    assert tq.memory_bytes(*shape[:3])["compressed_bytes"] == 2 * 8192 * (64 + 2 + 32 + 2)
+    native = pkg._native
+    comps = [pkg.TurboQuantV3(128, 4, 2, residual_window=0, layer_idx=l, n_layers=L, protected_layers=0, device=DEV) for l in range(L)]
+    xs = [outlier_kv((1, 2, 1024, 128), seed=2_000_000 + l, dtype=torch.float16).to(DEV) for l in range(L)]
+    jobs = [{"states": x, "idx_bytes": torch.zeros(1, 2, 1024, 64, dtype=torch.uint8, device=DEV),
+             "vec_norms": torch.zeros(1, 2, 1024, dtype=torch.float16, device=DEV), "table": c.key_compressor.table(), "bits": 4}
+            for x, c in zip(xs, comps)]
+    native.JobList(jobs, DEV).compress()
+    torch.cuda.synchronize()
+    for j, x, c in zip(jobs, xs, comps):
+        one = c.key_compressor.compress(x)
+        assert torch.equal(j["idx_bytes"], one["idx_bytes"]) and torch.equal(j["vec_norms"], one["vec_norms"])
+
+
+def test_config3_shape_k6v4_window(pkg, oracle):
+    """[8,2,4096,128] fp16, K6/V4, window 128, 16 query heads over 2 KV heads: 3968 compressed + 128 window
+    tokens per row; bytes against the oracle, the window verbatim, attention-score metrics as the reference
+    defines them (batch element 0) equal between the kernel path and the oracle path."""
+    B, H, S, D, G = 8, 2, 4096, 128, 8
+    tq = pkg.TurboQuantV3(D, key_bits=6, value_bits=4, residual_window=128, layer_idx=20, n_layers=36,
+                          protected_layers=0, device=DEV)
+    keys = outlier_kv((B, H, S, D), seed=3_000_200, dtype=torch.float16)
+    vals = outlier_kv((B, H, S, D), seed=3_000_201, dtype=torch.float16)
+    ck, cv = tq.compress_kv(keys.to(DEV), vals.to(DEV))
+    assert ck["split_at"] == 3968 and tuple(ck["compressed"]["idx_bytes"].shape) == (B, H, 3968, 128)
+    assert tuple(cv["compressed"]["idx_bytes"].shape) == (B, H, 3968, 64)
+    rk, rv = tq.decompress_kv(ck, cv)
+    assert torch.equal(rk[:, :, 3968:].cpu(), keys[:, :, 3968:]) and torch.equal(rv[:, :, 3968:].cpu(), vals[:, :, 3968:])
+    ref_k = None
+    for c, x, comp, name in ((ck, keys, tq.key_compressor, "K6"), (cv, vals, tq.val_compressor, "V4")):
+        Pi, cent = comp.Pi.cpu().numpy(), comp.centroids.cpu().numpy()
+        flat = np.ascontiguousarray(x[:, :, :3968].float().numpy()).reshape(-1, D)
+        ref, _ = check_codes(oracle, c["compressed"]["idx_bytes"].cpu().numpy(), flat, Pi, cent, comp.bits, f"config 3 {name}")
+        check_norms(oracle, bits16(c["compressed"]["vec_norms"]), ref["vec_norms"], f"config 3 {name}")
+        if name == "K6":
+            ref_k = oracle.COracle(Pi, cent, 6, True).decompress(ref["idx_bytes"], ref["vec_norms"]).reshape(B, H, 3968, D)
+    g = torch.Generator(device="cpu")
+    g.manual_seed(3_000_203)
+    q = torch.randn(B, H * G, 1, D, generator=g) / np.sqrt(D)
+    full_ref = torch.cat([torch.from_numpy(ref_k).to(torch.float16), keys[:, :, 3968:]], dim=2)
+    real = pkg.attention_scores(q, keys.repeat_interleave(G, dim=1))
+    hip = pkg.attention_scores(q, rk.cpu().repeat_interleave(G, dim=1))
+    cpu = pkg.attention_scores(q, full_ref.repeat_interleave(G, dim=1))
+    m_hip, m_cpu = pkg.compute_metrics(real, hip, H * G), pkg.compute_metrics(real, cpu, H * G)
+    print(f"[config 3] kernel path {m_hip}\n[config 3] oracle path {m_cpu}")
+    assert round(m_hip["cosine_sim"], 4) == round(m_cpu["cosine_sim"], 4) and m_hip["cosine_sim"] > 0.999
+    assert abs(m_hip["top1_matches"] - m_cpu["top1_matches"]) <= 1 and m_hip["top5_matches"] >= m_hip["top1_matches"]
+    mem = tq.memory_bytes(B, H, S)
+    assert mem["compressed_tokens"] == 3968 and mem["fp16_tokens"] == 128 and mem["key_bits"] == 6 and mem["value_bits"] == 4
+    assert mem["compressed_bytes"] == B * H * (3968 * (128 + 2 + 64 + 2) + 128 * D * 2 * 2)
