@@ -11,6 +11,8 @@
 // v_mfma_f32_32x32x16_f16; the A operand is Pi^T in fp16, fp32 accumulate.  The 32x128 result
 // tile is transposed through a wave-private, XOR-swizzled LDS buffer so that every store
 // instruction writes 1 KiB of consecutive memory.
+#include <type_traits>
+
 #include "tq_device.h"
 
 namespace {
@@ -69,38 +71,68 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     const uint32_t n = lane & 31u, hk = lane >> 5;
     const uint32_t st_vec = lane / PIECES, st_piece = lane % PIECES;
 
+    // Addressing of a tile.  The tile index is the same for the whole wave, so the split of its first
+    // vector into (row, token) is one scalar division per tile; the other vectors follow by adding
+    // per-lane constants, plus one fixed correction for those past the end of the row (rows hold at
+    // least 32 tokens on this path, so a tile crosses at most one row boundary).
+    const bool one_row = job.tokens >= job.n_vec;
+    const bool fast = (one_row || job.tokens >= 32u) && job.token_stride < (1ll << 24);
+    struct Origin {
+        long long out_base;   // byte offset of the tile's first vector in the output tensor
+        uint32_t slot_base;   // its packed slot
+        uint32_t in_row;      // vectors of the tile that still belong to that row
+    };
+    auto origin_of = [&](uint32_t tl) {
+        Origin o;
+        const uint32_t v0 = __builtin_amdgcn_readfirstlane(tl) * 32u;
+        const uint32_t row = one_row ? 0u : v0 / job.tokens;
+        const uint32_t tok = v0 - row * job.tokens;
+        o.out_base = (long long)row * job.row_stride + (long long)tok * job.token_stride;
+        o.slot_base = one_row ? tok : row * job.packed_row_stride + tok;
+        o.in_row = one_row ? 32u : job.tokens - tok;
+        return o;
+    };
+    // jump of the output offset / packed slot from the last vector of a row to the first of the next
+    const long long row_wrap = job.row_stride - (long long)job.tokens * job.token_stride;
+    const uint32_t slot_wrap = job.packed_row_stride - job.tokens;
+    uint32_t st_off[NSTORE];   // byte offset of this lane's piece of store j relative to the tile's first vector
+#pragma unroll
+    for (int j = 0; j < NSTORE; ++j) st_off[j] = (j * VEC_PER_STORE + st_vec) * (uint32_t)job.token_stride + st_piece * 16u;
+
     uint32_t raw[NW];
     uint16_t norm_bits = 0;
-    auto issue_loads = [&](uint32_t tl) {
-        const uint32_t v = tl * 32u + n;
-        const bool ok = v < job.n_vec;
-        const uint32_t slot = ok ? tq_packed_slot(job, v) : 0u;
+    // this lane's half vector of tile `tl` (FULL: all 32 vectors of the tile exist, nothing is predicated)
+    auto issue_loads = [&](auto full_tag, auto fast_tag, uint32_t tl) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        constexpr bool FAST = decltype(fast_tag)::value;
+        const bool ok = FULL || tl * 32u + n < job.n_vec;
+        const uint32_t vl = ok ? n : 0u;
+        uint32_t slot;
+        if constexpr (FAST) {
+            const Origin o = origin_of(tl);
+            slot = o.slot_base + vl + (vl >= o.in_row ? slot_wrap : 0u);
+        } else {   // rows shorter than a tile: the general formula
+            slot = tq_packed_slot(job, tl * 32u + vl);
+        }
         const uint8_t *src = job.idx_bytes + (size_t)slot * (2 * NB) + hk * NB;
         if constexpr (NW == 2) {
-            tq_u2 t = {0u, 0u};
-            if (ok) t = tq_gload8(src);
+            const tq_u2 t = tq_gload8(src);
             raw[0] = t[0]; raw[1] = t[1];
         } else {
 #pragma unroll
             for (int q = 0; q < NW / 4; ++q) {
-                tq_u4 t = {0u, 0u, 0u, 0u};
-                if (ok) t = tq_gload16(src + 16 * q);
+                const tq_u4 t = tq_gload16(src + 16 * q);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) raw[4 * q + i] = t[i];
             }
         }
-        norm_bits = ok ? tq_gload2(job.vec_norms + slot) : (uint16_t)0;
+        norm_bits = tq_gload2(job.vec_norms + slot);
     };
-    if (tile < n_tiles) issue_loads(tile);
 
-    while (tile < n_tiles) {
-        uint32_t cur[NW];
-#pragma unroll
-        for (int i = 0; i < NW; ++i) cur[i] = raw[i];
-        const float nrm = half_bits_to_float(norm_bits);
-        const uint32_t next = tile + tile_stride;
-        if (next < n_tiles) issue_loads(next);
-
+    // one tile: decode + rotate + scale + transpose + store
+    auto process = [&](auto full_tag, auto fast_tag, uint32_t tl, const uint32_t (&cur)[NW], float nrm) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        constexpr bool FAST = decltype(fast_tag)::value;
         // ---- x_hat[64h + 16t + r] = sum_j y[j] * Pi[j][.]   (un-scaled)
         tq_f16v acc[TQ_TILES];
 #pragma unroll
@@ -150,17 +182,71 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
                     *reinterpret_cast<tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ n) << 4)) = o;
                 }
         }
+        tq_u4 val[NSTORE];
 #pragma unroll
         for (int j = 0; j < NSTORE; ++j) {
             const uint32_t vl = j * VEC_PER_STORE + st_vec;
             const uint32_t swz = (ELEM == 2) ? (vl & 15u) : vl;
-            const tq_u4 o = *reinterpret_cast<const tq_u4 *>(stage + vl * VEC_BYTES + ((st_piece ^ swz) << 4));
-            const uint32_t v = tile * 32u + vl;
-            if (v < job.n_vec)
-                tq_gstore16(out_base + tq_vec_offset(job, v) + st_piece * 16u, o);
+            val[j] = *reinterpret_cast<const tq_u4 *>(stage + vl * VEC_BYTES + ((st_piece ^ swz) << 4));
         }
-        tile = next;
-    }
+        if constexpr (FAST) {
+            const Origin o = origin_of(tl);
+            uint8_t *base = out_base + o.out_base;
+#pragma unroll
+            for (int j = 0; j < NSTORE; ++j) {
+                const uint32_t vl = j * VEC_PER_STORE + st_vec;
+                if (FULL || tl * 32u + vl < job.n_vec)
+                    tq_gstore16(base + st_off[j] + (vl >= o.in_row ? row_wrap : 0ll), val[j]);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NSTORE; ++j) {
+                const uint32_t vl = j * VEC_PER_STORE + st_vec;
+                if (FULL || tl * 32u + vl < job.n_vec)
+                    tq_gstore16(out_base + tq_vec_offset(job, tl * 32u + vl) + st_piece * 16u, val[j]);
+            }
+        }
+    };
+
+    // Tiles whose 32 vectors all exist: the loads of the next tile are always issued (past the end: the
+    // current tile again, never used) and nothing is predicated, so loads -> stores -> wait for the loads
+    // leaves the stores in flight (s_waitcnt vmcnt(#stores)) instead of draining them every iteration.
+    const uint32_t n_full = job.n_vec / 32u;
+    auto run = [&](auto fast_tag) {
+        if (tile < n_full) {
+            uint32_t cur[NW];
+            issue_loads(std::true_type{}, fast_tag, tile);
+#pragma unroll
+            for (int i = 0; i < NW; ++i) cur[i] = raw[i];
+            float nrm = half_bits_to_float(norm_bits);
+            while (tile < n_full) {
+                const uint32_t next = tile + tile_stride;
+                issue_loads(std::true_type{}, fast_tag, next < n_full ? next : tile);
+                asm volatile("" ::: "memory");          // the prefetch stays ahead of the tile's work
+                process(std::true_type{}, fast_tag, tile, cur, nrm);
+                // take the prefetched registers here, behind the stores: the wait for them then sits inside
+                // the loop body, where the number of younger stores is known
+#pragma unroll
+                for (int i = 0; i < NW; ++i) {
+                    asm volatile("" : "+v"(raw[i]));
+                    cur[i] = raw[i];
+                }
+                uint32_t nb = norm_bits;
+                asm volatile("" : "+v"(nb));
+                nrm = half_bits_to_float((uint16_t)nb);
+                tile = next;
+            }
+        }
+        // the partial last tile of the job, for the wave whose turn it is
+        if (tile == n_full && n_full < n_tiles) {
+            issue_loads(std::false_type{}, fast_tag, tile);
+            uint32_t cur[NW];
+#pragma unroll
+            for (int i = 0; i < NW; ++i) cur[i] = raw[i];
+            process(std::false_type{}, fast_tag, tile, cur, half_bits_to_float(norm_bits));
+        }
+    };
+    if (fast) run(std::true_type{}); else run(std::false_type{});
 }
 
 // ---- host side --------------------------------------------------------------------------
