@@ -181,6 +181,22 @@ int tq_weighted_values(const uint8_t *idx_bytes, const uint16_t *vec_norms, long
                        const float *weights, long long weights_stride, int group,
                        float *partial, int splits, float *out_rot, void *stream);
 
+/*
+ * The same attention in one pass over the packed keys and values (scores, softmax statistics and the
+ * weighted value sums never leave the chip): for every (row, split of the token range, query head g)
+ *   partial[((r * splits + s) * group + g) * 130 + {0, 1, 2..129}] =
+ *       { m = largest score of the split,  sum_t exp(score_t - m),  sum_t exp(score_t - m) * norm_t * centroid[code(t, j)] }
+ * with score_t as tq_scores computes it (q_rot carries the softmax scale).  The caller merges the splits
+ * (and any uncompressed tokens) by the usual log-sum-exp rule and multiplies the 128 sums by Pi of the value
+ * codec.  Keys and values share rows, tokens and packed_row_stride; group <= 8.  Same replaced reference
+ * lines as tq_scores / tq_weighted_values.  tq_attend_splits suggests a split count.
+ */
+int tq_attend_splits(long long rows, long long tokens);
+int tq_attend_partials(const uint8_t *k_idx, const uint16_t *k_norms, const uint8_t *v_idx, const uint16_t *v_norms,
+                       long long packed_row_stride, long long rows, long long tokens,
+                       const void *table_k, const void *table_v, int head_dim, int bits_k, int bits_v,
+                       const float *q_rot, int group, int splits, float *partial, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

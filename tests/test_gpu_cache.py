@@ -244,6 +244,8 @@ def test_v3cache_attend_equals_attention_over_the_cache(pkg, oracle, rw, dtype):
                 q = (4 * torch.randn(B, H * G, 1, D, generator=g)).to(dtype).to(DEV)
                 out = b.attend(q, l)
                 assert out.shape == (B, H * G, 1, D) and out.dtype == dtype
+                three = b.attend(q, l, fused=False)              # scores / softmax / weighted values as separate steps
+                assert float((out.float() - three.float()).norm() / three.float().norm()) < 4e-3
                 tq = b._get_compressor(l, D, DEV)
                 kw, vw = sb.window()
                 parts_k, parts_v = [], []
@@ -265,3 +267,41 @@ def test_v3cache_attend_equals_attention_over_the_cache(pkg, oracle, rw, dtype):
         seen += n_new
     with pytest.raises(ValueError):
         b.attend(torch.zeros(B, H * G, 2, D, device=DEV), 0)
+
+
+@pytest.mark.parametrize("kb,vb,G,S", [(4, 2, 4, 1500), (8, 8, 8, 200), (2, 4, 1, 77), (3, 1, 2, 640), (6, 2, 8, 33)])
+def test_fused_attention_partials_against_oracle(pkg, oracle, kb, vb, G, S):
+    """The one-pass kernel (scores, online softmax, weighted values per split) merged by the log-sum-exp rule
+    equals float64 attention over the oracle-decoded packed keys and values."""
+    B, H, D = 2, 3, 128
+    kc = pkg.MSECompressor(D, kb, seed=11 + kb, device=DEV)
+    vc = pkg.MSECompressor(D, vb, seed=511 + vb, device=DEV)
+    keys = outlier_kv((B, H, S, D), seed=kb * 100 + S, dtype=torch.bfloat16).to(DEV)
+    vals = outlier_kv((B, H, S, D), seed=vb * 100 + S + 1, dtype=torch.bfloat16).to(DEV)
+    cap = S + 24
+    k_idx = torch.zeros(B, H, cap, D // (8 // kb), dtype=torch.uint8, device=DEV)
+    v_idx = torch.zeros(B, H, cap, D // (8 // vb), dtype=torch.uint8, device=DEV)
+    k_nrm = torch.zeros(B, H, cap, dtype=torch.float16, device=DEV)
+    v_nrm = torch.zeros(B, H, cap, dtype=torch.float16, device=DEV)
+    kc.compress_into(keys, k_idx[:, :, :S], k_nrm[:, :, :S])
+    vc.compress_into(vals, v_idx[:, :, :S], v_nrm[:, :, :S])
+    g = torch.Generator(device="cpu")
+    g.manual_seed(S)
+    q = (3 * torch.randn(B, H * G, D, generator=g) * torch.exp(0.5 * torch.randn(B, H * G, 1, generator=g))).to(DEV)
+    q[0, 0] = 0                                              # a zero query: uniform attention
+    scale = D ** -0.5
+    q_rot = torch.matmul(q, kc.Pi.T) * scale
+    part = torch.ops.tqamd.attend_partials(k_idx[:, :, :S], k_nrm[:, :, :S], v_idx[:, :, :S], v_nrm[:, :, :S],
+                                           kc.table(), vc.table(), kb, vb, q_rot)
+    assert part.shape[:2] == (B, H * G) and part.shape[3] == D + 2
+    m_s, l_s, a_s = part[..., 0], part[..., 1], part[..., 2:]
+    m_all = m_s.amax(dim=-1, keepdim=True)
+    f = torch.exp(m_s - m_all)
+    got = (torch.matmul((f.unsqueeze(-1) * a_s).sum(2), vc.Pi) / (f * l_s).sum(-1, keepdim=True)).cpu().numpy()
+    k_hat = _oracle_decode(oracle, kc, k_idx[:, :, :S], k_nrm[:, :, :S], (B, H, S, D))
+    v_hat = _oracle_decode(oracle, vc, v_idx[:, :, :S], v_nrm[:, :, :S], (B, H, S, D))
+    ref_scores, ref = oracle.attention_decode(q.cpu().numpy(), k_hat, v_hat, scale)
+    err = np.linalg.norm(got - ref) / np.linalg.norm(ref)
+    assert np.abs(m_all.squeeze(-1).cpu().numpy() - ref_scores.max(-1)).max() < 1e-3 * np.abs(ref_scores).max() + 1e-6
+    print(f"[fused attention] K{kb} V{vb} G{G} S{S}: relative L2 error {err:.2e}")
+    assert err < 2e-3

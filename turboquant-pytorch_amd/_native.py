@@ -87,7 +87,7 @@ EXPORTS = (
     "tq_abi_version", "tq_status_string", "tq_device_count", "tq_bytes_per_vector",
     "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_quantize_host",
     "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched",
-    "tq_scores", "tq_weighted_values", "tq_weighted_values_splits",
+    "tq_scores", "tq_weighted_values", "tq_weighted_values_splits", "tq_attend_partials", "tq_attend_splits",
 )
 
 _lib = None
@@ -119,6 +119,8 @@ def lib() -> ctypes.CDLL:
     L.tq_compress_batched.argtypes = [vp, vp, ci, ci, vp]
     L.tq_scores.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, vp, ll, vp]
     L.tq_weighted_values_splits.argtypes = [ll, ll]
+    L.tq_attend_splits.argtypes = [ll, ll]
+    L.tq_attend_partials.argtypes = [vp, vp, vp, vp, ll, ll, ll, vp, vp, ci, ci, ci, vp, ci, ci, vp, vp]
     L.tq_weighted_values.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ll, ci, vp, ci, vp, vp]
     L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp]
     for name in EXPORTS:
@@ -421,6 +423,38 @@ def weighted_values_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: 
 @weighted_values_op.register_fake
 def _(idx_bytes, vec_norms, table, bits, weights, head_dim):
     return weights.new_empty((weights.shape[0], weights.shape[1], head_dim), dtype=torch.float32)
+
+
+@torch.library.custom_op("tqamd::attend_partials", mutates_args=(), device_types="cuda")
+def attend_partials_op(k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.Tensor, v_norms: torch.Tensor,
+                       table_k: torch.Tensor, table_v: torch.Tensor, bits_k: int, bits_v: int,
+                       q_rot: torch.Tensor) -> torch.Tensor:
+    """One pass over packed keys and values of a [B,H,S,..] store pair: per (batch, query head, split)
+    [largest score, sum of exp, 128 weighted sums in the value codec's rotated space] -> [B, Hq, splits, 130]."""
+    _require_gpu(k_idx, "k_idx")
+    prs_k = packed_row_stride(k_idx, k_norms)
+    prs_v = packed_row_stride(v_idx, v_norms)
+    if prs_k is None or prs_v is None or prs_k != prs_v:
+        k_idx, k_norms, v_idx, v_norms = k_idx.contiguous(), k_norms.contiguous(), v_idx.contiguous(), v_norms.contiguous()
+        prs_k = 0
+    B, H, S, _ = k_idx.shape
+    Bq, Hq, D = q_rot.shape
+    group = Hq // H
+    q_rot = q_rot.to(torch.float32).contiguous()
+    L = lib()
+    splits = L.tq_attend_splits(B * H, S)
+    part = torch.empty((B, H, splits, group, D + 2), dtype=torch.float32, device=k_idx.device)
+    with torch.cuda.device(k_idx.device):
+        rc = L.tq_attend_partials(k_idx.data_ptr(), k_norms.data_ptr(), v_idx.data_ptr(), v_norms.data_ptr(), prs_k,
+                                  B * H, S, table_k.data_ptr(), table_v.data_ptr(), D, bits_k, bits_v,
+                                  q_rot.data_ptr(), group, splits, part.data_ptr(), _stream_handle(k_idx.device))
+    check(rc, "tq_attend_partials")
+    return part.permute(0, 1, 3, 2, 4).reshape(B, Hq, splits, D + 2)
+
+
+@attend_partials_op.register_fake
+def _(k_idx, k_norms, v_idx, v_norms, table_k, table_v, bits_k, bits_v, q_rot):
+    return q_rot.new_empty((q_rot.shape[0], q_rot.shape[1], 1, q_rot.shape[2] + 2), dtype=torch.float32)
 
 
 # ------------------------------------------------------------------------------------

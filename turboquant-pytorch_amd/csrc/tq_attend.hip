@@ -354,6 +354,307 @@ __global__ __launch_bounds__(256) void tq_reduce_splits_kernel(const float *part
     ((TQ_GLOBAL float *)out)[i] = s;
 }
 
+// ---- one pass over packed keys and values: scores, online softmax, weighted values ------------------------
+struct AttendArgs {
+    const uint8_t *k_idx, *v_idx;
+    const uint16_t *k_norms, *v_norms;
+    const uint8_t *table_k, *table_v;
+    const float *q_rot;      // [rows, group, 128], softmax scale folded in
+    float *partial;          // [rows, splits, group, 130]: largest score, sum of exp(score - largest), 128 weighted sums
+    uint32_t tokens, packed_row_stride, group, chunk;
+};
+constexpr int AT_WAVES = 4;
+constexpr int AT_RUN = 64;       // tokens per wave and trip
+constexpr int AT_PART = TQ_HEAD_DIM + 2;
+
+// Block (split, row), wave = runs of 64 tokens of the split, tile = 32 tokens.  Per tile:
+//   S^T = K_dec * Q~^T on the matrix cores with the decoded keys as the A operand (rows = tokens, the natural
+//     layout of the decode) and the rotated queries as B (columns = query heads), so that lane (g, h) ends up with
+//     the scores of query head g against 16 tokens of the tile: the softmax statistics of a head stay inside two lanes;
+//   online softmax in base 2 (running maximum m, sum l, both per lane; the two lanes of a head agree on m);
+//   the probabilities, already in the lanes that own head g as an MFMA row, become the A operand of
+//     P * V_dec (fp16 of p * 2^14); the tokens of a contraction slice are the ones the score registers hold,
+//     16ks + 8(i/4) + 4h + i%4, and the B operand is built for exactly those tokens the way the weighted-values
+//     kernel builds it (lane (n, h) owns coordinates 4n .. 4n+3, byte lookups + in-lane token-pair permutes, norms
+//     folded in as packed fp16);
+//   when a head's maximum moves, the value accumulators of its row are rescaled (factors passed through LDS).
+// The four waves' (m, l, sums) are merged in LDS; splits and the uncompressed window are merged by the caller.
+// Query heads per row: at most 8.
+template <int IPBK, int IPBV>
+__global__ __launch_bounds__(AT_WAVES *TQ_WAVE, 2) void tq_attend_kernel(AttendArgs a) {
+    constexpr int NBK = 64 / IPBK, NWK = NBK / 4;        // key bytes / dwords per lane (half a vector)
+    constexpr int GBV = TQ_HEAD_DIM / IPBV;              // value bytes per vector
+    constexpr int SUB = AT_RUN / 32;
+    constexpr int VBYTES = AT_RUN * GBV;                 // <= 8192
+    constexpr int VPIECES = VBYTES / 16, NVP = (VPIECES + 63) / 64;
+    constexpr int P_SHIFT = 14;
+    constexpr int AREA = VBYTES > 8 * AT_PART * 4 ? VBYTES : 8 * AT_PART * 4;   // staged value codes, later the wave's result
+    __shared__ __attribute__((aligned(16))) uint8_t lds_lut_k[4096];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_lut_v[4096];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_area[AT_WAVES][AREA];
+    __shared__ __attribute__((aligned(16))) uint16_t lds_kn[AT_WAVES][AT_RUN];
+    __shared__ __attribute__((aligned(16))) uint16_t lds_vn[AT_WAVES][AT_RUN];
+    __shared__ __attribute__((aligned(16))) float lds_corr[AT_WAVES][8];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t row = blockIdx.y, split = blockIdx.x;
+    const uint32_t n = lane & 31u, hk = lane >> 5;
+    const TqTableHeader *hk_hd = reinterpret_cast<const TqTableHeader *>(a.table_k);
+    const TqTableHeader *hv_hd = reinterpret_cast<const TqTableHeader *>(a.table_v);
+    tq_copy_to_lds(lds_lut_k, a.table_k + hk_hd->off_lut, 256u * 2u * IPBK, tid, AT_WAVES * TQ_WAVE);
+    tq_copy_to_lds(lds_lut_v, a.table_v + hv_hd->off_lut, 256u * 2u * IPBV, tid, AT_WAVES * TQ_WAVE);
+
+    const uint32_t G = a.group;
+    const bool live = n < G;
+    // ---- B operand of the score product: query head g = n, contraction slice (s, hk) = coordinates 64hk + 8s + i,
+    //      fp16 hi + lo of q * 2^(10 - e) with e the binary exponent of the head's largest magnitude
+    tq_u4 qhi[TQ_STEPS], qlo[TQ_STEPS];
+    float c1;                // score in base-2 units = t * c1, t = accumulator * key norm
+    float rowscale;          // natural score = t * rowscale
+    {
+        const TQ_GLOBAL float *q = (const TQ_GLOBAL float *)a.q_rot + ((size_t)row * G + (live ? n : 0u)) * TQ_HEAD_DIM + 64u * hk;
+        float big = 0.f;
+        for (int i = 0; i < 64; ++i) big = fmaxf(big, fabsf(q[i]));
+        big = fmaxf(big, __shfl_xor(big, 32));
+        int e = 0;
+        if (big > 0.f && big < __builtin_inff()) (void)frexpf(big, &e);
+        e = e < -100 ? -100 : e;
+        const float up = ldexpf(1.f, TQ_F16_PI_SHIFT - e);
+        rowscale = live ? ldexpf(1.f, e - TQ_F16_PI_SHIFT) : 0.f;
+        c1 = rowscale * 1.44269504088896341f;
+#pragma unroll
+        for (int s = 0; s < TQ_STEPS; ++s) {
+            tq_half8 h, l;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float x = live ? q[8 * s + i] * up : 0.f;
+                const _Float16 xh = (_Float16)x;
+                h[i] = xh;
+                l[i] = (_Float16)(x - (float)xh);
+            }
+            qhi[s] = __builtin_bit_cast(tq_u4, h);
+            qlo[s] = __builtin_bit_cast(tq_u4, l);
+        }
+    }
+    __syncthreads();
+
+    const uint32_t t_begin = split * a.chunk;
+    const uint32_t t_end = min(a.tokens, t_begin + a.chunk);
+    const size_t slot0 = (size_t)row * a.packed_row_stride;
+    uint8_t *vcodes = lds_area[wave];
+
+    tq_f16v acc[TQ_TILES];   // weighted value sums: row = query head, column n of tile c = coordinate 4n + c
+#pragma unroll
+    for (int c = 0; c < TQ_TILES; ++c) acc[c] = tq_zero16();
+    float m_run = -1e30f;    // running maximum of t for this lane's head
+    float l_run = 0.f;       // running sum of p * 2^P_SHIFT over this lane's tokens
+
+    // loads of a run, issued one run ahead
+    uint32_t kraw_next[SUB][NWK];
+    tq_u4 vpiece_next[NVP];
+    uint16_t kn_next = 0, vn_next = 0;
+    auto issue_loads = [&](uint32_t t0) {
+        const uint32_t n_tok = min((uint32_t)AT_RUN, t_end - t0);
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) {
+            const uint32_t tl = 32u * u + n;
+            const uint8_t *src = a.k_idx + (slot0 + t0 + (tl < n_tok ? tl : 0u)) * (2 * NBK) + hk * NBK;
+            if constexpr (NWK == 2) {
+                const tq_u2 v = tq_gload8(src);
+                kraw_next[u][0] = v[0]; kraw_next[u][1] = v[1];
+            } else {
+#pragma unroll
+                for (int q = 0; q < NWK / 4; ++q) {
+                    const tq_u4 v = tq_gload16(src + 16 * q);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) kraw_next[u][4 * q + i] = v[i];
+                }
+            }
+        }
+        const uint8_t *vsrc = a.v_idx + (slot0 + t0) * GBV;
+#pragma unroll
+        for (int p = 0; p < NVP; ++p) {
+            const uint32_t piece = p * 64u + lane;
+            const bool ok = piece < VPIECES && piece * 16u < n_tok * GBV;
+            vpiece_next[p] = tq_gload16(vsrc + (ok ? piece : 0u) * 16u);
+        }
+        kn_next = lane < n_tok ? tq_gload2(a.k_norms + slot0 + t0 + lane) : (uint16_t)0;
+        vn_next = lane < n_tok ? tq_gload2(a.v_norms + slot0 + t0 + lane) : (uint16_t)0;   // tokens past the end weigh nothing
+    };
+    uint32_t t0 = t_begin + AT_RUN * wave;
+    if (t0 < t_end) issue_loads(t0);
+    while (t0 < t_end) {
+        const uint32_t n_tok = min((uint32_t)AT_RUN, t_end - t0);
+        uint32_t kraw[SUB][NWK];
+#pragma unroll
+        for (int u = 0; u < SUB; ++u)
+#pragma unroll
+            for (int i = 0; i < NWK; ++i) kraw[u][i] = kraw_next[u][i];
+#pragma unroll
+        for (int p = 0; p < NVP; ++p) {
+            const uint32_t piece = p * 64u + lane;
+            if (piece < VPIECES) *reinterpret_cast<tq_u4 *>(vcodes + piece * 16u) = vpiece_next[p];
+        }
+        lds_kn[wave][lane] = kn_next;
+        lds_vn[wave][lane] = vn_next;
+        const uint32_t t_next = t0 + AT_RUN * AT_WAVES;
+        if (t_next < t_end) issue_loads(t_next);
+        asm volatile("" ::: "memory");    // staged with one access width, read back with others (LDS serves a wave in order)
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) {
+            if (32u * u >= n_tok) break;  // uniform
+            // ---- scores: lane (g, hk) gets tokens 8*(r/4) + 4*hk + r%4 of the tile in register r
+            tq_f16v sc = tq_zero16();
+#pragma unroll
+            for (int s = 0; s < TQ_STEPS; ++s) {
+                const tq_half8 kd = __builtin_bit_cast(tq_half8, decode_step<IPBK, NWK>(kraw[u], s, lds_lut_k));
+                sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kd, __builtin_bit_cast(tq_half8, qhi[s]), sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kd, __builtin_bit_cast(tq_half8, qlo[s]), sc, 0, 0, 0);
+            }
+            float t[16];
+            float tmax = -1e30f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const tq_u2 kn4 = *reinterpret_cast<const tq_u2 *>(&lds_kn[wave][32u * u + 8u * j + 4u * hk]);
+                // (whole-vector cast: casting single 32-bit elements of a vector to fp16 pairs miscompiles)
+                typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+                const half4 k4 = __builtin_bit_cast(half4, kn4);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) t[4 * j + q] = sc[4 * j + q] * (float)k4[q];
+            }
+            const bool partial_tile = 32u * u + 32u > n_tok;   // uniform
+            if (partial_tile) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    if (32u * u + 8u * (r / 4) + 4u * hk + (r % 4) >= n_tok) t[r] = -1e30f;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, t[r]);
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+            const float m_new = fmaxf(m_run, tmax);
+            const float corr = __builtin_amdgcn_exp2f((m_run - m_new) * c1);
+            const float bias = P_SHIFT - m_new * c1;
+            float ps[16];
+            float lsum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                ps[r] = __builtin_amdgcn_exp2f(fmaf(t[r], c1, bias));     // p * 2^P_SHIFT
+                lsum += ps[r];
+            }
+            if (partial_tile) {       // a zero query makes every exponent 0: masked tokens need an explicit zero
+                lsum = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    if (32u * u + 8u * (r / 4) + 4u * hk + (r % 4) >= n_tok) ps[r] = 0.f;
+                    lsum += ps[r];
+                }
+            }
+            l_run = l_run * corr + lsum;
+            // ---- the head's maximum moved: rescale the value sums of its row
+            if (__any(m_new != m_run)) {
+                if (hk == 0u && n < 8u) lds_corr[wave][n] = corr;
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_wave_barrier();
+                const float4 c4 = *reinterpret_cast<const float4 *>(&lds_corr[wave][4u * hk]);
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int c = 0; c < TQ_TILES; ++c) {
+                    acc[c][0] *= c4.x; acc[c][1] *= c4.y; acc[c][2] *= c4.z; acc[c][3] *= c4.w;
+                }
+            }
+            m_run = m_new;
+            // ---- P * V for the tile: contraction slices ks, tokens 16ks + 8(i/4) + 4hk + i%4
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                tq_half8 pa;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) pa[i] = (_Float16)ps[8 * ks + i];
+                const uint32_t tl0 = 32u * u + 16u * ks + 4u * hk;
+                const tq_u2 vn_a = *reinterpret_cast<const tq_u2 *>(&lds_vn[wave][tl0]);        // tokens tl0 .. tl0+3
+                const tq_u2 vn_b = *reinterpret_cast<const tq_u2 *>(&lds_vn[wave][tl0 + 8u]);   // tokens tl0+8 .. tl0+11
+                const tq_u4 nrm = {vn_a[0], vn_a[1], vn_b[0], vn_b[1]};
+                uint32_t lo[8], hi[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint8_t *tok = vcodes + (tl0 + 8u * (i / 4) + (i % 4)) * GBV;
+                    if constexpr (IPBV == 8) {
+                        const uint32_t b = tok[n >> 1];
+                        const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lds_lut_v + b * 16u + (n & 1u) * 8u);
+                        lo[i] = v[0]; hi[i] = v[1];
+                    } else if constexpr (IPBV == 4) {
+                        const uint32_t b = tok[n];
+                        const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lds_lut_v + b * 8u);
+                        lo[i] = v[0]; hi[i] = v[1];
+                    } else if constexpr (IPBV == 2) {
+                        const uint32_t two = *reinterpret_cast<const uint16_t *>(tok + 2u * n);
+                        lo[i] = *reinterpret_cast<const uint32_t *>(lds_lut_v + (two & 0xffu) * 4u);
+                        hi[i] = *reinterpret_cast<const uint32_t *>(lds_lut_v + (two >> 8) * 4u);
+                    } else {
+                        const uint32_t four = *reinterpret_cast<const uint32_t *>(tok + 4u * n);
+                        const uint32_t c0 = *reinterpret_cast<const uint16_t *>(lds_lut_v + (four & 0xffu) * 2u);
+                        const uint32_t c1v = *reinterpret_cast<const uint16_t *>(lds_lut_v + ((four >> 8) & 0xffu) * 2u);
+                        const uint32_t c2 = *reinterpret_cast<const uint16_t *>(lds_lut_v + ((four >> 16) & 0xffu) * 2u);
+                        const uint32_t c3 = *reinterpret_cast<const uint16_t *>(lds_lut_v + (four >> 24) * 2u);
+                        lo[i] = c0 | (c1v << 16); hi[i] = c2 | (c3 << 16);
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < TQ_TILES; ++c) {
+                    tq_u4 bt;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const uint32_t even = c < 2 ? lo[2 * d] : hi[2 * d], odd = c < 2 ? lo[2 * d + 1] : hi[2 * d + 1];
+                        bt[d] = __builtin_amdgcn_perm(odd, even, (c & 1) ? 0x07060302u : 0x05040100u);
+                    }
+                    const tq_half8 y = __builtin_bit_cast(tq_half8, bt) * __builtin_bit_cast(tq_half8, nrm);
+                    acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(pa, y, acc[c], 0, 0, 0);
+                }
+            }
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        t0 = t_next;
+    }
+    asm volatile("" ::: "memory");
+    // ---- this wave's result for heads 0..7: [head][largest natural score, sum, 128 sums] in its LDS area
+    float *res = reinterpret_cast<float *>(lds_area[wave]);
+    {
+        const float l_all = (l_run + __shfl_xor(l_run, 32)) * (1.0f / (float)(1 << P_SHIFT));
+        if (hk == 0u && n < 8u) {
+            res[n * AT_PART + 0] = m_run * rowscale;
+            res[n * AT_PART + 1] = l_all;
+        }
+#pragma unroll
+        for (int c = 0; c < TQ_TILES; ++c)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                res[(4u * hk + r) * AT_PART + 2 + 4u * n + c] = acc[c][r] * (1.0f / (float)(1 << P_SHIFT));
+    }
+    __syncthreads();
+    // ---- merge the four waves
+    float *dst = a.partial + ((size_t)row * gridDim.x + split) * G * AT_PART;
+    for (uint32_t i = tid; i < G * AT_PART; i += AT_WAVES * TQ_WAVE) {
+        const uint32_t g = i / AT_PART, j = i % AT_PART;
+        float mw[AT_WAVES], mall = -3.0e38f;
+#pragma unroll
+        for (int w = 0; w < AT_WAVES; ++w) {
+            mw[w] = reinterpret_cast<const float *>(lds_area[w])[g * AT_PART];
+            mall = fmaxf(mall, mw[w]);
+        }
+        float out;
+        if (j == 0) {
+            out = mall;
+        } else {
+            out = 0.f;
+#pragma unroll
+            for (int w = 0; w < AT_WAVES; ++w)
+                out += __expf(mw[w] - mall) * reinterpret_cast<const float *>(lds_area[w])[g * AT_PART + j];
+        }
+        ((TQ_GLOBAL float *)dst)[i] = out;
+    }
+}
+
 int device_cus(int &cus) {
     static int cache[64] = {};
     int dev = 0;
@@ -477,4 +778,61 @@ extern "C" int tq_weighted_values(const uint8_t *idx_bytes, const uint16_t *vec_
     if (rc) return rc;
     hipLaunchKernelGGL(tq_reduce_splits_kernel, dim3((total + 255) / 256), dim3(256), 0, s, partial, out_rot, per_row, (uint32_t)splits, total);
     return (int)hipGetLastError();
+}
+
+namespace {
+template <int IPBK>
+int launch_attend(int ipbv, dim3 grid, dim3 block, hipStream_t s, const AttendArgs &a) {
+    switch (ipbv) {
+        case 8: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 8>), grid, block, 0, s, a); break;
+        case 4: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 4>), grid, block, 0, s, a); break;
+        case 2: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 2>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 1>), grid, block, 0, s, a); break;
+    }
+    return (int)hipGetLastError();
+}
+}  // namespace
+
+extern "C" int tq_attend_splits(long long rows, long long tokens) {
+    if (rows <= 0 || tokens <= 0) return 1;
+    int cus = 0;
+    if (device_cus(cus)) cus = 256;
+    long long splits = ((long long)cus * 4 + rows - 1) / rows;       // two resident four-wave blocks per compute unit, twice over
+    const long long most = (tokens + AT_RUN * AT_WAVES - 1) / (AT_RUN * AT_WAVES);
+    if (splits > most) splits = most;
+    if (splits > 4096) splits = 4096;
+    return splits < 1 ? 1 : (int)splits;
+}
+
+extern "C" int tq_attend_partials(const uint8_t *k_idx, const uint16_t *k_norms, const uint8_t *v_idx, const uint16_t *v_norms,
+                                  long long packed_row_stride, long long rows, long long tokens,
+                                  const void *table_k, const void *table_v, int head_dim, int bits_k, int bits_v,
+                                  const float *q_rot, int group, int splits, float *partial, void *stream) {
+    int rc = check_packed(k_idx, k_norms, packed_row_stride, rows, tokens, table_k, head_dim, bits_k);
+    if (rc) return rc;
+    rc = check_packed(v_idx, v_norms, packed_row_stride, rows, tokens, table_v, head_dim, bits_v);
+    if (rc) return rc;
+    if (group < 1 || group > 8 || splits < 1 || splits > 65535) return TQ_ERR_SIZE;
+    if (rows == 0 || tokens == 0) return TQ_ERR_SIZE;          // nothing to attend to: the caller handles it
+    if (!q_rot || !partial) return TQ_ERR_NULL;
+    if (((uintptr_t)q_rot & 3u) || ((uintptr_t)partial & 3u)) return TQ_ERR_ALIGN;
+    AttendArgs a;
+    a.k_idx = k_idx; a.v_idx = v_idx; a.k_norms = k_norms; a.v_norms = v_norms;
+    a.table_k = static_cast<const uint8_t *>(table_k);
+    a.table_v = static_cast<const uint8_t *>(table_v);
+    a.q_rot = q_rot;
+    a.partial = partial;
+    a.tokens = (uint32_t)tokens;
+    a.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
+    a.group = (uint32_t)group;
+    const long long per_split = (tokens + splits - 1) / splits;
+    a.chunk = (uint32_t)((per_split + AT_RUN - 1) / AT_RUN * AT_RUN);
+    dim3 grid((unsigned)splits, (unsigned)rows, 1), block(AT_WAVES * TQ_WAVE, 1, 1);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (8 / bits_k) {
+        case 8: return launch_attend<8>(8 / bits_v, grid, block, s, a);
+        case 4: return launch_attend<4>(8 / bits_v, grid, block, s, a);
+        case 2: return launch_attend<2>(8 / bits_v, grid, block, s, a);
+        default: return launch_attend<1>(8 / bits_v, grid, block, s, a);
+    }
 }

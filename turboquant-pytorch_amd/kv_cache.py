@@ -196,12 +196,14 @@ class V3Cache:
         self._push(self._store(key_states, layer_idx), key_states, value_states)
 
     @torch.no_grad()
-    def attend(self, query_states: torch.Tensor, layer_idx: int, scale: Optional[float] = None) -> torch.Tensor:
+    def attend(self, query_states: torch.Tensor, layer_idx: int, scale: Optional[float] = None,
+               fused: Optional[bool] = None) -> torch.Tensor:
         """softmax(scale * q K^T) V of one query token per sequence, [B,Hq,1,D] -> [B,Hq,1,D], over everything
         cached for the layer -- what the model computes from the tensors `update` returns -- read
-        straight from the packed store: scores from the packed keys (query rotated once), softmax in
-        float32, the weighted sum of the packed values in the rotated space, window tokens as they are.
-        Query head j uses kv head j // (Hq / H)."""
+        straight from the packed store.  Query head j uses kv head j // (Hq / H).
+        fused (default: whenever at most 8 query heads share a kv head): one kernel pass over packed keys and
+        values with an online softmax per split of the history; otherwise three steps (scores from the packed
+        keys, softmax in float32, weighted sum of the packed values).  Window tokens are used as they are."""
         st = self._stores[layer_idx]
         B, Hq, Sq, D = query_states.shape
         if Sq != 1 or B != st.B or Hq % st.H:
@@ -210,6 +212,33 @@ class V3Cache:
         scale = D ** -0.5 if scale is None else scale
         n_c, n_w = st.n_compressed, st.n_recent
         kc, vc = st.comp.key_compressor, st.comp.val_compressor
+        if fused is None:
+            fused = G <= 8
+        q4 = query_states.reshape(B, st.H, G, D).to(torch.float32)
+        kw, vw = st.window()
+        if fused and n_c:
+            q_rot = torch.matmul(query_states.reshape(B, Hq, D).to(torch.float32), kc.Pi.T) * scale
+            part = torch.ops.tqamd.attend_partials(st.k_idx[:, :, :n_c], st.k_nrm[:, :, :n_c], st.v_idx[:, :, :n_c],
+                                                   st.v_nrm[:, :, :n_c], kc.table(), vc.table(), kc.bits, vc.bits, q_rot)
+            m_s, l_s, a_s = part[..., 0], part[..., 1], part[..., 2:]          # [B,Hq,splits], .., [B,Hq,splits,D]
+            if n_w:
+                s_w = (torch.matmul(q4, kw.to(torch.float32).transpose(-2, -1)) * scale).reshape(B, Hq, n_w)
+                m_w = s_w.amax(dim=-1)
+                p_w = torch.exp(s_w - m_w.unsqueeze(-1))
+                l_w = p_w.sum(dim=-1)
+                a_w = torch.matmul(p_w.reshape(B, st.H, G, n_w), vw.to(torch.float32)).reshape(B, Hq, D)
+                m_all = torch.maximum(m_s.amax(dim=-1), m_w)
+            else:
+                m_all = m_s.amax(dim=-1)
+            f_s = torch.exp(m_s - m_all.unsqueeze(-1))                          # log-sum-exp merge of the splits
+            num = torch.matmul((f_s.unsqueeze(-1) * a_s).sum(dim=2), vc.Pi)    # rotate the value sums back once
+            den = (f_s * l_s).sum(dim=-1)
+            if n_w:
+                f_w = torch.exp(m_w - m_all)
+                num = num + f_w.unsqueeze(-1) * a_w
+                den = den + f_w * l_w
+            out = num / den.unsqueeze(-1)
+            return out.to(query_states.dtype).reshape(B, Hq, 1, D)
         # rows padded to a multiple of 8 floats (the kernels read weights with 16-byte loads); the padding
         # scores are -inf, so the softmax runs over the whole contiguous buffer
         total = n_c + n_w
@@ -219,16 +248,12 @@ class V3Cache:
             scores[:, :, total:] = float("-inf")
         if n_c:
             kc.packed_scores(st.k_idx[:, :, :n_c], st.k_nrm[:, :, :n_c], query_states, scale, out=scores[:, :, :n_c])
-        q4 = query_states.reshape(B, st.H, G, D).to(torch.float32)
-        kw, vw = st.window()
         if n_w:
-            kw = kw.to(torch.float32)
-            scores[:, :, n_c:total] = (torch.matmul(q4, kw.transpose(-2, -1)) * scale).reshape(B, Hq, n_w)
+            scores[:, :, n_c:total] = (torch.matmul(q4, kw.to(torch.float32).transpose(-2, -1)) * scale).reshape(B, Hq, n_w)
         probs = torch.softmax(scores, dim=-1)
         out = vc.packed_weighted_values(st.v_idx[:, :, :n_c], st.v_nrm[:, :, :n_c], probs[:, :, :n_c])
         if n_w:
-            vw = vw.to(torch.float32)
-            out = out + torch.matmul(probs[:, :, n_c:total].reshape(B, st.H, G, n_w), vw).reshape(B, Hq, D)
+            out = out + torch.matmul(probs[:, :, n_c:total].reshape(B, st.H, G, n_w), vw.to(torch.float32)).reshape(B, Hq, D)
         return out.to(query_states.dtype).reshape(B, Hq, 1, D)
 
     def get_seq_length(self, layer_idx: int = 0) -> int:
