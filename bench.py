@@ -230,41 +230,44 @@ def main():
     order = sorted(groups)
     torch.cuda.synchronize()
 
-    def step(events=None):
-        for b in order:
-            if events is not None:
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-            comp_lists[b].compress()
-            if events is not None:
-                e1.record()
-                events.setdefault(("compress", b), []).append((e0, e1))
-        for b in order:
-            if events is not None:
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-            deco_lists[b].decompress()
-            if events is not None:
-                e1.record()
-                events.setdefault(("decompress", b), []).append((e0, e1))
+    launches = [("compress", b) for b in order] + [("decompress", b) for b in order]
 
+    def step(evs=None):
+        """One pass over the cache.  `evs`: pre-created (start, stop) event pairs, one per launch."""
+        for i, (direction, b) in enumerate(launches):
+            if evs is not None:
+                evs[i][0].record()
+            (comp_lists[b].compress if direction == "compress" else deco_lists[b].decompress)()
+            if evs is not None:
+                evs[i][1].record()
+
+    # HIP events are created (and recorded once, which is what allocates them) before the timed region
+    step_events = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in launches]
+                   for _ in range(args.steps)]
     for _ in range(args.warmup):
         step()
+    for evs in step_events:
+        for e0, e1 in evs:
+            e0.record()
+            e1.record()
     torch.cuda.synchronize()
 
     # ---- timed region: exactly `steps` steps ----------------------------------------------------
-    events = {}
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     start.record()
-    for _ in range(args.steps):
-        step(events)
+    for k in range(args.steps):
+        step(step_events[k])
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     gpu_ms = start.elapsed_time(stop)
     ms_per_step = wall * 1000.0 / args.steps
+    events = {}
+    for evs in step_events:
+        for launch, pair in zip(launches, evs):
+            events.setdefault(launch, []).append(pair)
 
     # ---- sanity: what was timed is a real round trip ----------------------------------------------
     j = groups[order[0]][0]
