@@ -192,6 +192,23 @@ int tq_weighted_values(const uint8_t *idx_bytes, const uint16_t *vec_norms, long
  * lines as tq_scores / tq_weighted_values.  tq_attend_splits suggests a split count.
  */
 int tq_attend_splits(long long rows, long long tokens);
+/*
+ * The two small ends of such a decode step, so that a layer costs three launches:
+ *   tq_attend_prepare  q_rot[r][g] = scale * Pi_k q[r][g]  for the one query token of every head ([rows, group, 128]
+ *                      elements of q_dtype), and the same {largest score, sum of exp, 128 weighted value sums} record
+ *                      over the n_win (<= 512) uncompressed window tokens of every row (row r, token t at element
+ *                      r * win_stride + t * 128 of k_win / v_win; plain, un-rotated space) -> part_w [rows, group, 130];
+ *   tq_attend_merge    log-sum-exp merge of the splits' records (tq_attend_partials) and of the window's, rotation
+ *                      of the packed part back by Pi_v, normalisation, cast -> out [rows, group, 128].
+ * pi_k_t: device copy of the key codec's rotation, transposed (float32 [128,128], element [i][j] = Pi[j][i]);
+ * pi_v: the value codec's rotation as MSECompressor keeps it (float32 [128,128] row-major).
+ * k_win / v_win are 16-byte aligned and win_stride is a multiple of 8 (TQ_ERR_ALIGN otherwise).
+ */
+int tq_attend_prepare(const void *queries, int q_dtype, long long rows, int group, float scale,
+                      const float *pi_k_t, const void *k_win, const void *v_win, int win_dtype,
+                      long long n_win, long long win_stride, float *q_rot, float *part_w, void *stream);
+int tq_attend_merge(const float *partial, int splits, const float *part_w, const float *pi_v,
+                    long long rows, int group, void *out, int out_dtype, void *stream);
 int tq_attend_partials(const uint8_t *k_idx, const uint16_t *k_norms, const uint8_t *v_idx, const uint16_t *v_norms,
                        long long packed_row_stride, long long rows, long long tokens,
                        const void *table_k, const void *table_v, int head_dim, int bits_k, int bits_v,

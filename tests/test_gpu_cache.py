@@ -305,3 +305,23 @@ def test_fused_attention_partials_against_oracle(pkg, oracle, kb, vb, G, S):
     assert np.abs(m_all.squeeze(-1).cpu().numpy() - ref_scores.max(-1)).max() < 1e-3 * np.abs(ref_scores).max() + 1e-6
     print(f"[fused attention] K{kb} V{vb} G{G} S{S}: relative L2 error {err:.2e}")
     assert err < 2e-3
+
+
+def test_attend_with_window_only_and_without_window(pkg, oracle):
+    """Decode-step attention when nothing is compressed yet (window tokens only) and when there is no window."""
+    B, H, G, D = 2, 2, 4, 128
+    for rw, n in ((128, 50), (0, 90)):
+        cache = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=rw, n_layers=1)
+        k = outlier_kv((B, H, n, D), seed=800 + rw, dtype=torch.bfloat16).to(DEV)
+        v = outlier_kv((B, H, n, D), seed=801 + rw, dtype=torch.bfloat16).to(DEV)
+        fk, fv = cache.update(k, v, 0)
+        g = torch.Generator(device="cpu")
+        g.manual_seed(rw)
+        q = (2 * torch.randn(B, H * G, 1, D, generator=g)).to(torch.bfloat16).to(DEV)
+        out = cache.attend(q, 0)
+        ref = torch.nn.functional.scaled_dot_product_attention(
+            q.float(), fk.float().repeat_interleave(G, dim=1), fv.float().repeat_interleave(G, dim=1))
+        err = float((out.float() - ref).norm() / ref.norm())
+        print(f"[attend] rw={rw}, {n} tokens: vs attention over update() tensors {err:.2e}")
+        assert out.shape == q.shape and err < (4e-3 if rw else 2e-2)
+        assert float((out.float() - cache.attend(q, 0, fused=False).float()).norm() / ref.norm()) < 4e-3

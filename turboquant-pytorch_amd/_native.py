@@ -88,6 +88,7 @@ EXPORTS = (
     "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_quantize_host",
     "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched",
     "tq_scores", "tq_weighted_values", "tq_weighted_values_splits", "tq_attend_partials", "tq_attend_splits",
+    "tq_attend_prepare", "tq_attend_merge",
 )
 
 _lib = None
@@ -120,6 +121,8 @@ def lib() -> ctypes.CDLL:
     L.tq_scores.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, vp, ll, vp]
     L.tq_weighted_values_splits.argtypes = [ll, ll]
     L.tq_attend_splits.argtypes = [ll, ll]
+    L.tq_attend_prepare.argtypes = [vp, ci, ll, ci, ctypes.c_float, vp, vp, vp, ci, ll, ll, vp, vp, vp]
+    L.tq_attend_merge.argtypes = [vp, ci, vp, vp, ll, ci, vp, ci, vp]
     L.tq_attend_partials.argtypes = [vp, vp, vp, vp, ll, ll, ll, vp, vp, ci, ci, ci, vp, ci, ci, vp, vp]
     L.tq_weighted_values.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ll, ci, vp, ci, vp, vp]
     L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp]
@@ -455,6 +458,66 @@ def attend_partials_op(k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.
 @attend_partials_op.register_fake
 def _(k_idx, k_norms, v_idx, v_norms, table_k, table_v, bits_k, bits_v, q_rot):
     return q_rot.new_empty((q_rot.shape[0], q_rot.shape[1], 1, q_rot.shape[2] + 2), dtype=torch.float32)
+
+
+@torch.library.custom_op("tqamd::attend_packed", mutates_args=(), device_types="cuda")
+def attend_packed_op(queries: torch.Tensor, k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.Tensor,
+                     v_norms: torch.Tensor, table_k: torch.Tensor, table_v: torch.Tensor, bits_k: int, bits_v: int,
+                     pi_k_t: torch.Tensor, pi_v: torch.Tensor, k_win: torch.Tensor, v_win: torch.Tensor,
+                     scale: float) -> torch.Tensor:
+    """Decode-step attention of queries [B,Hq,1,D] over a packed history ([B,H,S,..] store slices, S may be 0)
+    plus uncompressed window tokens [B,H,n_w,D] (n_w may be 0, not both): three launches."""
+    _require_gpu(queries, "queries")
+    B, Hq, _, D = queries.shape
+    H = k_idx.shape[1]
+    S = k_idx.shape[2]
+    n_w = k_win.shape[2]
+    group = Hq // H
+    rows = B * H
+    dev = queries.device
+    q = queries.contiguous()
+    pi_k_t, pi_v = pi_k_t.contiguous(), pi_v.contiguous()       # copies only if the caller kept a strided view
+    L = lib()
+    stream = _stream_handle(dev)
+    q_rot = torch.empty((B, Hq, D), dtype=torch.float32, device=dev)
+    part_w = torch.empty((rows, group, D + 2), dtype=torch.float32, device=dev) if n_w else None
+    win_stride = 0
+    if n_w:
+        lay_k, lay_v = row_layout(k_win), row_layout(v_win)
+        if (lay_k is None or lay_v is None or lay_k != lay_v or lay_k[3] != D or k_win.dtype != v_win.dtype
+                or lay_k[2] % 8 or k_win.data_ptr() % 16 or v_win.data_ptr() % 16):
+            k_win, v_win = k_win.contiguous(), v_win.contiguous()
+            lay_k = row_layout(k_win)
+        win_stride = lay_k[2] if rows > 1 else n_w * D
+    out = torch.empty((B, Hq, 1, D), dtype=queries.dtype, device=dev)
+    with torch.cuda.device(dev):
+        rc = L.tq_attend_prepare(q.data_ptr(), dtype_code(q.dtype), rows, group, scale, pi_k_t.data_ptr(),
+                                 k_win.data_ptr() if n_w else None, v_win.data_ptr() if n_w else None,
+                                 dtype_code(k_win.dtype) if n_w else 0, n_w, win_stride, q_rot.data_ptr(),
+                                 part_w.data_ptr() if n_w else None, stream)
+        check(rc, "tq_attend_prepare")
+        splits = 0
+        part = None
+        if S:
+            prs_k, prs_v = packed_row_stride(k_idx, k_norms), packed_row_stride(v_idx, v_norms)
+            if prs_k is None or prs_v is None or prs_k != prs_v:
+                k_idx, k_norms, v_idx, v_norms = k_idx.contiguous(), k_norms.contiguous(), v_idx.contiguous(), v_norms.contiguous()
+                prs_k = 0
+            splits = L.tq_attend_splits(rows, S)
+            part = torch.empty((rows, splits, group, D + 2), dtype=torch.float32, device=dev)
+            rc = L.tq_attend_partials(k_idx.data_ptr(), k_norms.data_ptr(), v_idx.data_ptr(), v_norms.data_ptr(), prs_k,
+                                      rows, S, table_k.data_ptr(), table_v.data_ptr(), D, bits_k, bits_v,
+                                      q_rot.data_ptr(), group, splits, part.data_ptr(), stream)
+            check(rc, "tq_attend_partials")
+        rc = L.tq_attend_merge(part.data_ptr() if S else None, splits, part_w.data_ptr() if n_w else None, pi_v.data_ptr(),
+                               rows, group, out.data_ptr(), dtype_code(out.dtype), stream)
+        check(rc, "tq_attend_merge")
+    return out
+
+
+@attend_packed_op.register_fake
+def _(queries, k_idx, k_norms, v_idx, v_norms, table_k, table_v, bits_k, bits_v, pi_k_t, pi_v, k_win, v_win, scale):
+    return torch.empty_like(queries)
 
 
 # ------------------------------------------------------------------------------------

@@ -52,7 +52,7 @@ class MSECompressor:
 
         pi_host = _cached_rotation(head_dim, seed)
         cent_host = _cached_centroids(head_dim, bits)
-        self.Pi = pi_host.to(device)
+        self.Pi = pi_host.to(device).contiguous()      # row-major in memory: the kernels take its address
         self.centroids = cent_host.to(device)
         # Everything the kernels read, baked once: split rotation tiles, quantiser grid, decode tables.
         # (above 8 bits the reference constructs fine and fails in compress(); keep that order)
@@ -67,11 +67,18 @@ class MSECompressor:
         self.head_dim = Pi.shape[0]
         self.bits = bits
         self.device = device
-        self.Pi = Pi.to(device=device, dtype=torch.float32)
+        self.Pi = Pi.to(device=device, dtype=torch.float32).contiguous()
         self.centroids = centroids.to(device=device, dtype=torch.float32)
         self._table_host = _native.build_table(Pi, centroids, bits)
         self._table = None
         return self
+
+    def pi_transposed(self) -> torch.Tensor:
+        """Pi^T as its own contiguous tensor (made on first use): the decode-step kernels read it row by row."""
+        t = getattr(self, "_pi_t", None)
+        if t is None:
+            t = self._pi_t = self.Pi.t().contiguous()
+        return t
 
     def table(self) -> torch.Tensor:
         """Device copy of the codec table (uploaded on first use)."""

@@ -655,6 +655,236 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, 2) void tq_attend_kernel(AttendA
     }
 }
 
+// ---- the small ends of a decode step: query rotation + uncompressed window, and the final merge -----------
+struct PrepareArgs {
+    const void *queries;     // [rows, group, 128] elements of q_dtype (one query token), contiguous
+    const float *pi_k_t;     // [128, 128] transposed rotation of the key codec: element [i][j] = Pi[j][i]
+    const void *k_win, *v_win;   // window keys / values: row r, token t at element r * win_stride + t * 128
+    float *q_rot;            // out: [rows, group, 128] = scale * Pi q
+    float *part_w;           // out: [rows, group, 130]: largest window score, sum of exp, 128 weighted value sums
+    long long win_stride;
+    float scale;
+    uint32_t group, n_win;
+    int q_dtype, win_dtype;
+};
+
+__device__ __forceinline__ float tq_load_elem(const void *base, size_t i, int dtype) {
+    if (dtype == TQ_F32) return ((const TQ_GLOBAL float *)base)[i];
+    const uint16_t b = ((const TQ_GLOBAL uint16_t *)base)[i];
+    if (dtype == TQ_F16) return (float)__builtin_bit_cast(_Float16, b);
+    return __uint_as_float((uint32_t)b << 16);
+}
+
+// Eight consecutive window elements starting at element index i (a multiple of 8) as floats.
+template <int WD>
+__device__ __forceinline__ void tq_load8(const void *base, size_t i, float (&x)[8]) {
+    if constexpr (WD == TQ_F32) {
+        const tq_u4 lo = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL float *)base + i);
+        const tq_u4 hi = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL float *)base + i + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { x[e] = __uint_as_float(lo[e]); x[4 + e] = __uint_as_float(hi[e]); }
+    } else {
+        const tq_u4 u = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL uint16_t *)base + i);
+        if constexpr (WD == TQ_F16) {
+            const tq_half8 h = __builtin_bit_cast(tq_half8, u);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = (float)h[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { x[2 * e] = __uint_as_float(u[e] << 16); x[2 * e + 1] = __uint_as_float(u[e] & 0xffff0000u); }
+        }
+    }
+}
+
+// Two consecutive window elements starting at element index i (even).
+template <int WD>
+__device__ __forceinline__ void tq_load2(const void *base, size_t i, float &x0, float &x1) {
+    if constexpr (WD == TQ_F32) {
+        const tq_u2 u = *reinterpret_cast<const TQ_GLOBAL tq_u2 *>((const TQ_GLOBAL float *)base + i);
+        x0 = __uint_as_float(u[0]); x1 = __uint_as_float(u[1]);
+    } else {
+        const uint32_t u = *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint16_t *)base + i);
+        if constexpr (WD == TQ_F16) {
+            const tq_half2 h = __builtin_bit_cast(tq_half2, u);
+            x0 = (float)h[0]; x1 = (float)h[1];
+        } else {
+            x0 = __uint_as_float(u << 16); x1 = __uint_as_float(u & 0xffff0000u);
+        }
+    }
+}
+
+// One block per packed row (batch x kv head), four waves.  Rotates the row's query heads for the packed keys and
+// computes attention statistics over the uncompressed window tokens in fp32 (a few hundred tokens at most).
+//   rotation   : thread (j, half) sums 64 of the 128 terms of every head's q_rot[j]; Pi^T is read once, coalesced
+//   scores     : 16 lanes x 16 bytes cover one token, a wave takes four tokens per load; sums meet over 16 lanes
+//   statistics : wave w owns heads w and w + 4
+//   value sums : thread (column pair, wave) over every fourth token, the four waves' sums meet in LDS
+template <int WD>
+__global__ __launch_bounds__(256) void tq_attend_prepare_kernel(PrepareArgs a) {
+    constexpr int MAXG = 8, MAXW = 512;
+    __shared__ float q[MAXG][TQ_HEAD_DIM];
+    __shared__ float sc[MAXG][MAXW];
+    __shared__ float red[MAXG][2];
+    __shared__ float part[4][MAXG][TQ_HEAD_DIM];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x, G = a.group, lane = tid & 63u, wave = tid >> 6;
+    for (uint32_t i = tid; i < MAXG * TQ_HEAD_DIM; i += 256u)
+        q[i / TQ_HEAD_DIM][i % TQ_HEAD_DIM] =
+            i < G * TQ_HEAD_DIM ? tq_load_elem(a.queries, (size_t)row * G * TQ_HEAD_DIM + i, a.q_dtype) * a.scale : 0.f;
+    __syncthreads();
+    {   // rotated queries: q_rot[g][j] = sum_i Pi[j][i] * q[g][i]
+        const uint32_t j = tid & 127u, half = tid >> 7;
+        const TQ_GLOBAL float *pc = (const TQ_GLOBAL float *)a.pi_k_t + (size_t)half * 64u * TQ_HEAD_DIM + j;
+        float s[MAXG];
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) s[g] = 0.f;
+#pragma unroll 8
+        for (int i = 0; i < 64; ++i) {
+            const float p = pc[(size_t)i * TQ_HEAD_DIM];
+#pragma unroll
+            for (int g = 0; g < MAXG; ++g) s[g] = fmaf(p, q[g][half * 64u + i], s[g]);
+        }
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) part[half][g][j] = s[g];
+    }
+    __syncthreads();
+    for (uint32_t o = tid; o < G * TQ_HEAD_DIM; o += 256u)
+        ((TQ_GLOBAL float *)a.q_rot)[(size_t)row * G * TQ_HEAD_DIM + o] =
+            part[0][o / TQ_HEAD_DIM][o % TQ_HEAD_DIM] + part[1][o / TQ_HEAD_DIM][o % TQ_HEAD_DIM];
+    if (!a.part_w) return;
+    const uint32_t W = a.n_win;
+    const size_t win_base = (size_t)row * a.win_stride;
+    {   // scores of the window tokens
+        const uint32_t sub = lane & 15u, tk = lane >> 4;
+        float qq[MAXG][8];
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qq[g][e] = q[g][8u * sub + e];
+        for (uint32_t t0 = 4u * wave; t0 < W; t0 += 16u) {
+            const uint32_t t = t0 + tk;
+            float x[8];
+            if (t < W) {
+                tq_load8<WD>(a.k_win, win_base + (size_t)t * TQ_HEAD_DIM + 8u * sub, x);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = 0.f;
+            }
+#pragma unroll
+            for (int g = 0; g < MAXG; ++g) {
+                if ((uint32_t)g < G) {           // uniform over the block
+                    float sg = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sg = fmaf(x[e], qq[g][e], sg);
+                    sg += __shfl_xor(sg, 1);
+                    sg += __shfl_xor(sg, 2);
+                    sg += __shfl_xor(sg, 4);
+                    sg += __shfl_xor(sg, 8);
+                    if (sub == 0u && t < W) sc[g][t] = sg;
+                }
+            }
+        }
+    }
+    __syncthreads();                      // (the value sums below reuse `part`: every q_rot read of it is behind us)
+    for (uint32_t g = wave; g < G; g += 4u) {
+        float m = -3.0e38f;
+        for (uint32_t t = lane; t < W; t += 64u) m = fmaxf(m, sc[g][t]);
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d));
+        float l = 0.f;
+        for (uint32_t t = lane; t < W; t += 64u) {
+            const float p = __expf(sc[g][t] - m);
+            sc[g][t] = p;
+            l += p;
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) l += __shfl_xor(l, d);
+        if (lane == 0u) { red[g][0] = m; red[g][1] = l; }
+    }
+    __syncthreads();
+    {   // weighted value sums: this thread's two columns over tokens wave, wave + 4, ...
+        float acc[MAXG][2];
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) acc[g][0] = acc[g][1] = 0.f;
+#pragma unroll 4
+        for (uint32_t t = wave; t < W; t += 4u) {
+            float x0, x1;
+            tq_load2<WD>(a.v_win, win_base + (size_t)t * TQ_HEAD_DIM + 2u * lane, x0, x1);
+#pragma unroll
+            for (int g = 0; g < MAXG; ++g) {
+                if ((uint32_t)g < G) {
+                    const float p = sc[g][t];
+                    acc[g][0] = fmaf(p, x0, acc[g][0]);
+                    acc[g][1] = fmaf(p, x1, acc[g][1]);
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) { part[wave][g][2u * lane] = acc[g][0]; part[wave][g][2u * lane + 1u] = acc[g][1]; }
+    }
+    __syncthreads();
+    float *out = a.part_w + (size_t)row * G * AT_PART;
+    for (uint32_t o = tid; o < G * AT_PART; o += 256u) {
+        const uint32_t g = o / AT_PART, j = o % AT_PART;
+        ((TQ_GLOBAL float *)out)[o] = j < 2u ? red[g][j] : part[0][g][j - 2u] + part[1][g][j - 2u] + part[2][g][j - 2u] + part[3][g][j - 2u];
+    }
+}
+
+struct MergeArgs {
+    const float *partial;    // [rows, splits, group, 130] from the packed history (rotated value space)
+    const float *part_w;     // [rows, group, 130] from the window (plain space) or NULL
+    const float *pi_v;       // [128, 128] rotation of the value codec
+    void *out;               // [rows, group, 128] elements of out_dtype
+    uint32_t group, splits;
+    int out_dtype;
+};
+
+// One block per packed row: log-sum-exp merge of the splits, rotation of the value sums back (x = y @ Pi),
+// the window's share, normalisation, cast.
+__global__ __launch_bounds__(256) void tq_attend_merge_kernel(MergeArgs a) {
+    constexpr int MAXG = 8;
+    __shared__ float rot[MAXG][TQ_HEAD_DIM];
+    __shared__ float den[MAXG], fw[MAXG];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x, G = a.group, S = a.splits;
+    const TQ_GLOBAL float *part = (const TQ_GLOBAL float *)a.partial + (size_t)row * S * G * AT_PART;
+    const TQ_GLOBAL float *pw = a.part_w ? (const TQ_GLOBAL float *)a.part_w + (size_t)row * G * AT_PART : nullptr;
+    for (uint32_t o = tid; o < G * TQ_HEAD_DIM; o += 256u) {
+        const uint32_t g = o / TQ_HEAD_DIM, j = o % TQ_HEAD_DIM;
+        float m = pw ? pw[g * AT_PART] : -3.0e38f;
+        for (uint32_t s = 0; s < S; ++s) m = fmaxf(m, part[(s * G + g) * AT_PART]);
+        float acc = 0.f, l = 0.f;
+        for (uint32_t s = 0; s < S; ++s) {
+            const TQ_GLOBAL float *ps = part + (s * G + g) * AT_PART;
+            const float f = __expf(ps[0] - m);
+            acc = fmaf(f, ps[2 + j], acc);
+            l = fmaf(f, ps[1], l);
+        }
+        rot[g][j] = acc;
+        if (j == 0) {
+            const float f = pw ? __expf(pw[g * AT_PART] - m) : 0.f;
+            fw[g] = f;
+            den[g] = l + (pw ? f * pw[g * AT_PART + 1] : 0.f);
+        }
+    }
+    __syncthreads();
+    for (uint32_t o = tid; o < G * TQ_HEAD_DIM; o += 256u) {
+        const uint32_t g = o / TQ_HEAD_DIM, i = o % TQ_HEAD_DIM;
+        float x = 0.f;
+        for (int j = 0; j < TQ_HEAD_DIM; ++j) x = fmaf(rot[g][j], ((const TQ_GLOBAL float *)a.pi_v)[(size_t)j * TQ_HEAD_DIM + i], x);
+        if (pw) x = fmaf(fw[g], pw[g * AT_PART + 2 + i], x);
+        x /= den[g];
+        const size_t idx = (size_t)row * G * TQ_HEAD_DIM + o;
+        if (a.out_dtype == TQ_F32) {
+            ((TQ_GLOBAL float *)a.out)[idx] = x;
+        } else if (a.out_dtype == TQ_F16) {
+            const _Float16 h = (_Float16)x;
+            ((TQ_GLOBAL uint16_t *)a.out)[idx] = __builtin_bit_cast(uint16_t, h);
+        } else {
+            const __bf16 h = (__bf16)x;
+            ((TQ_GLOBAL uint16_t *)a.out)[idx] = __builtin_bit_cast(uint16_t, h);
+        }
+    }
+}
+
 int device_cus(int &cus) {
     static int cache[64] = {};
     int dev = 0;
@@ -835,4 +1065,42 @@ extern "C" int tq_attend_partials(const uint8_t *k_idx, const uint16_t *k_norms,
         case 2: return launch_attend<2>(8 / bits_v, grid, block, s, a);
         default: return launch_attend<1>(8 / bits_v, grid, block, s, a);
     }
+}
+
+extern "C" int tq_attend_prepare(const void *queries, int q_dtype, long long rows, int group, float scale,
+                                 const float *pi_k_t, const void *k_win, const void *v_win, int win_dtype,
+                                 long long n_win, long long win_stride, float *q_rot, float *part_w, void *stream) {
+    if (rows < 0 || rows > 0x7fffffff || group < 1 || group > 8 || n_win < 0 || n_win > 512) return TQ_ERR_SIZE;
+    if ((q_dtype != TQ_F32 && q_dtype != TQ_F16 && q_dtype != TQ_BF16) ||
+        (n_win && win_dtype != TQ_F32 && win_dtype != TQ_F16 && win_dtype != TQ_BF16)) return TQ_ERR_DTYPE;
+    if (rows == 0) return TQ_OK;
+    if (!queries || !pi_k_t || !q_rot) return TQ_ERR_NULL;
+    if (n_win && (!k_win || !v_win || !part_w)) return TQ_ERR_NULL;
+    if (n_win && win_stride < n_win * TQ_HEAD_DIM) return TQ_ERR_SIZE;
+    // window tokens are read with 16-byte loads
+    if (n_win && (((uintptr_t)k_win & 15u) || ((uintptr_t)v_win & 15u) || (win_stride & 7))) return TQ_ERR_ALIGN;
+    PrepareArgs a;
+    a.queries = queries; a.pi_k_t = pi_k_t; a.k_win = k_win; a.v_win = v_win;
+    a.q_rot = q_rot; a.part_w = n_win ? part_w : nullptr;
+    a.win_stride = win_stride; a.scale = scale;
+    a.group = (uint32_t)group; a.n_win = (uint32_t)n_win;
+    a.q_dtype = q_dtype; a.win_dtype = win_dtype;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    if (n_win && win_dtype == TQ_F32) hipLaunchKernelGGL(tq_attend_prepare_kernel<TQ_F32>, dim3((unsigned)rows), dim3(256), 0, st, a);
+    else if (n_win && win_dtype == TQ_F16) hipLaunchKernelGGL(tq_attend_prepare_kernel<TQ_F16>, dim3((unsigned)rows), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(tq_attend_prepare_kernel<TQ_BF16>, dim3((unsigned)rows), dim3(256), 0, st, a);
+    return (int)hipGetLastError();
+}
+
+extern "C" int tq_attend_merge(const float *partial, int splits, const float *part_w, const float *pi_v,
+                               long long rows, int group, void *out, int out_dtype, void *stream) {
+    if (rows < 0 || rows > 0x7fffffff || group < 1 || group > 8 || splits < 0) return TQ_ERR_SIZE;
+    if (out_dtype != TQ_F32 && out_dtype != TQ_F16 && out_dtype != TQ_BF16) return TQ_ERR_DTYPE;
+    if (rows == 0) return TQ_OK;
+    if (!pi_v || !out || (splits && !partial) || (!splits && !part_w)) return TQ_ERR_NULL;
+    MergeArgs a;
+    a.partial = partial; a.part_w = part_w; a.pi_v = pi_v; a.out = out;
+    a.group = (uint32_t)group; a.splits = (uint32_t)splits; a.out_dtype = out_dtype;
+    hipLaunchKernelGGL(tq_attend_merge_kernel, dim3((unsigned)rows), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+    return (int)hipGetLastError();
 }

@@ -216,29 +216,17 @@ class V3Cache:
             fused = G <= 8
         q4 = query_states.reshape(B, st.H, G, D).to(torch.float32)
         kw, vw = st.window()
-        if fused and n_c:
-            q_rot = torch.matmul(query_states.reshape(B, Hq, D).to(torch.float32), kc.Pi.T) * scale
-            part = torch.ops.tqamd.attend_partials(st.k_idx[:, :, :n_c], st.k_nrm[:, :, :n_c], st.v_idx[:, :, :n_c],
-                                                   st.v_nrm[:, :, :n_c], kc.table(), vc.table(), kc.bits, vc.bits, q_rot)
-            m_s, l_s, a_s = part[..., 0], part[..., 1], part[..., 2:]          # [B,Hq,splits], .., [B,Hq,splits,D]
-            if n_w:
-                s_w = (torch.matmul(q4, kw.to(torch.float32).transpose(-2, -1)) * scale).reshape(B, Hq, n_w)
-                m_w = s_w.amax(dim=-1)
-                p_w = torch.exp(s_w - m_w.unsqueeze(-1))
-                l_w = p_w.sum(dim=-1)
-                a_w = torch.matmul(p_w.reshape(B, st.H, G, n_w), vw.to(torch.float32)).reshape(B, Hq, D)
-                m_all = torch.maximum(m_s.amax(dim=-1), m_w)
-            else:
-                m_all = m_s.amax(dim=-1)
-            f_s = torch.exp(m_s - m_all.unsqueeze(-1))                          # log-sum-exp merge of the splits
-            num = torch.matmul((f_s.unsqueeze(-1) * a_s).sum(dim=2), vc.Pi)    # rotate the value sums back once
-            den = (f_s * l_s).sum(dim=-1)
-            if n_w:
-                f_w = torch.exp(m_w - m_all)
-                num = num + f_w.unsqueeze(-1) * a_w
-                den = den + f_w * l_w
-            out = num / den.unsqueeze(-1)
-            return out.to(query_states.dtype).reshape(B, Hq, 1, D)
+        if fused and (n_c or n_w) and n_w <= 512:
+            # three launches: rotate the queries + window statistics, one pass over the packed history,
+            # log-sum-exp merge + rotation back + cast
+            if n_c:
+                packed = (st.k_idx[:, :, :n_c], st.k_nrm[:, :, :n_c], st.v_idx[:, :, :n_c], st.v_nrm[:, :, :n_c])
+            else:                                   # nothing has left the window yet: an empty history
+                dev = query_states.device
+                packed = (torch.empty((B, st.H, 0, 1), dtype=torch.uint8, device=dev),
+                          torch.empty((B, st.H, 0), dtype=torch.float16, device=dev)) * 2
+            return torch.ops.tqamd.attend_packed(query_states, *packed, kc.table(), vc.table(),
+                                                 kc.bits, vc.bits, kc.pi_transposed(), vc.Pi, kw, vw, float(scale))
         # rows padded to a multiple of 8 floats (the kernels read weights with 16-byte loads); the padding
         # scores are -inf, so the softmax runs over the whole contiguous buffer
         total = n_c + n_w
@@ -251,7 +239,10 @@ class V3Cache:
         if n_w:
             scores[:, :, n_c:total] = (torch.matmul(q4, kw.to(torch.float32).transpose(-2, -1)) * scale).reshape(B, Hq, n_w)
         probs = torch.softmax(scores, dim=-1)
-        out = vc.packed_weighted_values(st.v_idx[:, :, :n_c], st.v_nrm[:, :, :n_c], probs[:, :, :n_c])
+        if n_c:
+            out = vc.packed_weighted_values(st.v_idx[:, :, :n_c], st.v_nrm[:, :, :n_c], probs[:, :, :n_c])
+        else:
+            out = torch.zeros((B, Hq, D), dtype=torch.float32, device=query_states.device)
         if n_w:
             out = out + torch.matmul(probs[:, :, n_c:total].reshape(B, st.H, G, n_w), vw.to(torch.float32)).reshape(B, Hq, D)
         return out.to(query_states.dtype).reshape(B, Hq, 1, D)
@@ -273,7 +264,8 @@ class V3Cache:
         n = 0
         for st in self._stores.values():
             rows = st.B * st.H
-            n += rows * st.n_compressed * (st.k_idx.shape[-1] + st.v_idx.shape[-1] + 4)
+            if st.n_compressed:
+                n += rows * st.n_compressed * (st.k_idx.shape[-1] + st.v_idx.shape[-1] + 4)
             n += 2 * rows * st.n_recent * st.D * st.k_win.element_size()
         return n
 
