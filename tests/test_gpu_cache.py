@@ -325,3 +325,77 @@ def test_attend_with_window_only_and_without_window(pkg, oracle):
         print(f"[attend] rw={rw}, {n} tokens: vs attention over update() tensors {err:.2e}")
         assert out.shape == q.shape and err < (4e-3 if rw else 2e-2)
         assert float((out.float() - cache.attend(q, 0, fused=False).float()).norm() / ref.norm()) < 4e-3
+
+
+@pytest.mark.parametrize("wdtype,qdtype,G,W,splits", [(torch.bfloat16, torch.bfloat16, 4, 128, 3), (torch.float16, torch.float16, 8, 512, 1),
+                                                      (torch.float32, torch.float32, 1, 37, 2), (torch.bfloat16, torch.float32, 7, 1, 0),
+                                                      (torch.float16, torch.bfloat16, 3, 0, 4)])
+def test_attend_prepare_and_merge_against_float64(pkg, wdtype, qdtype, G, W, splits):
+    """tq_attend_prepare / tq_attend_merge through the C-ABI against the same arithmetic in float64:
+    rotated queries to 1e-5, window records to 1e-5, merged output to the output type's rounding."""
+    nat = pkg._native
+    L = nat.lib()
+    B, H, D, cap = 2, 3, 128, 520
+    rows = B * H
+    g = torch.Generator(device="cpu")
+    g.manual_seed(1000 + G * 7 + W)
+    q = (3 * torch.randn(B, H * G, 1, D, generator=g)).to(qdtype).to(DEV)
+    kbuf = torch.randn(B, H, cap, D, generator=g).to(wdtype).to(DEV)
+    vbuf = torch.randn(B, H, cap, D, generator=g).to(wdtype).to(DEV)
+    kw, vw = kbuf[:, :, 8:8 + W], vbuf[:, :, 8:8 + W]                # token-axis slices of a larger buffer
+    pi_k = pkg.generate_rotation_matrix(D, seed=11).contiguous().to(DEV)
+    pi_v = pkg.generate_rotation_matrix(D, seed=12).contiguous().to(DEV)
+    scale = 0.11
+    q_rot = torch.empty(B, H * G, D, dtype=torch.float32, device=DEV)
+    part_w = torch.full((rows, G, D + 2), float("nan"), dtype=torch.float32, device=DEV)
+    rc = L.tq_attend_prepare(q.data_ptr(), nat.dtype_code(q.dtype), rows, G, scale, pi_k.t().contiguous().data_ptr(),
+                             kw.data_ptr() if W else None, vw.data_ptr() if W else None, nat.dtype_code(wdtype), W, cap * D,
+                             q_rot.data_ptr(), part_w.data_ptr() if W else None, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    q64 = q.double().reshape(B, H, G, D) * scale
+    ref_rot = torch.matmul(q64, pi_k.double().T).reshape(B, H * G, D)
+    assert float((q_rot.double() - ref_rot).norm() / ref_rot.norm()) < 1e-5
+    if W:
+        s = torch.matmul(q64, kw.double().transpose(-2, -1))
+        m = s.amax(-1)
+        p = torch.exp(s - m.unsqueeze(-1))
+        l = p.sum(-1)
+        a = torch.matmul(p, vw.double())
+        pw = part_w.double().reshape(B, H, G, D + 2)
+        assert float((pw[..., 0] - m).abs().max()) < 1e-4 and float(((pw[..., 1] - l) / l).abs().max()) < 1e-5
+        assert float(((pw[..., 2:] - a).norm(dim=-1) / a.norm(dim=-1)).max()) < 1e-5
+    # split records as the one-pass kernel would leave them: random maxima, sums, rotated value sums
+    part = None
+    if splits:
+        part = torch.randn(rows, splits, G, D + 2, generator=g).to(DEV)
+        part[..., 0] = part[..., 0] * 3 + (float(m.mean()) if W else 0.0)
+        part[..., 1] = part[..., 1].abs() + 0.5
+    for odtype in (torch.float32, qdtype):
+        out = torch.empty(B, H * G, 1, D, dtype=odtype, device=DEV)
+        rc = L.tq_attend_merge(part.data_ptr() if splits else None, splits, part_w.data_ptr() if W else None, pi_v.data_ptr(),
+                               rows, G, out.data_ptr(), nat.dtype_code(odtype), None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        m_all = torch.full((rows, G), -float("inf"), dtype=torch.float64, device=DEV)
+        if splits:
+            p64 = part.double()
+            m_all = torch.maximum(m_all, p64[..., 0].amax(dim=1))
+        if W:
+            w64 = part_w.double()
+            m_all = torch.maximum(m_all, w64[..., 0])
+        num = torch.zeros(rows, G, D, dtype=torch.float64, device=DEV)
+        den = torch.zeros(rows, G, dtype=torch.float64, device=DEV)
+        if splits:
+            f = torch.exp(p64[..., 0] - m_all.unsqueeze(1))
+            num = torch.matmul((f.unsqueeze(-1) * p64[..., 2:]).sum(1), pi_v.double())
+            den = (f * p64[..., 1]).sum(1)
+        if W:
+            f = torch.exp(w64[..., 0] - m_all)
+            num = num + f.unsqueeze(-1) * w64[..., 2:]
+            den = den + f * w64[..., 1]
+        ref = (num / den.unsqueeze(-1)).reshape(B, H * G, 1, D)
+        err = float((out.double() - ref).norm() / ref.norm())
+        tol = {torch.float32: 1e-5, torch.float16: 1e-3, torch.bfloat16: 6e-3}[odtype]
+        print(f"[prepare/merge] window {W} x {wdtype}, {G} heads, {splits} splits -> {odtype}: {err:.2e}")
+        assert err < tol
