@@ -11,10 +11,12 @@ from .rotation import generate_rotation_matrix
 from .compressors_v3 import MSECompressor, TurboQuantV3
 from .kv_cache import V3Cache, hf_cache_class
 from .metrics import attention_scores, compute_metrics
+from .serialize import save_cache, load_cache, save_compressed, load_compressed, codec_digest, FormatError
 from . import _native
 
 __all__ = [
     "MSECompressor", "TurboQuantV3", "V3Cache", "hf_cache_class", "attention_scores", "compute_metrics",
     "LloydMaxCodebook", "solve_lloyd_max",
     "generate_rotation_matrix", "_native",
+    "save_cache", "load_cache", "save_compressed", "load_compressed", "codec_digest", "FormatError",
 ]

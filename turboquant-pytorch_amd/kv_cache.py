@@ -259,6 +259,17 @@ class V3Cache:
         total = st.total_seq if st is not None else 0
         return f"{comp} compressed, {total - comp} fp16, {total} total"
 
+    def save(self, path: str, include_codec: bool = True) -> None:
+        """Write configuration, packed history and window of every layer to one safetensors file."""
+        from .serialize import save_cache
+        save_cache(self, path, include_codec=include_codec)
+
+    @classmethod
+    def load(cls, path: str, device="cuda") -> "V3Cache":
+        """A cache in the state `save` wrote: `update` / `append` / `attend` continue from there."""
+        from .serialize import load_cache
+        return load_cache(path, device=device, cls=cls)
+
     def stored_bytes(self) -> int:
         """Bytes held for the tokens seen so far (packed codes, norms, window), over all layers."""
         n = 0
