@@ -272,7 +272,8 @@ def test_v3cache_attend_equals_attention_over_the_cache(pkg, oracle, rw, dtype):
 @pytest.mark.parametrize("kb,vb,G,S", [(4, 2, 4, 1500), (8, 8, 8, 200), (2, 4, 1, 77), (3, 1, 2, 640), (6, 2, 8, 33)])
 def test_fused_attention_partials_against_oracle(pkg, oracle, kb, vb, G, S):
     """The one-pass kernel (scores, online softmax, weighted values per split) merged by the log-sum-exp rule
-    equals float64 attention over the oracle-decoded packed keys and values."""
+    equals float64 attention over the oracle-decoded packed keys and values; its records are consistent
+    (reference score within the documented distance of the largest score, sums taken against it)."""
     B, H, D = 2, 3, 128
     kc = pkg.MSECompressor(D, kb, seed=11 + kb, device=DEV)
     vc = pkg.MSECompressor(D, vb, seed=511 + vb, device=DEV)
@@ -302,9 +303,19 @@ def test_fused_attention_partials_against_oracle(pkg, oracle, kb, vb, G, S):
     v_hat = _oracle_decode(oracle, vc, v_idx[:, :, :S], v_nrm[:, :, :S], (B, H, S, D))
     ref_scores, ref = oracle.attention_decode(q.cpu().numpy(), k_hat, v_hat, scale)
     err = np.linalg.norm(got - ref) / np.linalg.norm(ref)
-    assert np.abs(m_all.squeeze(-1).cpu().numpy() - ref_scores.max(-1)).max() < 1e-3 * np.abs(ref_scores).max() + 1e-6
+    # the record's reference score is at most the largest score and at most 8 binary orders below it ...
+    gap = ref_scores.max(-1) - m_all.squeeze(-1).cpu().numpy()
+    tol = 1e-3 * np.abs(ref_scores).max() + 1e-6
+    assert gap.min() > -tol and gap.max() < 8 * np.log(2.0) + tol
+    # ... and the sum of exponentials is taken against exactly that reference
+    l_got = (f * l_s).sum(-1).cpu().numpy()
+    l_ref = np.exp(ref_scores - m_all.cpu().numpy().astype(np.float64)).sum(-1)
+    # (a score error ds changes exp(score) by the factor e^ds: fp16 keys and queries put ds near 1e-4 of the largest |score|)
+    assert np.abs(l_got / l_ref - 1).max() < 3e-3 + 4e-4 * np.abs(ref_scores).max()
     print(f"[fused attention] K{kb} V{vb} G{G} S{S}: relative L2 error {err:.2e}")
-    assert err < 2e-3
+    # queries and decoded keys enter the score product as fp16 (2^-12 relative per coordinate), probabilities times
+    # value norms as fp16 as well; the queries here are scaled up to logits beyond 100, where that shows most
+    assert err < 3e-3
 
 
 def test_attend_with_window_only_and_without_window(pkg, oracle):

@@ -360,61 +360,129 @@ struct AttendArgs {
     const uint16_t *k_norms, *v_norms;
     const uint8_t *table_k, *table_v;
     const float *q_rot;      // [rows, group, 128], softmax scale folded in
-    float *partial;          // [rows, splits, group, 130]: largest score, sum of exp(score - largest), 128 weighted sums
+    float *partial;          // [rows, splits, group, 130]: reference score m, sum of exp(score - m), 128 weighted sums
     uint32_t tokens, packed_row_stride, group, chunk;
 };
-constexpr int AT_WAVES = 4;
-constexpr int AT_RUN = 64;       // tokens per wave and trip
+constexpr int AT_RUN = 64;       // tokens per wave and trip (32 when keys or values use 8-bit codes)
 constexpr int AT_PART = TQ_HEAD_DIM + 2;
 
-// Block (split, row), wave = runs of 64 tokens of the split, tile = 32 tokens.  Per tile:
-//   S^T = K_dec * Q~^T on the matrix cores with the decoded keys as the A operand (rows = tokens, the natural
-//     layout of the decode) and the rotated queries as B (columns = query heads), so that lane (g, h) ends up with
-//     the scores of query head g against 16 tokens of the tile: the softmax statistics of a head stay inside two lanes;
-//   online softmax in base 2 (running maximum m, sum l, both per lane; the two lanes of a head agree on m);
-//   the probabilities, already in the lanes that own head g as an MFMA row, become the A operand of
-//     P * V_dec (fp16 of p * 2^14); the tokens of a contraction slice are the ones the score registers hold,
-//     16ks + 8(i/4) + 4h + i%4, and the B operand is built for exactly those tokens the way the weighted-values
-//     kernel builds it (lane (n, h) owns coordinates 4n .. 4n+3, byte lookups + in-lane token-pair permutes, norms
-//     folded in as packed fp16);
-//   when a head's maximum moves, the value accumulators of its row are rescaled (factors passed through LDS).
-// The four waves' (m, l, sums) are merged in LDS; splits and the uncompressed window are merged by the caller.
-// Query heads per row: at most 8.
+// Block (split, row) of eight waves; a wave takes runs of 64 tokens of the split (staged one run ahead), a tile is 32
+// tokens = two blocks of 16, all matrix work is v_mfma_f32_16x16x32_f16 with the row's query heads (at most 8) padded
+// to 16 columns.  Lane (n16, q4) = (lane % 16, lane / 16).
+//   scores  S^T[token][head]: A = decoded keys, lane (token n16 of the block, q4) holds the 32 coordinates
+//     32 q4 .. 32 q4 + 31 of its token (KB contiguous packed bytes) and feeds 8 of them to each of 4 steps; B = rotated
+//     queries in the same coordinate order (lane (head n16, q4), step s: coordinates 32 q4 + 8 s + j), one fp16 term;
+//     result register r of lane (head n16, q4) = token 4 q4 + r of the block: a head's statistics live in four lanes;
+//   softmax in base 2 against a per-head reference that follows the running maximum lazily (see m_ref below), so the
+//     common tile needs no exchange between lanes;
+//   P * V_dec: A = probabilities times value norms, lane (head n16, q4) slice j: token 4 q4 + j of block 0 (j < 4) or
+//     block 1, which are the registers the lane already holds; B = decoded values for the same eight tokens, lane
+//     (n16, q4) owns coordinates 8 n16 .. 8 n16 + 7 (8 / IPBV packed bytes per token, one decode), column block c =
+//     coordinate 8 n16 + c; token pairs regrouped with v_perm;
+//     accumulator register r of block c in lane (n16, q4) = head 4 q4 + r, coordinate 8 n16 + c.
+// The waves' (m, l, sums) are merged in LDS; splits and the uncompressed window are merged by the caller.
+typedef float tq_f4v __attribute__((ext_vector_type(4)));
+constexpr int AT_WAVES = 8;      // one block per compute unit (two waves per SIMD): the table copies below are shared by its waves
+
+// The byte -> centroids tables are read with data-dependent addresses by every lane.  With one copy, 64 random
+// addresses over 32 banks serialise several times over (measured: the LDS pipe was busy 70 % of the kernel).  Here
+// every table entry is spread over 128 bytes = one slot per bank group, and a lane always reads the slot of its own
+// banks: entries of 2 or 4 bytes have 32 slots of 4 bytes (lane % 32), 8-byte entries 16 slots (lane % 16: a 64-bit
+// read serves 16 lanes per clock), 16-byte entries 8 slots.  256 entries x 128 bytes = 32 KiB per table.
+template <int IPB>
+struct RepLut {
+    static constexpr int ES = 2 * IPB;                    // bytes per entry
+    static constexpr int SL = ES < 4 ? 4 : ES;            // slot size
+    static constexpr int NC = 128 / SL;                   // copies
+    static __device__ __forceinline__ uint32_t lane_offset(uint32_t lane) { return (lane & (NC - 1)) * SL; }
+    static __device__ __forceinline__ void stage(uint8_t *lds, const uint8_t *src, uint32_t tid, uint32_t nthreads) {
+        for (uint32_t i = tid; i < 256u * NC; i += nthreads) {
+            const uint32_t e = i / NC, c = i % NC;
+            uint8_t *dst = lds + e * 128u + c * SL;
+            const TQ_GLOBAL uint8_t *g = (const TQ_GLOBAL uint8_t *)src + e * ES;
+            if constexpr (ES == 2) *reinterpret_cast<uint16_t *>(dst) = *reinterpret_cast<const TQ_GLOBAL uint16_t *>(g);
+            else if constexpr (ES == 4) *reinterpret_cast<uint32_t *>(dst) = *reinterpret_cast<const TQ_GLOBAL uint32_t *>(g);
+            else if constexpr (ES == 8) *reinterpret_cast<tq_u2 *>(dst) = *reinterpret_cast<const TQ_GLOBAL tq_u2 *>(g);
+            else *reinterpret_cast<tq_u4 *>(dst) = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>(g);
+        }
+    }
+};
+
+// decode_step against a replicated table; `lut` already points at the lane's slot of entry 0
+template <int IPB, int NW>
+__device__ __forceinline__ tq_u4 decode_rep(const uint32_t (&raw)[NW], int s, const uint8_t *lut) {
+    tq_u4 out;
+    if constexpr (IPB == 1) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const uint32_t b0 = (raw[2 * s + (2 * d) / 4] >> (8 * ((2 * d) % 4))) & 0xffu;
+            const uint32_t b1 = (raw[2 * s + (2 * d + 1) / 4] >> (8 * ((2 * d + 1) % 4))) & 0xffu;
+            const uint32_t lo = *reinterpret_cast<const uint16_t *>(lut + (b0 << 7));
+            const uint32_t hi = *reinterpret_cast<const uint16_t *>(lut + (b1 << 7));
+            out[d] = lo | (hi << 16);
+        }
+    } else if constexpr (IPB == 2) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) out[d] = *reinterpret_cast<const uint32_t *>(lut + (((raw[s] >> (8 * d)) & 0xffu) << 7));
+    } else if constexpr (IPB == 4) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t b = (raw[s / 2] >> (16 * (s % 2) + 8 * q)) & 0xffu;
+            const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lut + (b << 7));
+            out[2 * q] = v[0];
+            out[2 * q + 1] = v[1];
+        }
+    } else {
+        const uint32_t b = (raw[s / 4] >> (8 * (s % 4))) & 0xffu;
+        out = *reinterpret_cast<const tq_u4 *>(lut + (b << 7));
+    }
+    return out;
+}
+
 template <int IPBK, int IPBV>
-__global__ __launch_bounds__(AT_WAVES *TQ_WAVE, 2) void tq_attend_kernel(AttendArgs a) {
-    constexpr int NBK = 64 / IPBK, NWK = NBK / 4;        // key bytes / dwords per lane (half a vector)
+__global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_kernel(AttendArgs a) {
+    constexpr int KB = TQ_HEAD_DIM / IPBK / 4;           // key bytes per lane and token (32 coordinates): 4, 8, 16, 32
+    constexpr int NWK = KB / 4;
     constexpr int GBV = TQ_HEAD_DIM / IPBV;              // value bytes per vector
-    constexpr int SUB = AT_RUN / 32;
-    constexpr int VBYTES = AT_RUN * GBV;                 // <= 8192
+    constexpr int VB = 8 / IPBV;                         // value bytes per lane and token (8 coordinates): 1, 2, 4, 8
+    constexpr int NWV = VB > 4 ? 2 : 1;
+    constexpr int RUN = (IPBK == 1 || IPBV == 1) ? 32 : AT_RUN;   // tokens per wave and trip (8-bit codes: half, for registers)
+    constexpr int SUB = RUN / 32;
+    constexpr int VBYTES = RUN * GBV;                 // <= 8192
     constexpr int VPIECES = VBYTES / 16, NVP = (VPIECES + 63) / 64;
-    constexpr int P_SHIFT = 14;
+    constexpr int SLACK_LOG2 = 8;
+    constexpr int P_SHIFT = 14 - SLACK_LOG2;             // p * 2^P_SHIFT * (value norm / 2^ev_ref < 2) <= 2^15 fits fp16
     constexpr int AREA = VBYTES > 8 * AT_PART * 4 ? VBYTES : 8 * AT_PART * 4;   // staged value codes, later the wave's result
-    __shared__ __attribute__((aligned(16))) uint8_t lds_lut_k[4096];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_lut_v[4096];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_lut_k[32768];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_lut_v[32768];
     __shared__ __attribute__((aligned(16))) uint8_t lds_area[AT_WAVES][AREA];
-    __shared__ __attribute__((aligned(16))) uint16_t lds_kn[AT_WAVES][AT_RUN];
-    __shared__ __attribute__((aligned(16))) uint16_t lds_vn[AT_WAVES][AT_RUN];
+    __shared__ __attribute__((aligned(16))) float lds_kn[AT_WAVES][RUN];        // key norms as fp32
+    __shared__ __attribute__((aligned(16))) uint16_t lds_vn[AT_WAVES][RUN];     // value norms / 2^ev_ref as fp16
     __shared__ __attribute__((aligned(16))) float lds_corr[AT_WAVES][8];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t row = blockIdx.y, split = blockIdx.x;
-    const uint32_t n = lane & 31u, hk = lane >> 5;
+    const uint32_t n16 = lane & 15u, q4 = lane >> 4;
     const TqTableHeader *hk_hd = reinterpret_cast<const TqTableHeader *>(a.table_k);
     const TqTableHeader *hv_hd = reinterpret_cast<const TqTableHeader *>(a.table_v);
-    tq_copy_to_lds(lds_lut_k, a.table_k + hk_hd->off_lut, 256u * 2u * IPBK, tid, AT_WAVES * TQ_WAVE);
-    tq_copy_to_lds(lds_lut_v, a.table_v + hv_hd->off_lut, 256u * 2u * IPBV, tid, AT_WAVES * TQ_WAVE);
+    RepLut<IPBK>::stage(lds_lut_k, a.table_k + hk_hd->off_lut, tid, AT_WAVES * TQ_WAVE);
+    RepLut<IPBV>::stage(lds_lut_v, a.table_v + hv_hd->off_lut, tid, AT_WAVES * TQ_WAVE);
+    const uint8_t *lut_k = lds_lut_k + RepLut<IPBK>::lane_offset(lane);
+    const uint8_t *lut_v = lds_lut_v + RepLut<IPBV>::lane_offset(lane);
 
     const uint32_t G = a.group;
-    const bool live = n < G;
-    // ---- B operand of the score product: query head g = n, contraction slice (s, hk) = coordinates 64hk + 8s + i,
-    //      fp16 hi + lo of q * 2^(10 - e) with e the binary exponent of the head's largest magnitude
-    tq_u4 qhi[TQ_STEPS], qlo[TQ_STEPS];
+    const bool live = n16 < G;
+    // ---- B operand of the score product: fp16 of q * 2^(10 - e), e = binary exponent of the head's largest magnitude.
+    //      (One fp16 term: its rounding, 2^-12 relative per coordinate, is what the fp16 centroids of the decoded
+    //      keys already carry.)
+    tq_u4 qb[4];
     float c1;                // score in base-2 units = t * c1, t = accumulator * key norm
     float rowscale;          // natural score = t * rowscale
     {
-        const TQ_GLOBAL float *q = (const TQ_GLOBAL float *)a.q_rot + ((size_t)row * G + (live ? n : 0u)) * TQ_HEAD_DIM + 64u * hk;
+        const TQ_GLOBAL float *q = (const TQ_GLOBAL float *)a.q_rot + ((size_t)row * G + (live ? n16 : 0u)) * TQ_HEAD_DIM + 32u * q4;
         float big = 0.f;
-        for (int i = 0; i < 64; ++i) big = fmaxf(big, fabsf(q[i]));
+        for (int i = 0; i < 32; ++i) big = fmaxf(big, fabsf(q[i]));
+        big = fmaxf(big, __shfl_xor(big, 16));
         big = fmaxf(big, __shfl_xor(big, 32));
         int e = 0;
         if (big > 0.f && big < __builtin_inff()) (void)frexpf(big, &e);
@@ -423,17 +491,11 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, 2) void tq_attend_kernel(AttendA
         rowscale = live ? ldexpf(1.f, e - TQ_F16_PI_SHIFT) : 0.f;
         c1 = rowscale * 1.44269504088896341f;
 #pragma unroll
-        for (int s = 0; s < TQ_STEPS; ++s) {
-            tq_half8 h, l;
+        for (int s = 0; s < 4; ++s) {
+            tq_half8 h;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float x = live ? q[8 * s + i] * up : 0.f;
-                const _Float16 xh = (_Float16)x;
-                h[i] = xh;
-                l[i] = (_Float16)(x - (float)xh);
-            }
-            qhi[s] = __builtin_bit_cast(tq_u4, h);
-            qlo[s] = __builtin_bit_cast(tq_u4, l);
+            for (int i = 0; i < 8; ++i) h[i] = (_Float16)(live ? q[8 * s + i] * up : 0.f);
+            qb[s] = __builtin_bit_cast(tq_u4, h);
         }
     }
     __syncthreads();
@@ -443,34 +505,49 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, 2) void tq_attend_kernel(AttendA
     const size_t slot0 = (size_t)row * a.packed_row_stride;
     uint8_t *vcodes = lds_area[wave];
 
-    tq_f16v acc[TQ_TILES];   // weighted value sums: row = query head, column n of tile c = coordinate 4n + c
+    tq_f4v acc[8];           // weighted value sums: register r = query head 4 q4 + r, block c = coordinate 8 n16 + c
 #pragma unroll
-    for (int c = 0; c < TQ_TILES; ++c) acc[c] = tq_zero16();
-    float m_run = -1e30f;    // running maximum of t for this lane's head
+    for (int c = 0; c < 8; ++c) acc[c] = tq_f4v{0.f, 0.f, 0.f, 0.f};
+    // Softmax reference of this lane's head, in units of t (the four lanes of a head agree).  It is not the exact
+    // running maximum: it moves only when a score exceeds it by more than SLACK_LOG2 binary orders, so the common
+    // tile needs no exchange between lanes; probabilities relative to it reach 2^SLACK_LOG2 at most.
+    float m_ref = -1e30f;
     float l_run = 0.f;       // running sum of p * 2^P_SHIFT over this lane's tokens
+    const float slack = live ? (float)SLACK_LOG2 / c1 : 3.0e38f;
+    // Value norms are folded into the probabilities (A operand), relative to 2^ev_ref, ev_ref = the largest binary
+    // exponent of a value norm seen by this wave so far (uniform over the wave); the sums are in units of 2^ev_ref.
+    int ev_ref = -100;
 
-    // loads of a run, issued one run ahead
-    uint32_t kraw_next[SUB][NWK];
-    tq_u4 vpiece_next[NVP];
-    uint16_t kn_next = 0, vn_next = 0;
-    auto issue_loads = [&](uint32_t t0) {
-        const uint32_t n_tok = min((uint32_t)AT_RUN, t_end - t0);
+    // loads of a run, issued one run ahead into the other of two register sets
+    uint32_t kraw_buf[2][SUB][2][NWK];
+    tq_u4 vpiece_buf[2][NVP];
+    uint16_t kn_buf[2] = {0, 0}, vn_buf[2] = {0, 0};
+    auto issue_loads = [&](auto bsel, uint32_t t0) __attribute__((always_inline)) {
+        constexpr int B = decltype(bsel)::value;
+        auto &kraw_next = kraw_buf[B];
+        auto &vpiece_next = vpiece_buf[B];
+        uint16_t &kn_next = kn_buf[B], &vn_next = vn_buf[B];
+        const uint32_t n_tok = min((uint32_t)RUN, t_end - t0);
 #pragma unroll
-        for (int u = 0; u < SUB; ++u) {
-            const uint32_t tl = 32u * u + n;
-            const uint8_t *src = a.k_idx + (slot0 + t0 + (tl < n_tok ? tl : 0u)) * (2 * NBK) + hk * NBK;
-            if constexpr (NWK == 2) {
-                const tq_u2 v = tq_gload8(src);
-                kraw_next[u][0] = v[0]; kraw_next[u][1] = v[1];
-            } else {
+        for (int u = 0; u < SUB; ++u)
 #pragma unroll
-                for (int q = 0; q < NWK / 4; ++q) {
-                    const tq_u4 v = tq_gload16(src + 16 * q);
+            for (int b = 0; b < 2; ++b) {
+                const uint32_t tl = 32u * u + 16u * b + n16;
+                const uint8_t *src = a.k_idx + (slot0 + t0 + (tl < n_tok ? tl : 0u)) * (4 * KB) + q4 * KB;
+                if constexpr (KB == 4) {
+                    kraw_next[u][b][0] = *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)src);
+                } else if constexpr (KB == 8) {
+                    const tq_u2 v = tq_gload8(src);
+                    kraw_next[u][b][0] = v[0]; kraw_next[u][b][1] = v[1];
+                } else {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) kraw_next[u][4 * q + i] = v[i];
+                    for (int p = 0; p < KB / 16; ++p) {
+                        const tq_u4 v = tq_gload16(src + 16 * p);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) kraw_next[u][b][4 * p + i] = v[i];
+                    }
                 }
             }
-        }
         const uint8_t *vsrc = a.v_idx + (slot0 + t0) * GBV;
 #pragma unroll
         for (int p = 0; p < NVP; ++p) {
@@ -481,158 +558,178 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, 2) void tq_attend_kernel(AttendA
         kn_next = lane < n_tok ? tq_gload2(a.k_norms + slot0 + t0 + lane) : (uint16_t)0;
         vn_next = lane < n_tok ? tq_gload2(a.v_norms + slot0 + t0 + lane) : (uint16_t)0;   // tokens past the end weigh nothing
     };
-    uint32_t t0 = t_begin + AT_RUN * wave;
-    if (t0 < t_end) issue_loads(t0);
-    while (t0 < t_end) {
-        const uint32_t n_tok = min((uint32_t)AT_RUN, t_end - t0);
-        uint32_t kraw[SUB][NWK];
-#pragma unroll
-        for (int u = 0; u < SUB; ++u)
-#pragma unroll
-            for (int i = 0; i < NWK; ++i) kraw[u][i] = kraw_next[u][i];
-#pragma unroll
-        for (int p = 0; p < NVP; ++p) {
-            const uint32_t piece = p * 64u + lane;
-            if (piece < VPIECES) *reinterpret_cast<tq_u4 *>(vcodes + piece * 16u) = vpiece_next[p];
-        }
-        lds_kn[wave][lane] = kn_next;
-        lds_vn[wave][lane] = vn_next;
-        const uint32_t t_next = t0 + AT_RUN * AT_WAVES;
-        if (t_next < t_end) issue_loads(t_next);
-        asm volatile("" ::: "memory");    // staged with one access width, read back with others (LDS serves a wave in order)
-        __builtin_amdgcn_wave_barrier();
+
+    // one run of up to 64 staged tokens; FULL: all 64 exist (no per-token masks in the code).
+    // The score products of both tiles are issued first, so that the second tile's matrix work runs under the
+    // first tile's softmax arithmetic.
+    auto run = [&](auto full_tag, const uint32_t (&kraw)[SUB][2][NWK], uint32_t n_tok) __attribute__((always_inline)) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        tq_f4v sc[SUB][2];   // register r of block b = token 32 u + 16 b + 4 q4 + r
 #pragma unroll
         for (int u = 0; u < SUB; ++u) {
-            if (32u * u >= n_tok) break;  // uniform
-            // ---- scores: lane (g, hk) gets tokens 8*(r/4) + 4*hk + r%4 of the tile in register r
-            tq_f16v sc = tq_zero16();
 #pragma unroll
-            for (int s = 0; s < TQ_STEPS; ++s) {
-                const tq_half8 kd = __builtin_bit_cast(tq_half8, decode_step<IPBK, NWK>(kraw[u], s, lds_lut_k));
-                sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kd, __builtin_bit_cast(tq_half8, qhi[s]), sc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kd, __builtin_bit_cast(tq_half8, qlo[s]), sc, 0, 0, 0);
-            }
-            float t[16];
-            float tmax = -1e30f;
+            for (int b = 0; b < 2; ++b) {
+                sc[u][b] = tq_f4v{0.f, 0.f, 0.f, 0.f};
+                if (!FULL && 32u * u >= n_tok) continue;   // uniform
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const tq_u2 kn4 = *reinterpret_cast<const tq_u2 *>(&lds_kn[wave][32u * u + 8u * j + 4u * hk]);
-                // (whole-vector cast: casting single 32-bit elements of a vector to fp16 pairs miscompiles)
-                typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-                const half4 k4 = __builtin_bit_cast(half4, kn4);
-#pragma unroll
-                for (int q = 0; q < 4; ++q) t[4 * j + q] = sc[4 * j + q] * (float)k4[q];
-            }
-            const bool partial_tile = 32u * u + 32u > n_tok;   // uniform
-            if (partial_tile) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    if (32u * u + 8u * (r / 4) + 4u * hk + (r % 4) >= n_tok) t[r] = -1e30f;
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, t[r]);
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-            const float m_new = fmaxf(m_run, tmax);
-            const float corr = __builtin_amdgcn_exp2f((m_run - m_new) * c1);
-            const float bias = P_SHIFT - m_new * c1;
-            float ps[16];
-            float lsum = 0.f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                ps[r] = __builtin_amdgcn_exp2f(fmaf(t[r], c1, bias));     // p * 2^P_SHIFT
-                lsum += ps[r];
-            }
-            if (partial_tile) {       // a zero query makes every exponent 0: masked tokens need an explicit zero
-                lsum = 0.f;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    if (32u * u + 8u * (r / 4) + 4u * hk + (r % 4) >= n_tok) ps[r] = 0.f;
-                    lsum += ps[r];
+                for (int s = 0; s < 4; ++s) {
+                    const tq_half8 kd = __builtin_bit_cast(tq_half8, decode_rep<IPBK, NWK>(kraw[u][b], s, lut_k));
+                    sc[u][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd, __builtin_bit_cast(tq_half8, qb[s]), sc[u][b], 0, 0, 0);
                 }
             }
-            l_run = l_run * corr + lsum;
-            // ---- the head's maximum moved: rescale the value sums of its row
-            if (__any(m_new != m_run)) {
-                if (hk == 0u && n < 8u) lds_corr[wave][n] = corr;
+        }
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) {
+            if (!FULL && 32u * u >= n_tok) break;  // uniform
+            float t[8];
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const float4 k4 = *reinterpret_cast<const float4 *>(&lds_kn[wave][32u * u + 16u * b + 4u * q4]);
+                t[4 * b + 0] = sc[u][b][0] * k4.x; t[4 * b + 1] = sc[u][b][1] * k4.y;
+                t[4 * b + 2] = sc[u][b][2] * k4.z; t[4 * b + 3] = sc[u][b][3] * k4.w;
+            }
+            if constexpr (!FULL) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (32u * u + 16u * (j / 4) + 4u * q4 + (j % 4) >= n_tok) t[j] = -1e30f;
+            }
+            const float tmax = fmaxf(fmaxf(fmaxf(t[0], t[1]), fmaxf(t[2], t[3])), fmaxf(fmaxf(t[4], t[5]), fmaxf(t[6], t[7])));
+            // ---- a score left the range the reference covers (rare after the first tiles): move the head's
+            //      reference to the largest score seen and rescale its sums
+            if (__any(tmax > m_ref + slack)) {
+                float tm = fmaxf(tmax, __shfl_xor(tmax, 16));
+                tm = fmaxf(tm, __shfl_xor(tm, 32));
+                const float m_new = fmaxf(m_ref, tm);
+                const float corr = __builtin_amdgcn_exp2f((m_ref - m_new) * c1);
+                l_run *= corr;
+                m_ref = m_new;
+                if (q4 == 0u && n16 < 8u) lds_corr[wave][n16] = corr;
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
-                const float4 c4 = *reinterpret_cast<const float4 *>(&lds_corr[wave][4u * hk]);
+                const float4 c4 = *reinterpret_cast<const float4 *>(&lds_corr[wave][4u * (q4 & 1u)]);
                 asm volatile("" ::: "memory");
 #pragma unroll
-                for (int c = 0; c < TQ_TILES; ++c) {
+                for (int c = 0; c < 8; ++c) {
                     acc[c][0] *= c4.x; acc[c][1] *= c4.y; acc[c][2] *= c4.z; acc[c][3] *= c4.w;
                 }
             }
-            m_run = m_new;
-            // ---- P * V for the tile: contraction slices ks, tokens 16ks + 8(i/4) + 4hk + i%4
+            const float bias = P_SHIFT - m_ref * c1;
+            float ps[8];
+            float lsum = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                tq_half8 pa;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) pa[i] = (_Float16)ps[8 * ks + i];
-                const uint32_t tl0 = 32u * u + 16u * ks + 4u * hk;
-                const tq_u2 vn_a = *reinterpret_cast<const tq_u2 *>(&lds_vn[wave][tl0]);        // tokens tl0 .. tl0+3
-                const tq_u2 vn_b = *reinterpret_cast<const tq_u2 *>(&lds_vn[wave][tl0 + 8u]);   // tokens tl0+8 .. tl0+11
-                const tq_u4 nrm = {vn_a[0], vn_a[1], vn_b[0], vn_b[1]};
-                uint32_t lo[8], hi[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const uint8_t *tok = vcodes + (tl0 + 8u * (i / 4) + (i % 4)) * GBV;
-                    if constexpr (IPBV == 8) {
-                        const uint32_t b = tok[n >> 1];
-                        const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lds_lut_v + b * 16u + (n & 1u) * 8u);
-                        lo[i] = v[0]; hi[i] = v[1];
-                    } else if constexpr (IPBV == 4) {
-                        const uint32_t b = tok[n];
-                        const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lds_lut_v + b * 8u);
-                        lo[i] = v[0]; hi[i] = v[1];
-                    } else if constexpr (IPBV == 2) {
-                        const uint32_t two = *reinterpret_cast<const uint16_t *>(tok + 2u * n);
-                        lo[i] = *reinterpret_cast<const uint32_t *>(lds_lut_v + (two & 0xffu) * 4u);
-                        hi[i] = *reinterpret_cast<const uint32_t *>(lds_lut_v + (two >> 8) * 4u);
-                    } else {
-                        const uint32_t four = *reinterpret_cast<const uint32_t *>(tok + 4u * n);
-                        const uint32_t c0 = *reinterpret_cast<const uint16_t *>(lds_lut_v + (four & 0xffu) * 2u);
-                        const uint32_t c1v = *reinterpret_cast<const uint16_t *>(lds_lut_v + ((four >> 8) & 0xffu) * 2u);
-                        const uint32_t c2 = *reinterpret_cast<const uint16_t *>(lds_lut_v + ((four >> 16) & 0xffu) * 2u);
-                        const uint32_t c3 = *reinterpret_cast<const uint16_t *>(lds_lut_v + (four >> 24) * 2u);
-                        lo[i] = c0 | (c1v << 16); hi[i] = c2 | (c3 << 16);
-                    }
+            for (int j = 0; j < 8; ++j) {
+                ps[j] = __builtin_amdgcn_exp2f(fmaf(t[j], c1, bias));     // p * 2^P_SHIFT, p <= 2^SLACK_LOG2
+                if constexpr (!FULL) {   // a zero query makes every exponent 0: masked tokens need an explicit zero
+                    if (32u * u + 16u * (j / 4) + 4u * q4 + (j % 4) >= n_tok) ps[j] = 0.f;
                 }
+                lsum += ps[j];
+            }
+            l_run += lsum;
+            // ---- P * V: contraction slice j of lane (., q4) = token 32 u + 4 q4 + j (j < 4), 32 u + 16 + 4 q4 + j - 4
+            tq_half8 pa;
 #pragma unroll
-                for (int c = 0; c < TQ_TILES; ++c) {
-                    tq_u4 bt;
+            for (int j = 0; j < 8; ++j) pa[j] = (_Float16)ps[j];
+            const uint32_t tok_a = 32u * u + 4u * q4, tok_b = tok_a + 16u;
+            const tq_u2 vn_a = *reinterpret_cast<const tq_u2 *>(&lds_vn[wave][tok_a]);
+            const tq_u2 vn_b = *reinterpret_cast<const tq_u2 *>(&lds_vn[wave][tok_b]);
+            const tq_u4 nrm = {vn_a[0], vn_a[1], vn_b[0], vn_b[1]};
+            pa = pa * __builtin_bit_cast(tq_half8, nrm);          // weight of token j = p_j * |v_j| / 2^ev_ref
+            tq_u4 dec[8];        // per token: the lane's eight coordinates as fp16
 #pragma unroll
-                    for (int d = 0; d < 4; ++d) {
-                        const uint32_t even = c < 2 ? lo[2 * d] : hi[2 * d], odd = c < 2 ? lo[2 * d + 1] : hi[2 * d + 1];
-                        bt[d] = __builtin_amdgcn_perm(odd, even, (c & 1) ? 0x07060302u : 0x05040100u);
-                    }
-                    const tq_half8 y = __builtin_bit_cast(tq_half8, bt) * __builtin_bit_cast(tq_half8, nrm);
-                    acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(pa, y, acc[c], 0, 0, 0);
-                }
+            for (int j = 0; j < 8; ++j) {
+                const uint8_t *src = vcodes + ((j < 4 ? tok_a : tok_b) + (uint32_t)(j % 4)) * GBV + n16 * VB;
+                uint32_t raw[NWV];
+                if constexpr (VB == 1) raw[0] = *src;
+                else if constexpr (VB == 2) raw[0] = *reinterpret_cast<const uint16_t *>(src);
+                else if constexpr (VB == 4) raw[0] = *reinterpret_cast<const uint32_t *>(src);
+                else { const tq_u2 v = *reinterpret_cast<const tq_u2 *>(src); raw[0] = v[0]; raw[1] = v[1]; }
+                dec[j] = decode_rep<IPBV, NWV>(raw, 0, lut_v);
+            }
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                tq_u4 bt;
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    bt[d] = __builtin_amdgcn_perm(dec[2 * d + 1][c / 2], dec[2 * d][c / 2], (c & 1) ? 0x07060302u : 0x05040100u);
+                acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(tq_half8, bt), acc[c], 0, 0, 0);
             }
         }
+    };
+
+    // one trip: stage the run held in register set B, start the loads of the next run into the other set, compute
+    auto trip = [&](auto bsel, uint32_t t0) __attribute__((always_inline)) {
+        constexpr int B = decltype(bsel)::value;
+        const uint32_t n_tok = min((uint32_t)RUN, t_end - t0);
+#pragma unroll
+        for (int p = 0; p < NVP; ++p) {
+            const uint32_t piece = p * 64u + lane;
+            if (piece < VPIECES) *reinterpret_cast<tq_u4 *>(vcodes + piece * 16u) = vpiece_buf[B][p];
+        }
+        {
+            const _Float16 kh = __builtin_bit_cast(_Float16, kn_buf[B]);
+            if (RUN == 64 || lane < (uint32_t)RUN) lds_kn[wave][lane] = (float)kh;     // one token per lane
+            // largest exponent field of the run's value norms: row-wise running maximum, then the four row ends
+            uint32_t e = ((uint32_t)vn_buf[B] >> 10) & 31u;
+            e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x111, 0xf, 0xf, true));
+            e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x112, 0xf, 0xf, true));
+            e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x114, 0xf, 0xf, true));
+            e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x118, 0xf, 0xf, true));
+            const uint32_t emax = max(max((uint32_t)__builtin_amdgcn_readlane((int)e, 15), (uint32_t)__builtin_amdgcn_readlane((int)e, 31)),
+                                      max((uint32_t)__builtin_amdgcn_readlane((int)e, 47), (uint32_t)__builtin_amdgcn_readlane((int)e, 63)));
+            const int ev = (int)max(emax, 1u) - 15;
+            if (ev > ev_ref) {                       // uniform; a handful of times per wave
+                const float f = ldexpf(1.f, ev_ref - ev);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) acc[c] *= f;
+                ev_ref = ev;
+            }
+            const _Float16 vh = __builtin_bit_cast(_Float16, vn_buf[B]);
+            const _Float16 vs = (_Float16)ldexpf((float)vh, -ev_ref);
+            if (RUN == 64 || lane < (uint32_t)RUN) lds_vn[wave][lane] = __builtin_bit_cast(uint16_t, vs);
+        }
+        const uint32_t t_next = t0 + RUN * AT_WAVES;
+        if (t_next < t_end) issue_loads(std::integral_constant<int, 1 - B>{}, t_next);
+        asm volatile("" ::: "memory");    // staged with one access width, read back with others (LDS serves a wave in order)
+        __builtin_amdgcn_wave_barrier();
+        if (n_tok == RUN) run(std::true_type{}, kraw_buf[B], n_tok);
+        else run(std::false_type{}, kraw_buf[B], n_tok);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();
-        t0 = t_next;
+        return t_next;
+    };
+    {
+        uint32_t t0 = t_begin + RUN * wave;
+        if (t0 < t_end) {
+            issue_loads(std::integral_constant<int, 0>{}, t0);
+            for (;;) {
+                t0 = trip(std::integral_constant<int, 0>{}, t0);
+                if (t0 >= t_end) break;
+                t0 = trip(std::integral_constant<int, 1>{}, t0);
+                if (t0 >= t_end) break;
+            }
+        }
     }
     asm volatile("" ::: "memory");
     // ---- this wave's result for heads 0..7: [head][largest natural score, sum, 128 sums] in its LDS area
     float *res = reinterpret_cast<float *>(lds_area[wave]);
     {
-        const float l_all = (l_run + __shfl_xor(l_run, 32)) * (1.0f / (float)(1 << P_SHIFT));
-        if (hk == 0u && n < 8u) {
-            res[n * AT_PART + 0] = m_run * rowscale;
-            res[n * AT_PART + 1] = l_all;
+        float l_all = l_run + __shfl_xor(l_run, 16);
+        l_all = (l_all + __shfl_xor(l_all, 32)) * (1.0f / (float)(1 << P_SHIFT));
+        if (q4 == 0u && n16 < 8u) {
+            res[n16 * AT_PART + 0] = m_ref * rowscale;
+            res[n16 * AT_PART + 1] = l_all;
         }
+        const float out_scale = ldexpf(1.f, ev_ref - P_SHIFT);
+        if (q4 < 2u) {
 #pragma unroll
-        for (int c = 0; c < TQ_TILES; ++c)
+            for (int c = 0; c < 8; ++c)
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                res[(4u * hk + r) * AT_PART + 2 + 4u * n + c] = acc[c][r] * (1.0f / (float)(1 << P_SHIFT));
+                for (int r = 0; r < 4; ++r)
+                    res[(4u * q4 + r) * AT_PART + 2 + 8u * n16 + c] = acc[c][r] * out_scale;
+        }
     }
     __syncthreads();
-    // ---- merge the four waves
+    // ---- merge the waves
     float *dst = a.partial + ((size_t)row * gridDim.x + split) * G * AT_PART;
     for (uint32_t i = tid; i < G * AT_PART; i += AT_WAVES * TQ_WAVE) {
         const uint32_t g = i / AT_PART, j = i % AT_PART;
@@ -1014,10 +1111,10 @@ namespace {
 template <int IPBK>
 int launch_attend(int ipbv, dim3 grid, dim3 block, hipStream_t s, const AttendArgs &a) {
     switch (ipbv) {
-        case 8: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 8>), grid, block, 0, s, a); break;
-        case 4: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 4>), grid, block, 0, s, a); break;
-        case 2: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 2>), grid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 1>), grid, block, 0, s, a); break;
+        case 8: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 8>), grid, dim3(AT_WAVES * TQ_WAVE), 0, s, a); break;
+        case 4: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 4>), grid, dim3(AT_WAVES * TQ_WAVE), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 2>), grid, dim3(AT_WAVES * TQ_WAVE), 0, s, a); break;
+        default: hipLaunchKernelGGL((tq_attend_kernel<IPBK, 1>), grid, dim3(AT_WAVES * TQ_WAVE), 0, s, a); break;
     }
     return (int)hipGetLastError();
 }
@@ -1027,7 +1124,7 @@ extern "C" int tq_attend_splits(long long rows, long long tokens) {
     if (rows <= 0 || tokens <= 0) return 1;
     int cus = 0;
     if (device_cus(cus)) cus = 256;
-    long long splits = ((long long)cus * 4 + rows - 1) / rows;       // two resident four-wave blocks per compute unit, twice over
+    long long splits = ((long long)cus * 2 + rows - 1) / rows;       // one resident eight-wave block per compute unit, twice over
     const long long most = (tokens + AT_RUN * AT_WAVES - 1) / (AT_RUN * AT_WAVES);
     if (splits > most) splits = most;
     if (splits > 4096) splits = 4096;
