@@ -772,113 +772,173 @@ __device__ __forceinline__ float tq_load_elem(const void *base, size_t i, int dt
     return __uint_as_float((uint32_t)b << 16);
 }
 
-// Eight consecutive window elements starting at element index i (a multiple of 8) as floats.
+// Eight consecutive window elements (element index i a multiple of 8): the load and the conversion apart, so that
+// loads can be issued long before their use.
+template <int WD> struct Raw8 { tq_u4 v[WD == TQ_F32 ? 2 : 1]; };
+
 template <int WD>
-__device__ __forceinline__ void tq_load8(const void *base, size_t i, float (&x)[8]) {
+__device__ __forceinline__ Raw8<WD> tq_load8_raw(const void *base, size_t i) {
+    Raw8<WD> r;
     if constexpr (WD == TQ_F32) {
-        const tq_u4 lo = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL float *)base + i);
-        const tq_u4 hi = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL float *)base + i + 4);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) { x[e] = __uint_as_float(lo[e]); x[4 + e] = __uint_as_float(hi[e]); }
+        r.v[0] = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL float *)base + i);
+        r.v[1] = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL float *)base + i + 4);
     } else {
-        const tq_u4 u = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL uint16_t *)base + i);
-        if constexpr (WD == TQ_F16) {
-            const tq_half8 h = __builtin_bit_cast(tq_half8, u);
+        r.v[0] = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL uint16_t *)base + i);
+    }
+    return r;
+}
+
+template <int WD>
+__device__ __forceinline__ void tq_cvt8(const Raw8<WD> &r, float (&x)[8]) {
+    if constexpr (WD == TQ_F32) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = (float)h[e];
-        } else {
+        for (int e = 0; e < 4; ++e) { x[e] = __uint_as_float(r.v[0][e]); x[4 + e] = __uint_as_float(r.v[1][e]); }
+    } else if constexpr (WD == TQ_F16) {
+        const tq_half8 h = __builtin_bit_cast(tq_half8, r.v[0]);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { x[2 * e] = __uint_as_float(u[e] << 16); x[2 * e + 1] = __uint_as_float(u[e] & 0xffff0000u); }
-        }
+        for (int e = 0; e < 8; ++e) x[e] = (float)h[e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { x[2 * e] = __uint_as_float(r.v[0][e] << 16); x[2 * e + 1] = __uint_as_float(r.v[0][e] & 0xffff0000u); }
     }
 }
 
-// Two consecutive window elements starting at element index i (even).
-template <int WD>
-__device__ __forceinline__ void tq_load2(const void *base, size_t i, float &x0, float &x1) {
-    if constexpr (WD == TQ_F32) {
-        const tq_u2 u = *reinterpret_cast<const TQ_GLOBAL tq_u2 *>((const TQ_GLOBAL float *)base + i);
-        x0 = __uint_as_float(u[0]); x1 = __uint_as_float(u[1]);
-    } else {
-        const uint32_t u = *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint16_t *)base + i);
-        if constexpr (WD == TQ_F16) {
-            const tq_half2 h = __builtin_bit_cast(tq_half2, u);
-            x0 = (float)h[0]; x1 = (float)h[1];
-        } else {
-            x0 = __uint_as_float(u << 16); x1 = __uint_as_float(u & 0xffff0000u);
-        }
-    }
+// Sum over the 16 lanes of a DPP row; the total lands in lane 15 of the row.
+__device__ __forceinline__ float tq_row_sum16(float x) {
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x111, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x112, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x114, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x118, 0xf, 0xf, true));
+    return x;
 }
 
 // One block per packed row (batch x kv head), four waves.  Rotates the row's query heads for the packed keys and
 // computes attention statistics over the uncompressed window tokens in fp32 (a few hundred tokens at most).
+// GP = heads per row rounded up to 1, 2, 4 or 8: the padding heads are zero queries, so no loop tests the head count.
+// The loads of the first 128 window tokens, keys and values, are issued before anything else: the kernel waits for
+// memory once.
 //   rotation   : thread (j, half) sums 64 of the 128 terms of every head's q_rot[j]; Pi^T is read once, coalesced
-//   scores     : 16 lanes x 16 bytes cover one token, a wave takes four tokens per load; sums meet over 16 lanes
+//   scores     : 16 lanes x 8 elements cover a key, a wave takes 16 tokens per trip of 64; per token and head a dot
+//                product summed over the DPP row of its 16 lanes
 //   statistics : wave w owns heads w and w + 4
-//   value sums : thread (column pair, wave) over every fourth token, the four waves' sums meet in LDS
-template <int WD>
+//   value sums : 32 lanes x 4 columns cover a value, a wave takes 8 tokens per trip of 32; the two token slots of a
+//                wave meet through one exchange, the four waves in LDS
+template <int WD, int GP>
 __global__ __launch_bounds__(256) void tq_attend_prepare_kernel(PrepareArgs a) {
     constexpr int MAXG = 8, MAXW = 512;
-    __shared__ float q[MAXG][TQ_HEAD_DIM];
+    constexpr int PRE_K = 2;      // key trips (64 tokens each) loaded up front
+    constexpr int PRE_V = 4;      // value trips (32 tokens each) loaded up front
+    constexpr int VW = WD == TQ_F32 ? 4 : 2;             // dwords per four value elements
+    __shared__ __attribute__((aligned(16))) float qt[TQ_HEAD_DIM][MAXG];     // scaled queries, head index fastest
     __shared__ float sc[MAXG][MAXW];
     __shared__ float red[MAXG][2];
     __shared__ float part[4][MAXG][TQ_HEAD_DIM];
     const uint32_t row = blockIdx.x, tid = threadIdx.x, G = a.group, lane = tid & 63u, wave = tid >> 6;
-    for (uint32_t i = tid; i < MAXG * TQ_HEAD_DIM; i += 256u)
-        q[i / TQ_HEAD_DIM][i % TQ_HEAD_DIM] =
-            i < G * TQ_HEAD_DIM ? tq_load_elem(a.queries, (size_t)row * G * TQ_HEAD_DIM + i, a.q_dtype) * a.scale : 0.f;
+    const uint32_t sub = lane & 15u, tk = lane >> 4;          // key side: elements 8 sub .., token slot tk of 4
+    const uint32_t sub5 = lane & 31u, tk5 = lane >> 5;        // value side: columns 4 sub5 .., token slot tk5 of 2
+    const uint32_t W = a.part_w ? a.n_win : 0u;
+    const size_t win_base = (size_t)row * a.win_stride;
+    // past the end the last token is read again and not used
+    auto ktoken = [&](uint32_t trip, int k) { return 64u * trip + 16u * wave + 4u * (uint32_t)k + tk; };
+    auto vtoken = [&](uint32_t trip, int k) { return 32u * trip + 8u * wave + 2u * (uint32_t)k + tk5; };
+    auto vload = [&](uint32_t t, uint32_t (&r)[VW]) __attribute__((always_inline)) {
+        const size_t at = win_base + (size_t)min(t, W - 1u) * TQ_HEAD_DIM + 4u * sub5;
+        if constexpr (WD == TQ_F32) {
+            const tq_u4 v = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>((const TQ_GLOBAL float *)a.v_win + at);
+            r[0] = v[0]; r[1] = v[1]; r[2] = v[2]; r[3] = v[3];
+        } else {
+            const tq_u2 v = *reinterpret_cast<const TQ_GLOBAL tq_u2 *>((const TQ_GLOBAL uint16_t *)a.v_win + at);
+            r[0] = v[0]; r[1] = v[1];
+        }
+    };
+    auto vcvt = [&](const uint32_t (&r)[VW], float (&x)[4]) __attribute__((always_inline)) {
+        if constexpr (WD == TQ_F32) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = __uint_as_float(r[e]);
+        } else if constexpr (WD == TQ_F16) {
+            typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+            const tq_u2 v = {r[0], r[1]};
+            const half4 h = __builtin_bit_cast(half4, v);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = (float)h[e];
+        } else {
+            x[0] = __uint_as_float(r[0] << 16); x[1] = __uint_as_float(r[0] & 0xffff0000u);
+            x[2] = __uint_as_float(r[1] << 16); x[3] = __uint_as_float(r[1] & 0xffff0000u);
+        }
+    };
+    Raw8<WD> kpre[PRE_K][4];
+    uint32_t vpre[PRE_V][4][VW];
+    if (W) {
+#pragma unroll
+        for (int tr = 0; tr < PRE_K; ++tr)
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                kpre[tr][k] = tq_load8_raw<WD>(a.k_win, win_base + (size_t)min(ktoken(tr, k), W - 1u) * TQ_HEAD_DIM + 8u * sub);
+#pragma unroll
+        for (int tr = 0; tr < PRE_V; ++tr)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) vload(vtoken(tr, k), vpre[tr][k]);
+    }
+    for (uint32_t i = tid; i < MAXG * TQ_HEAD_DIM; i += 256u) {
+        const uint32_t g = i / TQ_HEAD_DIM, c = i % TQ_HEAD_DIM;
+        qt[c][g] = i < G * TQ_HEAD_DIM ? tq_load_elem(a.queries, (size_t)row * G * TQ_HEAD_DIM + i, a.q_dtype) * a.scale : 0.f;
+    }
     __syncthreads();
-    {   // rotated queries: q_rot[g][j] = sum_i Pi[j][i] * q[g][i]
+    {   // rotated queries: q_rot[g][j] = sum_i Pi[j][i] * q[g][i]; all heads of a coordinate come with 16-byte reads
         const uint32_t j = tid & 127u, half = tid >> 7;
         const TQ_GLOBAL float *pc = (const TQ_GLOBAL float *)a.pi_k_t + (size_t)half * 64u * TQ_HEAD_DIM + j;
-        float s[MAXG];
+        float s[GP];
 #pragma unroll
-        for (int g = 0; g < MAXG; ++g) s[g] = 0.f;
-#pragma unroll 8
+        for (int g = 0; g < GP; ++g) s[g] = 0.f;
+#pragma unroll 16
         for (int i = 0; i < 64; ++i) {
             const float p = pc[(size_t)i * TQ_HEAD_DIM];
+            float qv[8];
+            *reinterpret_cast<float4 *>(&qv[0]) = *reinterpret_cast<const float4 *>(&qt[half * 64u + i][0]);
+            if constexpr (GP > 4) *reinterpret_cast<float4 *>(&qv[4]) = *reinterpret_cast<const float4 *>(&qt[half * 64u + i][4]);
 #pragma unroll
-            for (int g = 0; g < MAXG; ++g) s[g] = fmaf(p, q[g][half * 64u + i], s[g]);
+            for (int g = 0; g < GP; ++g) s[g] = fmaf(p, qv[g], s[g]);
         }
 #pragma unroll
-        for (int g = 0; g < MAXG; ++g) part[half][g][j] = s[g];
+        for (int g = 0; g < GP; ++g) part[half][g][j] = s[g];
     }
     __syncthreads();
     for (uint32_t o = tid; o < G * TQ_HEAD_DIM; o += 256u)
         ((TQ_GLOBAL float *)a.q_rot)[(size_t)row * G * TQ_HEAD_DIM + o] =
             part[0][o / TQ_HEAD_DIM][o % TQ_HEAD_DIM] + part[1][o / TQ_HEAD_DIM][o % TQ_HEAD_DIM];
-    if (!a.part_w) return;
-    const uint32_t W = a.n_win;
-    const size_t win_base = (size_t)row * a.win_stride;
+    if (!W) return;
     {   // scores of the window tokens
-        const uint32_t sub = lane & 15u, tk = lane >> 4;
-        float qq[MAXG][8];
+        const uint32_t trips = (W + 63u) / 64u;
+        float qq[GP][8];
 #pragma unroll
-        for (int g = 0; g < MAXG; ++g)
+        for (int g = 0; g < GP; ++g)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) qq[g][e] = q[g][8u * sub + e];
-        for (uint32_t t0 = 4u * wave; t0 < W; t0 += 16u) {
-            const uint32_t t = t0 + tk;
-            float x[8];
-            if (t < W) {
-                tq_load8<WD>(a.k_win, win_base + (size_t)t * TQ_HEAD_DIM + 8u * sub, x);
-            } else {
+            for (int e = 0; e < 8; ++e) qq[g][e] = qt[8u * sub + e][g];
+        auto score4 = [&](uint32_t trip, const Raw8<WD> (&raw)[4]) __attribute__((always_inline)) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) x[e] = 0.f;
-            }
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t t = ktoken(trip, k);
+                float x[8];
+                tq_cvt8<WD>(raw[k], x);
 #pragma unroll
-            for (int g = 0; g < MAXG; ++g) {
-                if ((uint32_t)g < G) {           // uniform over the block
+                for (int g = 0; g < GP; ++g) {
                     float sg = 0.f;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) sg = fmaf(x[e], qq[g][e], sg);
-                    sg += __shfl_xor(sg, 1);
-                    sg += __shfl_xor(sg, 2);
-                    sg += __shfl_xor(sg, 4);
-                    sg += __shfl_xor(sg, 8);
-                    if (sub == 0u && t < W) sc[g][t] = sg;
+                    sg = tq_row_sum16(sg);
+                    if (sub == 15u && t < W) sc[g][t] = sg;
                 }
             }
+        };
+#pragma unroll
+        for (int tr = 0; tr < PRE_K; ++tr)
+            if ((uint32_t)tr < trips) score4(tr, kpre[tr]);      // uniform
+        for (uint32_t trip = PRE_K; trip < trips; ++trip) {
+            Raw8<WD> raw[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                raw[k] = tq_load8_raw<WD>(a.k_win, win_base + (size_t)min(ktoken(trip, k), W - 1u) * TQ_HEAD_DIM + 8u * sub);
+            score4(trip, raw);
         }
     }
     __syncthreads();                      // (the value sums below reuse `part`: every q_rot read of it is behind us)
@@ -898,25 +958,43 @@ __global__ __launch_bounds__(256) void tq_attend_prepare_kernel(PrepareArgs a) {
         if (lane == 0u) { red[g][0] = m; red[g][1] = l; }
     }
     __syncthreads();
-    {   // weighted value sums: this thread's two columns over tokens wave, wave + 4, ...
-        float acc[MAXG][2];
+    {   // weighted value sums: this lane's four columns over its tokens
+        const uint32_t trips = (W + 31u) / 32u;
+        float acc[GP][4];
 #pragma unroll
-        for (int g = 0; g < MAXG; ++g) acc[g][0] = acc[g][1] = 0.f;
-#pragma unroll 4
-        for (uint32_t t = wave; t < W; t += 4u) {
-            float x0, x1;
-            tq_load2<WD>(a.v_win, win_base + (size_t)t * TQ_HEAD_DIM + 2u * lane, x0, x1);
+        for (int g = 0; g < GP; ++g)
 #pragma unroll
-            for (int g = 0; g < MAXG; ++g) {
-                if ((uint32_t)g < G) {
-                    const float p = sc[g][t];
-                    acc[g][0] = fmaf(p, x0, acc[g][0]);
-                    acc[g][1] = fmaf(p, x1, acc[g][1]);
+            for (int e = 0; e < 4; ++e) acc[g][e] = 0.f;
+        auto sum4 = [&](uint32_t trip, const uint32_t (&raw)[4][VW]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t t = vtoken(trip, k);
+                float x[4];
+                vcvt(raw[k], x);
+#pragma unroll
+                for (int g = 0; g < GP; ++g) {
+                    const float p = (t < W && (uint32_t)g < G) ? sc[g][t] : 0.f;    // rows g >= G of sc are never written
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[g][e] = fmaf(p, x[e], acc[g][e]);
                 }
             }
+        };
+#pragma unroll
+        for (int tr = 0; tr < PRE_V; ++tr)
+            if ((uint32_t)tr < trips) sum4(tr, vpre[tr]);        // uniform
+        for (uint32_t trip = PRE_V; trip < trips; ++trip) {
+            uint32_t raw[4][VW];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) vload(vtoken(trip, k), raw[k]);
+            sum4(trip, raw);
         }
 #pragma unroll
-        for (int g = 0; g < MAXG; ++g) { part[wave][g][2u * lane] = acc[g][0]; part[wave][g][2u * lane + 1u] = acc[g][1]; }
+        for (int g = 0; g < GP; ++g)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float v = acc[g][e] + __shfl_xor(acc[g][e], 32);
+                if (tk5 == 0u) part[wave][g][4u * sub5 + e] = v;
+            }
     }
     __syncthreads();
     float *out = a.part_w + (size_t)row * G * AT_PART;
@@ -1183,9 +1261,15 @@ extern "C" int tq_attend_prepare(const void *queries, int q_dtype, long long row
     a.group = (uint32_t)group; a.n_win = (uint32_t)n_win;
     a.q_dtype = q_dtype; a.win_dtype = win_dtype;
     const hipStream_t st = static_cast<hipStream_t>(stream);
-    if (n_win && win_dtype == TQ_F32) hipLaunchKernelGGL(tq_attend_prepare_kernel<TQ_F32>, dim3((unsigned)rows), dim3(256), 0, st, a);
-    else if (n_win && win_dtype == TQ_F16) hipLaunchKernelGGL(tq_attend_prepare_kernel<TQ_F16>, dim3((unsigned)rows), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(tq_attend_prepare_kernel<TQ_BF16>, dim3((unsigned)rows), dim3(256), 0, st, a);
+    const int wd = n_win ? win_dtype : TQ_BF16;
+    const int gp = group > 4 ? 8 : group > 2 ? 4 : group;
+    const dim3 grid((unsigned)rows), block(256);
+#define TQ_PREP_CASE(WD, GP) \
+    if (wd == WD && gp == GP) hipLaunchKernelGGL((tq_attend_prepare_kernel<WD, GP>), grid, block, 0, st, a)
+    TQ_PREP_CASE(TQ_F32, 1); TQ_PREP_CASE(TQ_F32, 2); TQ_PREP_CASE(TQ_F32, 4); TQ_PREP_CASE(TQ_F32, 8);
+    TQ_PREP_CASE(TQ_F16, 1); TQ_PREP_CASE(TQ_F16, 2); TQ_PREP_CASE(TQ_F16, 4); TQ_PREP_CASE(TQ_F16, 8);
+    TQ_PREP_CASE(TQ_BF16, 1); TQ_PREP_CASE(TQ_BF16, 2); TQ_PREP_CASE(TQ_BF16, 4); TQ_PREP_CASE(TQ_BF16, 8);
+#undef TQ_PREP_CASE
     return (int)hipGetLastError();
 }
 
