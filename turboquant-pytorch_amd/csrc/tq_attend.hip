@@ -384,61 +384,6 @@ constexpr int AT_PART = TQ_HEAD_DIM + 2;
 typedef float tq_f4v __attribute__((ext_vector_type(4)));
 constexpr int AT_WAVES = 8;      // one block per compute unit (two waves per SIMD): the table copies below are shared by its waves
 
-// The byte -> centroids tables are read with data-dependent addresses by every lane.  With one copy, 64 random
-// addresses over 32 banks serialise several times over (measured: the LDS pipe was busy 70 % of the kernel).  Here
-// every table entry is spread over 128 bytes = one slot per bank group, and a lane always reads the slot of its own
-// banks: entries of 2 or 4 bytes have 32 slots of 4 bytes (lane % 32), 8-byte entries 16 slots (lane % 16: a 64-bit
-// read serves 16 lanes per clock), 16-byte entries 8 slots.  256 entries x 128 bytes = 32 KiB per table.
-template <int IPB>
-struct RepLut {
-    static constexpr int ES = 2 * IPB;                    // bytes per entry
-    static constexpr int SL = ES < 4 ? 4 : ES;            // slot size
-    static constexpr int NC = 128 / SL;                   // copies
-    static __device__ __forceinline__ uint32_t lane_offset(uint32_t lane) { return (lane & (NC - 1)) * SL; }
-    static __device__ __forceinline__ void stage(uint8_t *lds, const uint8_t *src, uint32_t tid, uint32_t nthreads) {
-        for (uint32_t i = tid; i < 256u * NC; i += nthreads) {
-            const uint32_t e = i / NC, c = i % NC;
-            uint8_t *dst = lds + e * 128u + c * SL;
-            const TQ_GLOBAL uint8_t *g = (const TQ_GLOBAL uint8_t *)src + e * ES;
-            if constexpr (ES == 2) *reinterpret_cast<uint16_t *>(dst) = *reinterpret_cast<const TQ_GLOBAL uint16_t *>(g);
-            else if constexpr (ES == 4) *reinterpret_cast<uint32_t *>(dst) = *reinterpret_cast<const TQ_GLOBAL uint32_t *>(g);
-            else if constexpr (ES == 8) *reinterpret_cast<tq_u2 *>(dst) = *reinterpret_cast<const TQ_GLOBAL tq_u2 *>(g);
-            else *reinterpret_cast<tq_u4 *>(dst) = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>(g);
-        }
-    }
-};
-
-// decode_step against a replicated table; `lut` already points at the lane's slot of entry 0
-template <int IPB, int NW>
-__device__ __forceinline__ tq_u4 decode_rep(const uint32_t (&raw)[NW], int s, const uint8_t *lut) {
-    tq_u4 out;
-    if constexpr (IPB == 1) {
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const uint32_t b0 = (raw[2 * s + (2 * d) / 4] >> (8 * ((2 * d) % 4))) & 0xffu;
-            const uint32_t b1 = (raw[2 * s + (2 * d + 1) / 4] >> (8 * ((2 * d + 1) % 4))) & 0xffu;
-            const uint32_t lo = *reinterpret_cast<const uint16_t *>(lut + (b0 << 7));
-            const uint32_t hi = *reinterpret_cast<const uint16_t *>(lut + (b1 << 7));
-            out[d] = lo | (hi << 16);
-        }
-    } else if constexpr (IPB == 2) {
-#pragma unroll
-        for (int d = 0; d < 4; ++d) out[d] = *reinterpret_cast<const uint32_t *>(lut + (((raw[s] >> (8 * d)) & 0xffu) << 7));
-    } else if constexpr (IPB == 4) {
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            const uint32_t b = (raw[s / 2] >> (16 * (s % 2) + 8 * q)) & 0xffu;
-            const tq_u2 v = *reinterpret_cast<const tq_u2 *>(lut + (b << 7));
-            out[2 * q] = v[0];
-            out[2 * q + 1] = v[1];
-        }
-    } else {
-        const uint32_t b = (raw[s / 4] >> (8 * (s % 4))) & 0xffu;
-        out = *reinterpret_cast<const tq_u4 *>(lut + (b << 7));
-    }
-    return out;
-}
-
 template <int IPBK, int IPBV>
 __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_kernel(AttendArgs a) {
     constexpr int KB = TQ_HEAD_DIM / IPBK / 4;           // key bytes per lane and token (32 coordinates): 4, 8, 16, 32
