@@ -410,3 +410,44 @@ def test_attend_prepare_and_merge_against_float64(pkg, wdtype, qdtype, G, W, spl
         tol = {torch.float32: 1e-5, torch.float16: 1e-3, torch.bfloat16: 6e-3}[odtype]
         print(f"[prepare/merge] window {W} x {wdtype}, {G} heads, {splits} splits -> {odtype}: {err:.2e}")
         assert err < tol
+
+
+def test_hf_model_runs_on_the_cache(pkg):
+    """A small randomly initialised Llama (transformers, no download) runs prefill + decode and `generate` with the
+    cache as `past_key_values`, the way generation_test_v2.py:178-201 drives the reference's cache.  With 8-bit keys
+    and values the logits stay close to those of the stock DynamicCache; with K4/V2 the run completes and the cache
+    holds what the model fed it."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM
+    torch.manual_seed(0)
+    cfg = LlamaConfig(vocab_size=256, hidden_size=512, intermediate_size=1024, num_hidden_layers=3, num_attention_heads=4,
+                      num_key_value_heads=2, head_dim=128, max_position_embeddings=512)
+    model = LlamaForCausalLM(cfg).to(DEV, dtype=torch.bfloat16).eval()
+    cls = pkg.hf_cache_class()
+    ids = torch.randint(0, 256, (2, 40), device=DEV)
+    mask = torch.ones_like(ids)
+    with torch.no_grad():
+        cache = cls(key_bits=8, value_bits=8, residual_window=8, n_layers=3)
+        ref_cache = DynamicCache()
+        out = model(ids, attention_mask=mask, past_key_values=cache, use_cache=True)
+        ref = model(ids, attention_mask=mask, past_key_values=ref_cache, use_cache=True)
+        # prefill attends over what update() returned: the de-quantised prompt (all but the window)
+        rel = float((out.logits.float() - ref.logits.float()).norm() / ref.logits.float().norm())
+        print(f"[hf] prefill logits, 8-bit cache vs DynamicCache: {rel:.2e}")
+        assert rel < 3e-2
+        for step in range(6):
+            nxt = torch.randint(0, 256, (2, 1), device=DEV)
+            mask = torch.cat([mask, torch.ones_like(nxt)], dim=1)
+            out = model(nxt, attention_mask=mask, past_key_values=cache, use_cache=True)
+            ref = model(nxt, attention_mask=mask, past_key_values=ref_cache, use_cache=True)
+            rel = float((out.logits.float() - ref.logits.float()).norm() / ref.logits.float().norm())
+            assert rel < 3e-2, (step, rel)
+        print(f"[hf] decode step logits, 8-bit cache vs DynamicCache: {rel:.2e}")
+        assert cache.get_seq_length() == 46 and ref_cache.get_seq_length() == 46
+        assert cache.get_compression_info() == "38 compressed, 8 fp16, 46 total"
+        small = cls(key_bits=4, value_bits=2, residual_window=16, n_layers=3)
+        gen = model.generate(ids, attention_mask=torch.ones_like(ids), past_key_values=small, max_new_tokens=12, do_sample=False)
+        assert gen.shape == (2, 52) and torch.equal(gen[:, :40], ids)
+        assert small.get_seq_length() == 51            # the last generated token has not been fed back
+        assert small.get_compression_info() == "35 compressed, 16 fp16, 51 total"
+        assert sorted(small._stores) == [0, 1, 2]
