@@ -451,3 +451,41 @@ def test_hf_model_runs_on_the_cache(pkg):
         assert small.get_seq_length() == 51            # the last generated token has not been fed back
         assert small.get_compression_info() == "35 compressed, 16 fp16, 51 total"
         assert sorted(small._stores) == [0, 1, 2]
+
+
+def test_hf_model_decodes_through_packed_attention(pkg):
+    """The same small Llama with the registered attention function: decode steps are answered from the packed
+    store (`attend`) and never de-quantise the history.  Same tokens fed to both, the logits equal those of the
+    ordinary `update` path of an identically configured cache up to rounding; `generate` runs on it."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import LlamaConfig, LlamaForCausalLM
+    torch.manual_seed(0)
+    cfg = LlamaConfig(vocab_size=256, hidden_size=512, intermediate_size=1024, num_hidden_layers=3, num_attention_heads=4,
+                      num_key_value_heads=2, head_dim=128, max_position_embeddings=512)
+    model = LlamaForCausalLM(cfg).to(DEV, dtype=torch.bfloat16).eval()
+    name = pkg.register_packed_attention()
+    cls = pkg.hf_cache_class()
+    ids = torch.randint(0, 256, (2, 70), device=DEV)
+    steps = [torch.randint(0, 256, (2, 1), device=DEV) for _ in range(8)]
+    logits = {}
+    with torch.no_grad():
+        for packed in (False, True):
+            model.config._attn_implementation = name if packed else "sdpa"
+            cache = cls(key_bits=4, value_bits=2, residual_window=16, n_layers=3, packed_attention=packed)
+            mask = torch.ones_like(ids)
+            out = [model(ids, attention_mask=mask, past_key_values=cache, use_cache=True).logits[:, -1:].float()]
+            for nxt in steps:
+                mask = torch.cat([mask, torch.ones_like(nxt)], dim=1)
+                out.append(model(nxt, attention_mask=mask, past_key_values=cache, use_cache=True).logits.float())
+            logits[packed] = torch.cat(out, dim=1)
+            assert cache.get_seq_length() == 78 and cache.get_compression_info() == "62 compressed, 16 fp16, 78 total"
+        a, b = logits[False], logits[True]
+        assert torch.equal(a[:, 0], b[:, 0])                       # prefill takes the same path in both
+        rel = float((a[:, 1:] - b[:, 1:]).norm() / a[:, 1:].norm())
+        print(f"[hf] decode logits, packed attention vs update path (K4/V2): {rel:.2e}")
+        assert rel < 2e-2
+        model.config._attn_implementation = name
+        cache = cls(key_bits=4, value_bits=2, residual_window=16, n_layers=3, packed_attention=True)
+        gen = model.generate(ids, attention_mask=torch.ones_like(ids), past_key_values=cache, max_new_tokens=10, do_sample=False)
+        assert gen.shape == (2, 80) and cache.get_seq_length() == 79
+        model.config._attn_implementation = "sdpa"

@@ -283,16 +283,28 @@ class V3Cache:
 
 def hf_cache_class():
     """A `V3Cache` that also derives from transformers.DynamicCache, so that it can be passed as
-    `past_key_values` to `model.generate` the way generation_test_v2.py:178-201 does."""
+    `past_key_values` to `model.generate` the way generation_test_v2.py:178-201 does.
+
+    With `packed_attention=True` (keyword of the returned class) decode steps do not de-quantise the history:
+    `update` only appends the new token and hands it back tagged, and the attention function registered by
+    `register_packed_attention()` computes the step's attention straight from the packed store (`attend`).
+    Prefill (more than one new token) takes the ordinary path.  Batches must not be padded in that mode: every
+    cached token is attended to."""
     from transformers import DynamicCache
 
     class HFV3Cache(V3Cache, DynamicCache):
-        def __init__(self, *args, **kwargs):
+        def __init__(self, *args, packed_attention: bool = False, **kwargs):
             DynamicCache.__init__(self)
             V3Cache.__init__(self, *args, **kwargs)
+            self.packed_attention = packed_attention
 
         def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
-            out = V3Cache.update(self, key_states, value_states, layer_idx, cache_kwargs)
+            if self.packed_attention and key_states.shape[2] == 1 and V3Cache.get_seq_length(self, layer_idx) > 0:
+                V3Cache.append(self, key_states, value_states, layer_idx)
+                key_states._tq_packed = (self, layer_idx)       # read by packed_attention_forward
+                out = (key_states, value_states)
+            else:
+                out = V3Cache.update(self, key_states, value_states, layer_idx, cache_kwargs)
             layers = getattr(self, "layers", None)
             if layers is not None:
                 from transformers.cache_utils import DynamicLayer
@@ -303,4 +315,30 @@ def hf_cache_class():
         def get_seq_length(self, layer_idx=0):
             return V3Cache.get_seq_length(self, layer_idx)
 
+        def get_mask_sizes(self, query_length, layer_idx=0):
+            # (length, offset) of the keys the next update() of this layer will return
+            return V3Cache.get_seq_length(self, layer_idx) + int(query_length), 0
+
     return HFV3Cache
+
+
+def packed_attention_forward(module, query, key, value, attention_mask, scaling=None, dropout=0.0, **kwargs):
+    """Attention function for transformers' AttentionInterface.  A decode step whose keys come tagged from a
+    cache in packed-attention mode is answered by `V3Cache.attend` (scores, softmax and value sum computed from
+    the packed codes; the mask is not consulted: all cached tokens count).  Everything else is passed to the
+    library's scaled-dot-product implementation unchanged."""
+    tag = getattr(key, "_tq_packed", None)
+    if tag is not None and query.shape[2] == 1:
+        cache, layer_idx = tag
+        out = cache.attend(query, layer_idx, scale=scaling)           # [B, Hq, 1, D]
+        return out.transpose(1, 2).contiguous(), None
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+    return ALL_ATTENTION_FUNCTIONS["sdpa"](module, query, key, value, attention_mask, dropout=dropout, scaling=scaling, **kwargs)
+
+
+def register_packed_attention(name: str = "tq_packed") -> str:
+    """Register `packed_attention_forward` under `name`; select it with
+    `model.config._attn_implementation = name` (or `model.set_attn_implementation(name)`)."""
+    from transformers import AttentionInterface
+    AttentionInterface.register(name, packed_attention_forward)
+    return name
