@@ -6,14 +6,14 @@ A "step" is one pass over the whole synthetic cache: every layer's K and V tenso
 (one launch per bit-width group and direction).  Inputs, packed buffers and outputs are
 resident in HBM before the timed region starts.
 
-Default workload (the one BASELINE.json quotes its target on): Llama-3-8B-shaped cache,
+Default workload (the headline configuration): Llama-3-8B-shaped cache,
 32 layers x [1, 8, 32768, 128] bf16, K4/V2, protected_layers=4 with the reference's semantics
 (the first and last 4 layers use 8-bit keys AND values, compressors_v3.py:158-160), no residual
 window.  `--workload llama3-8b-32k-k4v2` runs the same shape with every layer at K4/V2;
-`--workload qwen2.5-3b-8k` is BASELINE config 2 (fp16); `--workload decode-64x16k` is the streaming
+`--workload qwen2.5-3b-8k` is the small Qwen2.5-3B-shaped cache (36 layers x [1, 2, 8192, 128] fp16); `--workload decode-64x16k` is the streaming
 decode case (config 5): a step is one generated token through `V3Cache.update` on every layer.
 
-Prints ONE JSON line (see README / DESIGN.md for the fields).
+Prints ONE JSON line: metric, value (vectors/s), ms_per_step, config.workload, roofline (dominant kernel) and cpu_baseline.
 """
 import argparse
 import importlib
@@ -34,7 +34,7 @@ WORKLOADS = {
     "llama3-8b-32k": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2, protected=4),
     "llama3-8b-32k-k4v2": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2, protected=0),
     "qwen2.5-3b-8k": dict(layers=36, batch=1, heads=2, tokens=8192, dtype="f16", key_bits=4, value_bits=2, protected=0),
-    # streaming decode (BASELINE config 5): 64 sequences with 16384 compressed + 128 window tokens; a step is
+    # streaming decode: 64 sequences with 16384 compressed + 128 window tokens; a step is
     # one new token through V3Cache.update on all 32 layers (compress what leaves the window, de-quantise all)
     "decode-64x16k": dict(layers=32, batch=64, heads=8, tokens=16384, dtype="bf16", key_bits=4, value_bits=2,
                           protected=0, window=128, decode=True),

@@ -66,7 +66,7 @@ def test_roundtrip_fixtures_c(golden, oracle, accum_double):
 
 
 def test_config1_known_answer(golden, oracle):
-    """BASELINE config 1 (K [1,8,1024,128] fp32 N(0,1) seed 0, 4-bit, rotation seed 42): the
+    """The reference's CPU-runnable case (K [1,8,1024,128] fp32 N(0,1) seed 0, 4-bit, rotation seed 42): the
     reference's SHA-256 of packed bytes, norms and reconstruction, its MSE and cosine."""
     meta = golden["json"]["config1"]
     torch.manual_seed(0)
