@@ -489,3 +489,44 @@ def test_hf_model_decodes_through_packed_attention(pkg):
         gen = model.generate(ids, attention_mask=torch.ones_like(ids), past_key_values=cache, max_new_tokens=10, do_sample=False)
         assert gen.shape == (2, 80) and cache.get_seq_length() == 79
         model.config._attn_implementation = "sdpa"
+
+
+def test_fused_attention_over_extreme_value_norms(pkg, oracle):
+    """Value norms spanning twelve decimal orders inside one history (tiny, ordinary, huge, exactly zero) and keys
+    with zero vectors: the kernel scales value norms relative to the largest one it has seen, so the result follows
+    float64 attention over the oracle-decoded cache wherever the huge-norm tokens carry weight, and rows whose
+    values are all tiny or all zero come out tiny or zero, never NaN."""
+    B, H, G, S, D = 1, 4, 4, 700, 128
+    kc = pkg.MSECompressor(D, 4, seed=21, device=DEV)
+    vc = pkg.MSECompressor(D, 2, seed=521, device=DEV)
+    g = torch.Generator(device="cpu")
+    g.manual_seed(77)
+    keys = torch.randn(B, H, S, D, generator=g)
+    vals = torch.randn(B, H, S, D, generator=g)
+    vals[:, 0] *= 1e-6                                   # a row of tiny values
+    vals[:, 1, :300] *= 1e-6                             # tiny first, then huge: the reference exponent has to move
+    vals[:, 1, 300:] *= 3e3
+    vals[:, 2] = 0                                       # all zero
+    vals[:, 3, ::7] *= 3e3                               # mixed within every run (norms stay below the fp16 limit of 65504)
+    keys[:, 3, 100:140] = 0                              # zero keys score 0
+    keys, vals = keys.to(torch.bfloat16).to(DEV), vals.to(torch.bfloat16).to(DEV)
+    ck, cv = kc.compress(keys), vc.compress(vals)
+    k_idx, k_nrm = ck["idx_bytes"].reshape(B, H, S, -1), ck["vec_norms"].reshape(B, H, S)
+    v_idx, v_nrm = cv["idx_bytes"].reshape(B, H, S, -1), cv["vec_norms"].reshape(B, H, S)
+    q = torch.randn(B, H * G, D, generator=g).to(DEV)
+    scale = D ** -0.5
+    q_rot = torch.matmul(q, kc.Pi.T) * scale
+    part = torch.ops.tqamd.attend_partials(k_idx, k_nrm, v_idx, v_nrm, kc.table(), vc.table(), 4, 2, q_rot)
+    assert bool(torch.isfinite(part).all())
+    m_s, l_s, a_s = part[..., 0], part[..., 1], part[..., 2:]
+    f = torch.exp(m_s - m_s.amax(dim=-1, keepdim=True))
+    got = (torch.matmul((f.unsqueeze(-1) * a_s).sum(2), vc.Pi) / (f * l_s).sum(-1, keepdim=True)).cpu().numpy()
+    k_hat = _oracle_decode(oracle, kc, k_idx, k_nrm, (B, H, S, D))
+    v_hat = _oracle_decode(oracle, vc, v_idx, v_nrm, (B, H, S, D))
+    _, ref = oracle.attention_decode(q.cpu().numpy(), k_hat, v_hat, scale)
+    got, ref = got.reshape(H, G, D), ref.reshape(H, G, D)
+    for h in (0, 1, 3):
+        err = np.linalg.norm(got[h] - ref[h]) / np.linalg.norm(ref[h])
+        print(f"[fused attention] value-norm case {h}: relative L2 error {err:.2e}, |out| = {np.linalg.norm(ref[h]):.2e}")
+        assert err < 3e-3
+    assert np.all(got[2] == 0) and np.all(ref[2] == 0)
