@@ -365,3 +365,5 @@ def test_v3cache_refuses_cpu_tensors_and_reports_state(pkg):
     assert cache.get_seq_length() == 0 and cache.get_compression_info() == "no compression"
     with pytest.raises(Exception):                          # no CPU path: the codec tables live on HIP devices
         cache.update(torch.zeros(1, 1, 8, 128), torch.zeros(1, 1, 8, 128), 0)
+    with pytest.raises(ValueError, match="nothing is cached"):
+        pkg.V3Cache(key_bits=4, value_bits=2).attend(torch.zeros(1, 4, 1, 128), 0)

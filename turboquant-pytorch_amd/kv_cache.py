@@ -204,7 +204,9 @@ class V3Cache:
         fused (default: whenever at most 8 query heads share a kv head): one kernel pass over packed keys and
         values with an online softmax per split of the history; otherwise three steps (scores from the packed
         keys, softmax in float32, weighted sum of the packed values).  Window tokens are used as they are."""
-        st = self._stores[layer_idx]
+        st = self._stores.get(layer_idx)
+        if st is None or st.total_seq == 0:
+            raise ValueError(f"attend: nothing is cached for layer {layer_idx}")
         B, Hq, Sq, D = query_states.shape
         if Sq != 1 or B != st.B or Hq % st.H:
             raise ValueError(f"attend needs one query token per sequence, [B={st.B}, k*{st.H}, 1, {st.D}]; got {tuple(query_states.shape)}")
@@ -214,9 +216,8 @@ class V3Cache:
         kc, vc = st.comp.key_compressor, st.comp.val_compressor
         if fused is None:
             fused = G <= 8
-        q4 = query_states.reshape(B, st.H, G, D).to(torch.float32)
         kw, vw = st.window()
-        if fused and (n_c or n_w) and n_w <= 512:
+        if fused and n_w <= 512:
             # three launches: rotate the queries + window statistics, one pass over the packed history,
             # log-sum-exp merge + rotation back + cast
             if n_c:
@@ -229,6 +230,7 @@ class V3Cache:
                                                  kc.bits, vc.bits, kc.pi_transposed(), vc.Pi, kw, vw, float(scale))
         # rows padded to a multiple of 8 floats (the kernels read weights with 16-byte loads); the padding
         # scores are -inf, so the softmax runs over the whole contiguous buffer
+        q4 = query_states.reshape(B, st.H, G, D).to(torch.float32)
         total = n_c + n_w
         width = -(-total // 8) * 8
         scores = torch.empty((B, Hq, width), dtype=torch.float32, device=query_states.device)
