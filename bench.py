@@ -188,6 +188,8 @@ def main():
     ap.add_argument("--workload", default="llama3-8b-32k", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
+    ap.add_argument("--launch-order", default="",
+                    help="sequence of the step's launches, e.g. c2,c4,c8,d8,d4,d2 (default: compress by width, then decompress by width)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; the codec shards without communication "
@@ -231,6 +233,12 @@ def main():
     torch.cuda.synchronize()
 
     launches = [("compress", b) for b in order] + [("decompress", b) for b in order]
+    if args.launch_order:     # e.g. "c2,c4,c8,d8,d4,d2": the same six launches in another sequence
+        launches = [("compress" if t[0] == "c" else "decompress", int(t[1:])) for t in args.launch_order.split(",")]
+        if sorted(launches) != sorted([("compress", b) for b in order] + [("decompress", b) for b in order]):
+            raise SystemExit(f"--launch-order must name every launch of the workload once: {order}")
+        if any(launches.index(("compress", b)) > launches.index(("decompress", b)) for b in order):
+            raise SystemExit("--launch-order: a width group is de-quantised before it is compressed")
 
     def step(evs=None):
         """One pass over the cache.  `evs`: pre-created (start, stop) event pairs, one per launch."""

@@ -196,14 +196,14 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
             for (int j = 0; j < NSTORE; ++j) {
                 const uint32_t vl = j * VEC_PER_STORE + st_vec;
                 if (FULL || tl * 32u + vl < job.n_vec)
-                    tq_gstore16(base + st_off[j] + (vl >= o.in_row ? row_wrap : 0ll), val[j]);
+                    tq_gstore16_stream(base + st_off[j] + (vl >= o.in_row ? row_wrap : 0ll), val[j]);
             }
         } else {
 #pragma unroll
             for (int j = 0; j < NSTORE; ++j) {
                 const uint32_t vl = j * VEC_PER_STORE + st_vec;
                 if (FULL || tl * 32u + vl < job.n_vec)
-                    tq_gstore16(out_base + tq_vec_offset(job, tl * 32u + vl) + st_piece * 16u, val[j]);
+                    tq_gstore16_stream(out_base + tq_vec_offset(job, tl * 32u + vl) + st_piece * 16u, val[j]);
             }
         }
     };

@@ -72,6 +72,14 @@ __device__ __forceinline__ tq_u2 tq_gload8(const uint8_t *p) {
 __device__ __forceinline__ uint16_t tq_gload2(const uint16_t *p) {
     return *((const TQ_GLOBAL uint16_t *)p);
 }
+// Streaming store for bulk output that this launch does not read again (the de-quantised tensors): the
+// non-temporal hint keeps it out of the last-level cache.  Measured on the Llama-3-8B 32K workload: the 4- and
+// 8-bit decompress launches 4-5 % faster (436 -> 413 us, 340 -> 327 us), and packed codes that fit the
+// last-level cache stay there across launches.  The same hint on the compress kernel's loads changed nothing;
+// on its packed-code stores it cost 45 % on the 8-bit launch.
+__device__ __forceinline__ void tq_gstore16_stream(uint8_t *p, tq_u4 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<TQ_GLOBAL tq_u4 *>((TQ_GLOBAL uint8_t *)p));
+}
 __device__ __forceinline__ void tq_gstore16(uint8_t *p, tq_u4 v) {
     *reinterpret_cast<TQ_GLOBAL tq_u4 *>((TQ_GLOBAL uint8_t *)p) = v;
 }
