@@ -42,6 +42,9 @@ WORKLOADS = {
     # (32 query heads over 8 kv heads) computed from the packed store, nothing de-quantised to memory
     "decode-attend-64x16k": dict(layers=32, batch=64, heads=8, tokens=16384, dtype="bf16", key_bits=4, value_bits=2,
                                  protected=0, window=128, decode=True, attend=True, q_heads=32),
+    # one sequence with a long context: the latency-bound end of the same path
+    "decode-attend-1x32k": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2,
+                                protected=0, window=128, decode=True, attend=True, q_heads=32),
 }
 
 

@@ -309,13 +309,15 @@ def _packed_width(head_dim: int, bits: int) -> int:
     return -(-head_dim // ipb)
 
 
-@torch.library.custom_op("tqamd::compress", mutates_args=(), device_types="cuda")
-def compress_op(states: torch.Tensor, table: torch.Tensor, bits: int) -> Tuple[torch.Tensor, torch.Tensor]:
+def _compress_impl(states: torch.Tensor, table: torch.Tensor, bits: int) -> Tuple[torch.Tensor, torch.Tensor]:
     B, H, S, D = states.shape
     idx_bytes = torch.empty((B, H, S, _packed_width(D, bits)), dtype=torch.uint8, device=states.device)
     vec_norms = torch.empty((B, H, S), dtype=torch.float16, device=states.device)
     compress_into(states, table, bits, idx_bytes, vec_norms)
     return idx_bytes, vec_norms
+
+
+compress_op = torch.library.custom_op("tqamd::compress", _compress_impl, mutates_args=(), device_types="cuda")
 
 
 @compress_op.register_fake
@@ -325,19 +327,23 @@ def _(states, table, bits):
             states.new_empty((B, H, S), dtype=torch.float16))
 
 
-@torch.library.custom_op("tqamd::compress_into", mutates_args=("idx_bytes", "vec_norms"), device_types="cuda")
-def compress_into_op(states: torch.Tensor, table: torch.Tensor, bits: int,
+def _compress_into_impl(states: torch.Tensor, table: torch.Tensor, bits: int,
                      idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> None:
     compress_into(states, table, bits, idx_bytes, vec_norms)
 
 
-@torch.library.custom_op("tqamd::decompress", mutates_args=(), device_types="cuda")
-def decompress_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
+compress_into_op = torch.library.custom_op("tqamd::compress_into", _compress_into_impl, mutates_args=("idx_bytes", "vec_norms"), device_types="cuda")
+
+
+def _decompress_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
                   head_dim: int, out_dtype: torch.dtype) -> torch.Tensor:
     B, H, S, _ = idx_bytes.shape
     out = torch.empty((B, H, S, head_dim), dtype=out_dtype, device=idx_bytes.device)
     decompress_into(idx_bytes, vec_norms, table, bits, out)
     return out
+
+
+decompress_op = torch.library.custom_op("tqamd::decompress", _decompress_impl, mutates_args=(), device_types="cuda")
 
 
 @decompress_op.register_fake
@@ -346,10 +352,12 @@ def _(idx_bytes, vec_norms, table, bits, head_dim, out_dtype):
     return idx_bytes.new_empty((B, H, S, head_dim), dtype=out_dtype)
 
 
-@torch.library.custom_op("tqamd::decompress_into", mutates_args=("out",), device_types="cuda")
-def decompress_into_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
+def _decompress_into_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
                        out: torch.Tensor) -> None:
     decompress_into(idx_bytes, vec_norms, table, bits, out)
+
+
+decompress_into_op = torch.library.custom_op("tqamd::decompress_into", _decompress_into_impl, mutates_args=("out",), device_types="cuda")
 
 
 def _packed_rows(idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, int, int, int]:
@@ -362,8 +370,7 @@ def _packed_rows(idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> Tuple[torc
     return idx_bytes, vec_norms, prs, B * H, S
 
 
-@torch.library.custom_op("tqamd::scores_into", mutates_args=("scores",), device_types="cuda")
-def scores_into_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
+def _scores_into_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
                    q_rot: torch.Tensor, scores: torch.Tensor) -> None:
     """scores[b, h*G + g, t] = q_rot[b, h*G + g] . centroids[codes(b, h, t)] * norm(b, h, t), written into
     `scores` ([B, Hq, S] float32 view whose last dimension is dense and whose heads are equally spaced)."""
@@ -382,8 +389,10 @@ def scores_into_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torc
     check(rc, "tq_scores")
 
 
-@torch.library.custom_op("tqamd::weighted_values", mutates_args=(), device_types="cuda")
-def weighted_values_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
+scores_into_op = torch.library.custom_op("tqamd::scores_into", _scores_into_impl, mutates_args=("scores",), device_types="cuda")
+
+
+def _weighted_values_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
                        weights: torch.Tensor, head_dim: int) -> torch.Tensor:
     """out[b, h*G + g] = sum_t weights[b, h*G + g, t] * norm(b, h, t) * centroids[codes(b, h, t)]  (rotated space)."""
     _require_gpu(idx_bytes, "idx_bytes")
@@ -423,13 +432,15 @@ def weighted_values_op(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: 
     return out
 
 
+weighted_values_op = torch.library.custom_op("tqamd::weighted_values", _weighted_values_impl, mutates_args=(), device_types="cuda")
+
+
 @weighted_values_op.register_fake
 def _(idx_bytes, vec_norms, table, bits, weights, head_dim):
     return weights.new_empty((weights.shape[0], weights.shape[1], head_dim), dtype=torch.float32)
 
 
-@torch.library.custom_op("tqamd::attend_partials", mutates_args=(), device_types="cuda")
-def attend_partials_op(k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.Tensor, v_norms: torch.Tensor,
+def _attend_partials_impl(k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.Tensor, v_norms: torch.Tensor,
                        table_k: torch.Tensor, table_v: torch.Tensor, bits_k: int, bits_v: int,
                        q_rot: torch.Tensor) -> torch.Tensor:
     """One pass over packed keys and values of a [B,H,S,..] store pair: per (batch, query head, split)
@@ -455,13 +466,15 @@ def attend_partials_op(k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.
     return part.permute(0, 1, 3, 2, 4).reshape(B, Hq, splits, D + 2)
 
 
+attend_partials_op = torch.library.custom_op("tqamd::attend_partials", _attend_partials_impl, mutates_args=(), device_types="cuda")
+
+
 @attend_partials_op.register_fake
 def _(k_idx, k_norms, v_idx, v_norms, table_k, table_v, bits_k, bits_v, q_rot):
     return q_rot.new_empty((q_rot.shape[0], q_rot.shape[1], 1, q_rot.shape[2] + 2), dtype=torch.float32)
 
 
-@torch.library.custom_op("tqamd::attend_packed", mutates_args=(), device_types="cuda")
-def attend_packed_op(queries: torch.Tensor, k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.Tensor,
+def _attend_packed_impl(queries: torch.Tensor, k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.Tensor,
                      v_norms: torch.Tensor, table_k: torch.Tensor, table_v: torch.Tensor, bits_k: int, bits_v: int,
                      pi_k_t: torch.Tensor, pi_v: torch.Tensor, k_win: torch.Tensor, v_win: torch.Tensor,
                      scale: float) -> torch.Tensor:
@@ -515,6 +528,9 @@ def attend_packed_op(queries: torch.Tensor, k_idx: torch.Tensor, k_norms: torch.
     return out
 
 
+attend_packed_op = torch.library.custom_op("tqamd::attend_packed", _attend_packed_impl, mutates_args=(), device_types="cuda")
+
+
 @attend_packed_op.register_fake
 def _(queries, k_idx, k_norms, v_idx, v_norms, table_k, table_v, bits_k, bits_v, pi_k_t, pi_v, k_win, v_win, scale):
     return torch.empty_like(queries)
@@ -561,3 +577,18 @@ class JobList:
             rc = lib().tq_decompress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, HEAD_DIM,
                                              _stream_handle(self.device))
         check(rc, "tq_decompress_batched")
+
+
+# ------------------------------------------------------------------------------------
+# eager fast path
+# ------------------------------------------------------------------------------------
+_IMPL = {"compress": _compress_impl, "compress_into": _compress_into_impl, "decompress": _decompress_impl, "decompress_into": _decompress_into_impl, "scores_into": _scores_into_impl, "weighted_values": _weighted_values_impl, "attend_partials": _attend_partials_impl, "attend_packed": _attend_packed_impl}
+
+
+def call(name: str, *args):
+    """tqamd::<name>(*args).  In eager mode the Python implementation is called directly (the operator
+    dispatcher costs 20-30 us per call, more than the small launches of a decode step); while a compiler is
+    tracing, the registered operator is used so that the call stays one node of the graph."""
+    if torch.compiler.is_compiling():
+        return getattr(torch.ops.tqamd, name)(*args)
+    return _IMPL[name](*args)

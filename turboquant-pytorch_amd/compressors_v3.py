@@ -95,7 +95,7 @@ class MSECompressor:
         B, H, S, D = states.shape
         indices_per_byte = 8 // self.bits
         idx_pad = (indices_per_byte - D % indices_per_byte) % indices_per_byte
-        idx_bytes, vec_norms = torch.ops.tqamd.compress(states, self.table(), self.bits)
+        idx_bytes, vec_norms = _native.call("compress", states, self.table(), self.bits)
         return {
             "idx_bytes": idx_bytes,
             "vec_norms": vec_norms,
@@ -116,7 +116,7 @@ class MSECompressor:
         if idx_bytes.dtype != torch.uint8 or vec_norms.dtype != torch.float16:
             raise ValueError("packed buffers must be uint8 codes and float16 norms")
         if S * B * H:
-            torch.ops.tqamd.compress_into(states, self.table(), self.bits, idx_bytes, vec_norms)
+            _native.call("compress_into", states, self.table(), self.bits, idx_bytes, vec_norms)
 
     @torch.no_grad()
     def decompress_packed(self, idx_bytes: torch.Tensor, vec_norms: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -126,7 +126,7 @@ class MSECompressor:
             raise ValueError(f"packed buffers {tuple(idx_bytes.shape)} / {tuple(vec_norms.shape)} do not match "
                              f"output {tuple(out.shape)}")
         if S * B * H:
-            torch.ops.tqamd.decompress_into(idx_bytes, vec_norms, self.table(), self.bits, out)
+            _native.call("decompress_into", idx_bytes, vec_norms, self.table(), self.bits, out)
         return out
 
     @torch.no_grad()
@@ -145,7 +145,7 @@ class MSECompressor:
         if out is None:
             out = torch.empty((B, Hq, S), dtype=torch.float32, device=idx_bytes.device)
         if B * Hq * S:
-            torch.ops.tqamd.scores_into(idx_bytes, vec_norms, self.table(), self.bits, q_rot, out)
+            _native.call("scores_into", idx_bytes, vec_norms, self.table(), self.bits, q_rot, out)
         return out
 
     @torch.no_grad()
@@ -156,7 +156,7 @@ class MSECompressor:
         B, H, S, _ = idx_bytes.shape
         if S == 0:
             return torch.zeros((B, weights.shape[1], self.head_dim), dtype=torch.float32, device=idx_bytes.device)
-        out_rot = torch.ops.tqamd.weighted_values(idx_bytes, vec_norms, self.table(), self.bits, weights, self.head_dim)
+        out_rot = _native.call("weighted_values", idx_bytes, vec_norms, self.table(), self.bits, weights, self.head_dim)
         return torch.matmul(out_rot, self.Pi)
 
     @torch.no_grad()
@@ -166,7 +166,7 @@ class MSECompressor:
         width = math.ceil(D / (8 // self.bits))
         idx_bytes = compressed["idx_bytes"].reshape(B, H, S, width)
         vec_norms = compressed["vec_norms"].reshape(B, H, S)
-        return torch.ops.tqamd.decompress(idx_bytes, vec_norms, self.table(), self.bits, D, torch.float32)
+        return _native.call("decompress", idx_bytes, vec_norms, self.table(), self.bits, D, torch.float32)
 
     @torch.no_grad()
     def decompress_into(self, compressed: dict, out: torch.Tensor) -> torch.Tensor:
@@ -175,7 +175,7 @@ class MSECompressor:
         if tuple(out.shape) != (B, H, S, D):
             raise ValueError(f"output shape {tuple(out.shape)} does not match compressed shape {(B, H, S, D)}")
         width = math.ceil(D / (8 // self.bits))
-        torch.ops.tqamd.decompress_into(compressed["idx_bytes"].reshape(B, H, S, width),
+        _native.call("decompress_into", compressed["idx_bytes"].reshape(B, H, S, width),
                                         compressed["vec_norms"].reshape(B, H, S), self.table(), self.bits, out)
         return out
 

@@ -958,41 +958,62 @@ struct MergeArgs {
     int out_dtype;
 };
 
-// One block per packed row: log-sum-exp merge of the splits, rotation of the value sums back (x = y @ Pi),
-// the window's share, normalisation, cast.
-__global__ __launch_bounds__(256) void tq_attend_merge_kernel(MergeArgs a) {
-    constexpr int MAXG = 8;
-    __shared__ float rot[MAXG][TQ_HEAD_DIM];
-    __shared__ float den[MAXG], fw[MAXG];
-    const uint32_t row = blockIdx.x, tid = threadIdx.x, G = a.group, S = a.splits;
-    const TQ_GLOBAL float *part = (const TQ_GLOBAL float *)a.partial + (size_t)row * S * G * AT_PART;
-    const TQ_GLOBAL float *pw = a.part_w ? (const TQ_GLOBAL float *)a.part_w + (size_t)row * G * AT_PART : nullptr;
-    for (uint32_t o = tid; o < G * TQ_HEAD_DIM; o += 256u) {
-        const uint32_t g = o / TQ_HEAD_DIM, j = o % TQ_HEAD_DIM;
-        float m = pw ? pw[g * AT_PART] : -3.0e38f;
-        for (uint32_t s = 0; s < S; ++s) m = fmaxf(m, part[(s * G + g) * AT_PART]);
-        float acc = 0.f, l = 0.f;
-        for (uint32_t s = 0; s < S; ++s) {
-            const TQ_GLOBAL float *ps = part + (s * G + g) * AT_PART;
-            const float f = __expf(ps[0] - m);
-            acc = fmaf(f, ps[2 + j], acc);
-            l = fmaf(f, ps[1], l);
-        }
-        rot[g][j] = acc;
-        if (j == 0) {
-            const float f = pw ? __expf(pw[g * AT_PART] - m) : 0.f;
-            fw[g] = f;
-            den[g] = l + (pw ? f * pw[g * AT_PART + 1] : 0.f);
-        }
-    }
+// One block per (packed row, query head), 512 threads = (coordinate, quarter): log-sum-exp merge of the splits (each
+// quarter takes every fourth split, loads several splits ahead), rotation of the value sums back (x = y @ Pi, each
+// quarter a fourth of the contraction), the window's share, normalisation, cast.
+__global__ __launch_bounds__(512) void tq_attend_merge_kernel(MergeArgs a) {
+    __shared__ float red_m[8];
+    __shared__ float acc_q[4][TQ_HEAD_DIM];
+    __shared__ float l_q[4];
+    const uint32_t G = a.group, S = a.splits;
+    const uint32_t row = blockIdx.x / G, g = blockIdx.x % G;
+    const uint32_t tid = threadIdx.x, j = tid & 127u, q = tid >> 7, lane = tid & 63u, wave = tid >> 6;
+    const TQ_GLOBAL float *part = (const TQ_GLOBAL float *)a.partial + ((size_t)row * S * G + g) * AT_PART;   // split s at + s * G * AT_PART
+    const TQ_GLOBAL float *pw = a.part_w ? (const TQ_GLOBAL float *)a.part_w + ((size_t)row * G + g) * AT_PART : nullptr;
+    const size_t sstride = (size_t)G * AT_PART;
+    // 1. reference: the largest of the records' references
+    float m = pw ? pw[0] : -3.0e38f;
+    for (uint32_t s = tid; s < S; s += 512u) m = fmaxf(m, part[s * sstride]);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d));
+    if (lane == 0u) red_m[wave] = m;
     __syncthreads();
-    for (uint32_t o = tid; o < G * TQ_HEAD_DIM; o += 256u) {
-        const uint32_t g = o / TQ_HEAD_DIM, i = o % TQ_HEAD_DIM;
-        float x = 0.f;
-        for (int j = 0; j < TQ_HEAD_DIM; ++j) x = fmaf(rot[g][j], ((const TQ_GLOBAL float *)a.pi_v)[(size_t)j * TQ_HEAD_DIM + i], x);
-        if (pw) x = fmaf(fw[g], pw[g * AT_PART + 2 + i], x);
-        x /= den[g];
-        const size_t idx = (size_t)row * G * TQ_HEAD_DIM + o;
+    m = red_m[0];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) m = fmaxf(m, red_m[w]);
+    // 2. this quarter's splits
+    float acc = 0.f, l = 0.f;
+#pragma unroll 4
+    for (uint32_t s = q; s < S; s += 4u) {
+        const TQ_GLOBAL float *ps = part + s * sstride;
+        const float f = __expf(ps[0] - m);
+        acc = fmaf(f, ps[2 + j], acc);
+        l = fmaf(f, ps[1], l);
+    }
+    acc_q[q][j] = acc;
+    if (j == 0u) l_q[q] = l;
+    __syncthreads();
+    // 3. rotate back: this quarter's 32 terms of output coordinate i = j
+    float x = 0.f;
+#pragma unroll 8
+    for (uint32_t k = 32u * q; k < 32u * q + 32u; ++k) {
+        const float r = acc_q[0][k] + acc_q[1][k] + acc_q[2][k] + acc_q[3][k];
+        x = fmaf(r, ((const TQ_GLOBAL float *)a.pi_v)[(size_t)k * TQ_HEAD_DIM + j], x);
+    }
+    const float den_s = l_q[0] + l_q[1] + l_q[2] + l_q[3];
+    __syncthreads();                 // acc_q is reused for the quarters' partial rotations
+    acc_q[q][j] = x;
+    __syncthreads();
+    if (q == 0u) {
+        x = acc_q[0][j] + acc_q[1][j] + acc_q[2][j] + acc_q[3][j];
+        float den = den_s;
+        if (pw) {
+            const float f = __expf(pw[0] - m);
+            x = fmaf(f, pw[2 + j], x);
+            den = fmaf(f, pw[1], den);
+        }
+        x /= den;
+        const size_t idx = ((size_t)row * G + g) * TQ_HEAD_DIM + j;
         if (a.out_dtype == TQ_F32) {
             ((TQ_GLOBAL float *)a.out)[idx] = x;
         } else if (a.out_dtype == TQ_F16) {
@@ -1220,13 +1241,13 @@ extern "C" int tq_attend_prepare(const void *queries, int q_dtype, long long row
 
 extern "C" int tq_attend_merge(const float *partial, int splits, const float *part_w, const float *pi_v,
                                long long rows, int group, void *out, int out_dtype, void *stream) {
-    if (rows < 0 || rows > 0x7fffffff || group < 1 || group > 8 || splits < 0) return TQ_ERR_SIZE;
+    if (rows < 0 || rows > 0x7fffffff / 8 || group < 1 || group > 8 || splits < 0) return TQ_ERR_SIZE;    // one block per (row, head)
     if (out_dtype != TQ_F32 && out_dtype != TQ_F16 && out_dtype != TQ_BF16) return TQ_ERR_DTYPE;
     if (rows == 0) return TQ_OK;
     if (!pi_v || !out || (splits && !partial) || (!splits && !part_w)) return TQ_ERR_NULL;
     MergeArgs a;
     a.partial = partial; a.part_w = part_w; a.pi_v = pi_v; a.out = out;
     a.group = (uint32_t)group; a.splits = (uint32_t)splits; a.out_dtype = out_dtype;
-    hipLaunchKernelGGL(tq_attend_merge_kernel, dim3((unsigned)rows), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+    hipLaunchKernelGGL(tq_attend_merge_kernel, dim3((unsigned)(rows * group)), dim3(512), 0, static_cast<hipStream_t>(stream), a);
     return (int)hipGetLastError();
 }

@@ -24,6 +24,7 @@ from typing import Dict, Optional, Tuple
 
 import torch
 
+from . import _native
 from .compressors_v3 import TurboQuantV3
 
 
@@ -226,7 +227,7 @@ class V3Cache:
                 dev = query_states.device
                 packed = (torch.empty((B, st.H, 0, 1), dtype=torch.uint8, device=dev),
                           torch.empty((B, st.H, 0), dtype=torch.float16, device=dev)) * 2
-            return torch.ops.tqamd.attend_packed(query_states, *packed, kc.table(), vc.table(),
+            return _native.call("attend_packed", query_states, *packed, kc.table(), vc.table(),
                                                  kc.bits, vc.bits, kc.pi_transposed(), vc.Pi, kw, vw, float(scale))
         # rows padded to a multiple of 8 floats (the kernels read weights with 16-byte loads); the padding
         # scores are -inf, so the softmax runs over the whole contiguous buffer
