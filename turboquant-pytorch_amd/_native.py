@@ -317,7 +317,8 @@ def _compress_impl(states: torch.Tensor, table: torch.Tensor, bits: int) -> Tupl
     return idx_bytes, vec_norms
 
 
-compress_op = torch.library.custom_op("tqamd::compress", _compress_impl, mutates_args=(), device_types="cuda")
+compress_op = torch.library.custom_op("tqamd::compress", _compress_impl,
+                                      mutates_args=(), device_types="cuda")
 
 
 @compress_op.register_fake
@@ -328,22 +329,24 @@ def _(states, table, bits):
 
 
 def _compress_into_impl(states: torch.Tensor, table: torch.Tensor, bits: int,
-                     idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> None:
+                        idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> None:
     compress_into(states, table, bits, idx_bytes, vec_norms)
 
 
-compress_into_op = torch.library.custom_op("tqamd::compress_into", _compress_into_impl, mutates_args=("idx_bytes", "vec_norms"), device_types="cuda")
+compress_into_op = torch.library.custom_op("tqamd::compress_into", _compress_into_impl,
+                                           mutates_args=("idx_bytes", "vec_norms"), device_types="cuda")
 
 
 def _decompress_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
-                  head_dim: int, out_dtype: torch.dtype) -> torch.Tensor:
+                     head_dim: int, out_dtype: torch.dtype) -> torch.Tensor:
     B, H, S, _ = idx_bytes.shape
     out = torch.empty((B, H, S, head_dim), dtype=out_dtype, device=idx_bytes.device)
     decompress_into(idx_bytes, vec_norms, table, bits, out)
     return out
 
 
-decompress_op = torch.library.custom_op("tqamd::decompress", _decompress_impl, mutates_args=(), device_types="cuda")
+decompress_op = torch.library.custom_op("tqamd::decompress", _decompress_impl,
+                                        mutates_args=(), device_types="cuda")
 
 
 @decompress_op.register_fake
@@ -353,11 +356,12 @@ def _(idx_bytes, vec_norms, table, bits, head_dim, out_dtype):
 
 
 def _decompress_into_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
-                       out: torch.Tensor) -> None:
+                          out: torch.Tensor) -> None:
     decompress_into(idx_bytes, vec_norms, table, bits, out)
 
 
-decompress_into_op = torch.library.custom_op("tqamd::decompress_into", _decompress_into_impl, mutates_args=("out",), device_types="cuda")
+decompress_into_op = torch.library.custom_op("tqamd::decompress_into", _decompress_into_impl,
+                                             mutates_args=("out",), device_types="cuda")
 
 
 def _packed_rows(idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, int, int, int]:
@@ -371,7 +375,7 @@ def _packed_rows(idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> Tuple[torc
 
 
 def _scores_into_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
-                   q_rot: torch.Tensor, scores: torch.Tensor) -> None:
+                      q_rot: torch.Tensor, scores: torch.Tensor) -> None:
     """scores[b, h*G + g, t] = q_rot[b, h*G + g] . centroids[codes(b, h, t)] * norm(b, h, t), written into
     `scores` ([B, Hq, S] float32 view whose last dimension is dense and whose heads are equally spaced)."""
     _require_gpu(idx_bytes, "idx_bytes")
@@ -389,11 +393,12 @@ def _scores_into_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: t
     check(rc, "tq_scores")
 
 
-scores_into_op = torch.library.custom_op("tqamd::scores_into", _scores_into_impl, mutates_args=("scores",), device_types="cuda")
+scores_into_op = torch.library.custom_op("tqamd::scores_into", _scores_into_impl,
+                                         mutates_args=("scores",), device_types="cuda")
 
 
 def _weighted_values_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: torch.Tensor, bits: int,
-                       weights: torch.Tensor, head_dim: int) -> torch.Tensor:
+                          weights: torch.Tensor, head_dim: int) -> torch.Tensor:
     """out[b, h*G + g] = sum_t weights[b, h*G + g, t] * norm(b, h, t) * centroids[codes(b, h, t)]  (rotated space)."""
     _require_gpu(idx_bytes, "idx_bytes")
     idx_bytes, vec_norms, prs, rows, tokens = _packed_rows(idx_bytes, vec_norms)
@@ -432,7 +437,8 @@ def _weighted_values_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, tabl
     return out
 
 
-weighted_values_op = torch.library.custom_op("tqamd::weighted_values", _weighted_values_impl, mutates_args=(), device_types="cuda")
+weighted_values_op = torch.library.custom_op("tqamd::weighted_values", _weighted_values_impl,
+                                             mutates_args=(), device_types="cuda")
 
 
 @weighted_values_op.register_fake
@@ -441,8 +447,8 @@ def _(idx_bytes, vec_norms, table, bits, weights, head_dim):
 
 
 def _attend_partials_impl(k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.Tensor, v_norms: torch.Tensor,
-                       table_k: torch.Tensor, table_v: torch.Tensor, bits_k: int, bits_v: int,
-                       q_rot: torch.Tensor) -> torch.Tensor:
+                          table_k: torch.Tensor, table_v: torch.Tensor, bits_k: int, bits_v: int,
+                          q_rot: torch.Tensor) -> torch.Tensor:
     """One pass over packed keys and values of a [B,H,S,..] store pair: per (batch, query head, split)
     [largest score, sum of exp, 128 weighted sums in the value codec's rotated space] -> [B, Hq, splits, 130]."""
     _require_gpu(k_idx, "k_idx")
@@ -466,7 +472,8 @@ def _attend_partials_impl(k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: tor
     return part.permute(0, 1, 3, 2, 4).reshape(B, Hq, splits, D + 2)
 
 
-attend_partials_op = torch.library.custom_op("tqamd::attend_partials", _attend_partials_impl, mutates_args=(), device_types="cuda")
+attend_partials_op = torch.library.custom_op("tqamd::attend_partials", _attend_partials_impl,
+                                             mutates_args=(), device_types="cuda")
 
 
 @attend_partials_op.register_fake
@@ -475,9 +482,9 @@ def _(k_idx, k_norms, v_idx, v_norms, table_k, table_v, bits_k, bits_v, q_rot):
 
 
 def _attend_packed_impl(queries: torch.Tensor, k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.Tensor,
-                     v_norms: torch.Tensor, table_k: torch.Tensor, table_v: torch.Tensor, bits_k: int, bits_v: int,
-                     pi_k_t: torch.Tensor, pi_v: torch.Tensor, k_win: torch.Tensor, v_win: torch.Tensor,
-                     scale: float) -> torch.Tensor:
+                        v_norms: torch.Tensor, table_k: torch.Tensor, table_v: torch.Tensor, bits_k: int, bits_v: int,
+                        pi_k_t: torch.Tensor, pi_v: torch.Tensor, k_win: torch.Tensor, v_win: torch.Tensor,
+                        scale: float) -> torch.Tensor:
     """Decode-step attention of queries [B,Hq,1,D] over a packed history ([B,H,S,..] store slices, S may be 0)
     plus uncompressed window tokens [B,H,n_w,D] (n_w may be 0, not both): three launches."""
     _require_gpu(queries, "queries")
@@ -528,7 +535,8 @@ def _attend_packed_impl(queries: torch.Tensor, k_idx: torch.Tensor, k_norms: tor
     return out
 
 
-attend_packed_op = torch.library.custom_op("tqamd::attend_packed", _attend_packed_impl, mutates_args=(), device_types="cuda")
+attend_packed_op = torch.library.custom_op("tqamd::attend_packed", _attend_packed_impl,
+                                           mutates_args=(), device_types="cuda")
 
 
 @attend_packed_op.register_fake
@@ -582,7 +590,16 @@ class JobList:
 # ------------------------------------------------------------------------------------
 # eager fast path
 # ------------------------------------------------------------------------------------
-_IMPL = {"compress": _compress_impl, "compress_into": _compress_into_impl, "decompress": _decompress_impl, "decompress_into": _decompress_into_impl, "scores_into": _scores_into_impl, "weighted_values": _weighted_values_impl, "attend_partials": _attend_partials_impl, "attend_packed": _attend_packed_impl}
+_IMPL = {
+    "compress": _compress_impl,
+    "compress_into": _compress_into_impl,
+    "decompress": _decompress_impl,
+    "decompress_into": _decompress_into_impl,
+    "scores_into": _scores_into_impl,
+    "weighted_values": _weighted_values_impl,
+    "attend_partials": _attend_partials_impl,
+    "attend_packed": _attend_packed_impl,
+}
 
 
 def call(name: str, *args):
