@@ -474,3 +474,26 @@ def test_config3_shape_k6v4_window(pkg, oracle):
     mem = tq.memory_bytes(B, H, S)
     assert mem["compressed_tokens"] == 3968 and mem["fp16_tokens"] == 128 and mem["key_bits"] == 6 and mem["value_bits"] == 4
     assert mem["compressed_bytes"] == B * H * (3968 * (128 + 2 + 64 + 2) + 128 * D * 2 * 2)
+
+
+def test_operators_trace_under_a_compiler(pkg):
+    """The registered operators carry schemas and fake implementations: `torch.library.opcheck` accepts them, and a
+    compiled function (aot_eager backend: traced with fake tensors, executed with the real kernels) that goes
+    through MSECompressor.compress / decompress returns exactly what eager execution returns."""
+    comp = pkg.MSECompressor(128, 4, seed=5, device=DEV)
+    x = outlier_kv((1, 2, 96, 128), seed=91, dtype=torch.bfloat16).to(DEV)
+    table = comp.table()
+    for op, args in ((torch.ops.tqamd.compress.default, (x, table, 4)),):
+        torch.library.opcheck(op, args, test_utils=("test_schema", "test_faketensor"))
+    idx, nrm = torch.ops.tqamd.compress(x, table, 4)
+    torch.library.opcheck(torch.ops.tqamd.decompress.default, (idx, nrm, table, 4, 128, torch.bfloat16),
+                          test_utils=("test_schema", "test_faketensor"))
+
+    def round_trip(t):
+        c = comp.compress(t)
+        return comp.decompress(c), c["idx_bytes"], c["vec_norms"]
+
+    eager = round_trip(x)
+    compiled = torch.compile(round_trip, backend="aot_eager", fullgraph=True)(x)
+    for a, b in zip(eager, compiled):
+        assert torch.equal(a, b)
