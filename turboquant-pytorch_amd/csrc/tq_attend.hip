@@ -418,9 +418,11 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
     const uint32_t G = a.group;
     const bool live = n16 < G;
     // ---- B operand of the score product: fp16 of q * 2^(10 - e), e = binary exponent of the head's largest magnitude.
-    //      (One fp16 term: its rounding, 2^-12 relative per coordinate, is what the fp16 centroids of the decoded
-    //      keys already carry.)
+    //      One fp16 term for keys of up to 4 bits (its 2^-12 rounding per coordinate disappears under their
+    //      quantisation error); hi + lo for wider keys, where that launch is bound by memory and the term costs 1 %.
+    constexpr bool QLO = IPBK == 1;      // keys of 5 to 8 bits: a second term, the score then carries the keys' precision
     tq_u4 qb[4];
+    tq_u4 ql[QLO ? 4 : 1];
     float c1;                // score in base-2 units = t * c1, t = accumulator * key norm
     float rowscale;          // natural score = t * rowscale
     {
@@ -437,10 +439,15 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
         c1 = rowscale * 1.44269504088896341f;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            tq_half8 h;
+            tq_half8 h, l;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) h[i] = (_Float16)(live ? q[8 * s + i] * up : 0.f);
+            for (int i = 0; i < 8; ++i) {
+                const float x = live ? q[8 * s + i] * up : 0.f;
+                h[i] = (_Float16)x;
+                l[i] = (_Float16)(x - (float)h[i]);
+            }
             qb[s] = __builtin_bit_cast(tq_u4, h);
+            if constexpr (QLO) ql[s] = __builtin_bit_cast(tq_u4, l);
         }
     }
     __syncthreads();
@@ -520,6 +527,8 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
                 for (int s = 0; s < 4; ++s) {
                     const tq_half8 kd = __builtin_bit_cast(tq_half8, decode_rep<IPBK, NWK>(kraw[u][b], s, lut_k));
                     sc[u][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd, __builtin_bit_cast(tq_half8, qb[s]), sc[u][b], 0, 0, 0);
+                    if constexpr (QLO)
+                        sc[u][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd, __builtin_bit_cast(tq_half8, ql[s]), sc[u][b], 0, 0, 0);
                 }
             }
         }
