@@ -188,8 +188,8 @@ int tq_weighted_values(const uint8_t *idx_bytes, const uint16_t *vec_norms, long
  *       { m,  sum_t exp(score_t - m),  sum_t exp(score_t - m) * norm_t * centroid[code(t, j)] }
  * with score_t as tq_scores computes it (q_rot carries the softmax scale) and m a reference score of the split:
  * never above its largest score and at most 8 ln 2 below it (it follows the running maximum lazily).  The
- * rotated queries enter as one fp16 term per coordinate (relative rounding 2^-12, the precision the fp16
- * centroids of the decoded keys have).  The caller merges the splits
+ * rotated queries enter as one fp16 term per coordinate for keys of up to 4 bits (relative rounding 2^-12, the
+ * precision the fp16 centroids of the decoded keys have) and as fp16 hi + lo for wider keys.  The caller merges the splits
  * (and any uncompressed tokens) by the usual log-sum-exp rule and multiplies the 128 sums by Pi of the value
  * codec.  Keys and values share rows, tokens and packed_row_stride; group <= 8.  Same replaced reference
  * lines as tq_scores / tq_weighted_values.  tq_attend_splits suggests a split count.
