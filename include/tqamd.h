@@ -191,7 +191,7 @@ int tq_weighted_values(const uint8_t *idx_bytes, const uint16_t *vec_norms, long
  * rotated queries enter as one fp16 term per coordinate for keys of up to 4 bits (relative rounding 2^-12, the
  * precision the fp16 centroids of the decoded keys have) and as fp16 hi + lo for wider keys.  The caller merges the splits
  * (and any uncompressed tokens) by the usual log-sum-exp rule and multiplies the 128 sums by Pi of the value
- * codec.  Keys and values share rows, tokens and packed_row_stride; group <= 8.  Same replaced reference
+ * codec.  Keys and values share rows, tokens and packed_row_stride; group <= 16.  Same replaced reference
  * lines as tq_scores / tq_weighted_values.  tq_attend_splits suggests a split count.
  */
 int tq_attend_splits(long long rows, long long tokens);
@@ -205,7 +205,8 @@ int tq_attend_splits(long long rows, long long tokens);
  *                      of the packed part back by Pi_v, normalisation, cast -> out [rows, group, 128].
  * pi_k_t: device copy of the key codec's rotation, transposed (float32 [128,128], element [i][j] = Pi[j][i]);
  * pi_v: the value codec's rotation as MSECompressor keeps it (float32 [128,128] row-major).
- * k_win / v_win are 16-byte aligned and win_stride is a multiple of 8 (TQ_ERR_ALIGN otherwise).
+ * k_win / v_win are 16-byte aligned and win_stride is a multiple of 8 (TQ_ERR_ALIGN otherwise).  group <= 16
+ * in both.
  */
 int tq_attend_prepare(const void *queries, int q_dtype, long long rows, int group, float scale,
                       const float *pi_k_t, const void *k_win, const void *v_win, int win_dtype,

@@ -269,7 +269,7 @@ def test_v3cache_attend_equals_attention_over_the_cache(pkg, oracle, rw, dtype):
         b.attend(torch.zeros(B, H * G, 2, D, device=DEV), 0)
 
 
-@pytest.mark.parametrize("kb,vb,G,S", [(4, 2, 4, 1500), (8, 8, 8, 200), (2, 4, 1, 77), (3, 1, 2, 640), (6, 2, 8, 33)])
+@pytest.mark.parametrize("kb,vb,G,S", [(4, 2, 4, 1500), (8, 8, 8, 200), (2, 4, 1, 77), (3, 1, 2, 640), (6, 2, 8, 33), (4, 2, 16, 900), (8, 4, 13, 150)])
 def test_fused_attention_partials_against_oracle(pkg, oracle, kb, vb, G, S):
     """The one-pass kernel (scores, online softmax, weighted values per split) merged by the log-sum-exp rule
     equals float64 attention over the oracle-decoded packed keys and values; its records are consistent
@@ -340,7 +340,7 @@ def test_attend_with_window_only_and_without_window(pkg, oracle):
 
 @pytest.mark.parametrize("wdtype,qdtype,G,W,splits", [(torch.bfloat16, torch.bfloat16, 4, 128, 3), (torch.float16, torch.float16, 8, 512, 1),
                                                       (torch.float32, torch.float32, 1, 37, 2), (torch.bfloat16, torch.float32, 7, 1, 0),
-                                                      (torch.float16, torch.bfloat16, 3, 0, 4)])
+                                                      (torch.float16, torch.bfloat16, 3, 0, 4), (torch.bfloat16, torch.bfloat16, 16, 300, 2), (torch.float32, torch.float16, 11, 70, 1)])
 def test_attend_prepare_and_merge_against_float64(pkg, wdtype, qdtype, G, W, splits):
     """tq_attend_prepare / tq_attend_merge through the C-ABI against the same arithmetic in float64:
     rotated queries to 1e-5, window records to 1e-5, merged output to the output type's rounding."""
@@ -530,3 +530,26 @@ def test_fused_attention_over_extreme_value_norms(pkg, oracle):
         print(f"[fused attention] value-norm case {h}: relative L2 error {err:.2e}, |out| = {np.linalg.norm(ref[h]):.2e}")
         assert err < 3e-3
     assert np.all(got[2] == 0) and np.all(ref[2] == 0)
+
+
+def test_attend_with_sixteen_query_heads_per_kv_head(pkg, oracle):
+    """The widest group the one-pass path takes (128 query heads over 8 kv heads): same result as the three-step
+    form and as attention over the tensors update() returns."""
+    B, H, G, D = 1, 2, 16, 128
+    a = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=32, n_layers=1)
+    b = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=32, n_layers=1)
+    k = outlier_kv((B, H, 700, D), seed=900, dtype=torch.bfloat16).to(DEV)
+    v = outlier_kv((B, H, 700, D), seed=901, dtype=torch.bfloat16).to(DEV)
+    fk, fv = a.update(k, v, 0)
+    b.append(k, v, 0)
+    g = torch.Generator(device="cpu")
+    g.manual_seed(16)
+    q = (2 * torch.randn(B, H * G, 1, D, generator=g)).to(torch.bfloat16).to(DEV)
+    out = b.attend(q, 0)
+    three = b.attend(q, 0, fused=False)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.float(), fk.float().repeat_interleave(G, dim=1), fv.float().repeat_interleave(G, dim=1))
+    e1 = float((out.float() - three.float()).norm() / three.float().norm())
+    e2 = float((out.float() - ref).norm() / ref.norm())
+    print(f"[attend] 16 heads per kv head: vs three-step {e1:.2e}, vs attention over update() tensors {e2:.2e}")
+    assert e1 < 4e-3 and e2 < 1.5e-2

@@ -292,7 +292,7 @@ def test_c_abi_argument_errors(pkg):
     # the decode-step ends: (queries, q_dtype, rows, group, scale, pi_k_t, k_win, v_win, win_dtype, n_win, win_stride, q_rot, part_w)
     prep = lambda q=p, g=4, pit=p, kw=p, vw=p, wd=2, nw=8, ws=1024, qr=p, pw=p, rows=1, qd=2: lib.tq_attend_prepare(
         q, qd, rows, g, 0.5, pit, kw, vw, wd, nw, ws, qr, pw, None)
-    assert prep(g=0) == E["SIZE"] and prep(g=9) == E["SIZE"] and prep(nw=513) == E["SIZE"] and prep(nw=-1) == E["SIZE"]
+    assert prep(g=0) == E["SIZE"] and prep(g=17) == E["SIZE"] and prep(nw=513) == E["SIZE"] and prep(nw=-1) == E["SIZE"]
     assert prep(qd=5) == E["DTYPE"] and prep(wd=3) == E["DTYPE"]
     assert prep(rows=0) == 0
     assert prep(q=None) == E["NULL"] and prep(pit=None) == E["NULL"] and prep(qr=None) == E["NULL"]
@@ -300,7 +300,7 @@ def test_c_abi_argument_errors(pkg):
     assert prep(ws=512) == E["SIZE"]                       # rows of the window overlap
     assert prep(kw=p + 2) == E["ALIGN"] and prep(ws=1028) == E["ALIGN"]
     merge = lambda part=p, s=1, pw=p, piv=p, rows=1, g=4, out=p, od=2: lib.tq_attend_merge(part, s, pw, piv, rows, g, out, od, None)
-    assert merge(g=9) == E["SIZE"] and merge(s=-1) == E["SIZE"] and merge(od=4) == E["DTYPE"] and merge(rows=0) == 0
+    assert merge(g=17) == E["SIZE"] and merge(s=-1) == E["SIZE"] and merge(od=4) == E["DTYPE"] and merge(rows=0) == 0
     assert merge(piv=None) == E["NULL"] and merge(out=None) == E["NULL"] and merge(part=None) == E["NULL"]
     assert merge(part=None, s=0, pw=None) == E["NULL"]      # nothing to merge at all
 

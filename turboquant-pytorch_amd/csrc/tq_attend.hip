@@ -367,7 +367,7 @@ constexpr int AT_RUN = 64;       // tokens per wave and trip (32 when keys or va
 constexpr int AT_PART = TQ_HEAD_DIM + 2;
 
 // Block (split, row) of eight waves; a wave takes runs of 64 tokens of the split (staged one run ahead), a tile is 32
-// tokens = two blocks of 16, all matrix work is v_mfma_f32_16x16x32_f16 with the row's query heads (at most 8) padded
+// tokens = two blocks of 16, all matrix work is v_mfma_f32_16x16x32_f16 with the row's query heads (at most 16) padded
 // to 16 columns.  Lane (n16, q4) = (lane % 16, lane / 16).
 //   scores  S^T[token][head]: A = decoded keys, lane (token n16 of the block, q4) holds the 32 coordinates
 //     32 q4 .. 32 q4 + 31 of its token (KB contiguous packed bytes) and feeds 8 of them to each of 4 steps; B = rotated
@@ -397,13 +397,13 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
     constexpr int VPIECES = VBYTES / 16, NVP = (VPIECES + 63) / 64;
     constexpr int SLACK_LOG2 = 8;
     constexpr int P_SHIFT = 14 - SLACK_LOG2;             // p * 2^P_SHIFT * (value norm / 2^ev_ref < 2) <= 2^15 fits fp16
-    constexpr int AREA = VBYTES > 8 * AT_PART * 4 ? VBYTES : 8 * AT_PART * 4;   // staged value codes, later the wave's result
+    constexpr int AREA = VBYTES > 16 * AT_PART * 4 ? VBYTES : 16 * AT_PART * 4;  // staged value codes, later the wave's result (16 heads)
     __shared__ __attribute__((aligned(16))) uint8_t lds_lut_k[32768];
     __shared__ __attribute__((aligned(16))) uint8_t lds_lut_v[32768];
     __shared__ __attribute__((aligned(16))) uint8_t lds_area[AT_WAVES][AREA];
     __shared__ __attribute__((aligned(16))) float lds_kn[AT_WAVES][RUN];        // key norms as fp32
     __shared__ __attribute__((aligned(16))) uint16_t lds_vn[AT_WAVES][RUN];     // value norms / 2^ev_ref as fp16
-    __shared__ __attribute__((aligned(16))) float lds_corr[AT_WAVES][8];
+    __shared__ __attribute__((aligned(16))) float lds_corr[AT_WAVES][16];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t row = blockIdx.y, split = blockIdx.x;
@@ -557,10 +557,10 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
                 const float corr = __builtin_amdgcn_exp2f((m_ref - m_new) * c1);
                 l_run *= corr;
                 m_ref = m_new;
-                if (q4 == 0u && n16 < 8u) lds_corr[wave][n16] = corr;
+                if (q4 == 0u) lds_corr[wave][n16] = corr;
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
-                const float4 c4 = *reinterpret_cast<const float4 *>(&lds_corr[wave][4u * (q4 & 1u)]);
+                const float4 c4 = *reinterpret_cast<const float4 *>(&lds_corr[wave][4u * q4]);
                 asm volatile("" ::: "memory");
 #pragma unroll
                 for (int c = 0; c < 8; ++c) {
@@ -664,17 +664,17 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
         }
     }
     asm volatile("" ::: "memory");
-    // ---- this wave's result for heads 0..7: [head][largest natural score, sum, 128 sums] in its LDS area
+    // ---- this wave's result for heads 0..15: [head][largest natural score, sum, 128 sums] in its LDS area
     float *res = reinterpret_cast<float *>(lds_area[wave]);
     {
         float l_all = l_run + __shfl_xor(l_run, 16);
         l_all = (l_all + __shfl_xor(l_all, 32)) * (1.0f / (float)(1 << P_SHIFT));
-        if (q4 == 0u && n16 < 8u) {
+        if (q4 == 0u) {
             res[n16 * AT_PART + 0] = m_ref * rowscale;
             res[n16 * AT_PART + 1] = l_all;
         }
         const float out_scale = ldexpf(1.f, ev_ref - P_SHIFT);
-        if (q4 < 2u) {
+        {
 #pragma unroll
             for (int c = 0; c < 8; ++c)
 #pragma unroll
@@ -768,7 +768,7 @@ __device__ __forceinline__ float tq_row_sum16(float x) {
 
 // One block per packed row (batch x kv head), four waves.  Rotates the row's query heads for the packed keys and
 // computes attention statistics over the uncompressed window tokens in fp32 (a few hundred tokens at most).
-// GP = heads per row rounded up to 1, 2, 4 or 8: the padding heads are zero queries, so no loop tests the head count.
+// GP = heads per row rounded up to 1, 2, 4, 8 or 16: the padding heads are zero queries, so no loop tests the head count.
 // The loads of the first 128 window tokens, keys and values, are issued before anything else: the kernel waits for
 // memory once.
 //   rotation   : thread (j, half) sums 64 of the 128 terms of every head's q_rot[j]; Pi^T is read once, coalesced
@@ -779,7 +779,7 @@ __device__ __forceinline__ float tq_row_sum16(float x) {
 //                wave meet through one exchange, the four waves in LDS
 template <int WD, int GP>
 __global__ __launch_bounds__(256) void tq_attend_prepare_kernel(PrepareArgs a) {
-    constexpr int MAXG = 8, MAXW = 512;
+    constexpr int MAXG = 16, MAXW = 512;
     constexpr int PRE_K = 2;      // key trips (64 tokens each) loaded up front
     constexpr int PRE_V = 4;      // value trips (32 tokens each) loaded up front
     constexpr int VW = WD == TQ_F32 ? 4 : 2;             // dwords per four value elements
@@ -847,9 +847,10 @@ __global__ __launch_bounds__(256) void tq_attend_prepare_kernel(PrepareArgs a) {
 #pragma unroll 16
         for (int i = 0; i < 64; ++i) {
             const float p = pc[(size_t)i * TQ_HEAD_DIM];
-            float qv[8];
-            *reinterpret_cast<float4 *>(&qv[0]) = *reinterpret_cast<const float4 *>(&qt[half * 64u + i][0]);
-            if constexpr (GP > 4) *reinterpret_cast<float4 *>(&qv[4]) = *reinterpret_cast<const float4 *>(&qt[half * 64u + i][4]);
+            float qv[MAXG];
+#pragma unroll
+            for (int h = 0; h < (GP + 3) / 4; ++h)
+                *reinterpret_cast<float4 *>(&qv[4 * h]) = *reinterpret_cast<const float4 *>(&qt[half * 64u + i][4 * h]);
 #pragma unroll
             for (int g = 0; g < GP; ++g) s[g] = fmaf(p, qv[g], s[g]);
         }
@@ -1192,7 +1193,7 @@ extern "C" int tq_attend_partials(const uint8_t *k_idx, const uint16_t *k_norms,
     if (rc) return rc;
     rc = check_packed(v_idx, v_norms, packed_row_stride, rows, tokens, table_v, head_dim, bits_v);
     if (rc) return rc;
-    if (group < 1 || group > 8 || splits < 1 || splits > 65535) return TQ_ERR_SIZE;
+    if (group < 1 || group > 16 || splits < 1 || splits > 65535) return TQ_ERR_SIZE;
     if (rows == 0 || tokens == 0) return TQ_ERR_SIZE;          // nothing to attend to: the caller handles it
     if (!q_rot || !partial) return TQ_ERR_NULL;
     if (((uintptr_t)q_rot & 3u) || ((uintptr_t)partial & 3u)) return TQ_ERR_ALIGN;
@@ -1220,7 +1221,7 @@ extern "C" int tq_attend_partials(const uint8_t *k_idx, const uint16_t *k_norms,
 extern "C" int tq_attend_prepare(const void *queries, int q_dtype, long long rows, int group, float scale,
                                  const float *pi_k_t, const void *k_win, const void *v_win, int win_dtype,
                                  long long n_win, long long win_stride, float *q_rot, float *part_w, void *stream) {
-    if (rows < 0 || rows > 0x7fffffff || group < 1 || group > 8 || n_win < 0 || n_win > 512) return TQ_ERR_SIZE;
+    if (rows < 0 || rows > 0x7fffffff || group < 1 || group > 16 || n_win < 0 || n_win > 512) return TQ_ERR_SIZE;
     if ((q_dtype != TQ_F32 && q_dtype != TQ_F16 && q_dtype != TQ_BF16) ||
         (n_win && win_dtype != TQ_F32 && win_dtype != TQ_F16 && win_dtype != TQ_BF16)) return TQ_ERR_DTYPE;
     if (rows == 0) return TQ_OK;
@@ -1237,20 +1238,20 @@ extern "C" int tq_attend_prepare(const void *queries, int q_dtype, long long row
     a.q_dtype = q_dtype; a.win_dtype = win_dtype;
     const hipStream_t st = static_cast<hipStream_t>(stream);
     const int wd = n_win ? win_dtype : TQ_BF16;
-    const int gp = group > 4 ? 8 : group > 2 ? 4 : group;
+    const int gp = group > 8 ? 16 : group > 4 ? 8 : group > 2 ? 4 : group;
     const dim3 grid((unsigned)rows), block(256);
 #define TQ_PREP_CASE(WD, GP) \
     if (wd == WD && gp == GP) hipLaunchKernelGGL((tq_attend_prepare_kernel<WD, GP>), grid, block, 0, st, a)
-    TQ_PREP_CASE(TQ_F32, 1); TQ_PREP_CASE(TQ_F32, 2); TQ_PREP_CASE(TQ_F32, 4); TQ_PREP_CASE(TQ_F32, 8);
-    TQ_PREP_CASE(TQ_F16, 1); TQ_PREP_CASE(TQ_F16, 2); TQ_PREP_CASE(TQ_F16, 4); TQ_PREP_CASE(TQ_F16, 8);
-    TQ_PREP_CASE(TQ_BF16, 1); TQ_PREP_CASE(TQ_BF16, 2); TQ_PREP_CASE(TQ_BF16, 4); TQ_PREP_CASE(TQ_BF16, 8);
+    TQ_PREP_CASE(TQ_F32, 1); TQ_PREP_CASE(TQ_F32, 2); TQ_PREP_CASE(TQ_F32, 4); TQ_PREP_CASE(TQ_F32, 8); TQ_PREP_CASE(TQ_F32, 16);
+    TQ_PREP_CASE(TQ_F16, 1); TQ_PREP_CASE(TQ_F16, 2); TQ_PREP_CASE(TQ_F16, 4); TQ_PREP_CASE(TQ_F16, 8); TQ_PREP_CASE(TQ_F16, 16);
+    TQ_PREP_CASE(TQ_BF16, 1); TQ_PREP_CASE(TQ_BF16, 2); TQ_PREP_CASE(TQ_BF16, 4); TQ_PREP_CASE(TQ_BF16, 8); TQ_PREP_CASE(TQ_BF16, 16);
 #undef TQ_PREP_CASE
     return (int)hipGetLastError();
 }
 
 extern "C" int tq_attend_merge(const float *partial, int splits, const float *part_w, const float *pi_v,
                                long long rows, int group, void *out, int out_dtype, void *stream) {
-    if (rows < 0 || rows > 0x7fffffff / 8 || group < 1 || group > 8 || splits < 0) return TQ_ERR_SIZE;    // one block per (row, head)
+    if (rows < 0 || rows > 0x7fffffff / 16 || group < 1 || group > 16 || splits < 0) return TQ_ERR_SIZE;    // one block per (row, head)
     if (out_dtype != TQ_F32 && out_dtype != TQ_F16 && out_dtype != TQ_BF16) return TQ_ERR_DTYPE;
     if (rows == 0) return TQ_OK;
     if (!pi_v || !out || (splits && !partial) || (!splits && !part_w)) return TQ_ERR_NULL;

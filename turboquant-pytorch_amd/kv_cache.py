@@ -202,7 +202,7 @@ class V3Cache:
         """softmax(scale * q K^T) V of one query token per sequence, [B,Hq,1,D] -> [B,Hq,1,D], over everything
         cached for the layer -- what the model computes from the tensors `update` returns -- read
         straight from the packed store.  Query head j uses kv head j // (Hq / H).
-        fused (default: whenever at most 8 query heads share a kv head): one kernel pass over packed keys and
+        fused (default: whenever at most 16 query heads share a kv head): one kernel pass over packed keys and
         values with an online softmax per split of the history; otherwise three steps (scores from the packed
         keys, softmax in float32, weighted sum of the packed values).  Window tokens are used as they are."""
         st = self._stores.get(layer_idx)
@@ -216,7 +216,7 @@ class V3Cache:
         n_c, n_w = st.n_compressed, st.n_recent
         kc, vc = st.comp.key_compressor, st.comp.val_compressor
         if fused is None:
-            fused = G <= 8
+            fused = G <= 16
         kw, vw = st.window()
         if fused and n_w <= 512:
             # three launches: rotate the queries + window statistics, one pass over the packed history,
