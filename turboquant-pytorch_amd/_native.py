@@ -254,8 +254,32 @@ def packed_row_stride(idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> Optio
     return sh // G
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)     # what torch's own launchers use: no Stream object
+
+
 def _stream_handle(device: torch.device) -> int:
+    """The current HIP stream of `device` as an integer handle."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoScope:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SCOPE = _NoScope()
+
+
+def _on(device: torch.device):
+    """Context that makes `device` current for a launch; free when it already is (the usual case)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SCOPE
+    return torch.cuda.device(device)
 
 
 def compress_into(states: torch.Tensor, table: torch.Tensor, bits: int,
@@ -272,7 +296,7 @@ def compress_into(states: torch.Tensor, table: torch.Tensor, bits: int,
         states = states.contiguous()
         lay = row_layout(states) if prs else vector_layout(states)
     rows, tokens, row_stride, token_stride = lay
-    with torch.cuda.device(states.device):
+    with _on(states.device):
         rc = lib().tq_compress(states.data_ptr(), dtype_code(states.dtype), rows, tokens, row_stride, token_stride,
                                table.data_ptr(), states.shape[-1], bits,
                                idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, _stream_handle(states.device))
@@ -293,7 +317,7 @@ def decompress_into(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: tor
         raise TqError("decompress output must have a dense last dimension, 16-byte aligned rows and at most "
                       "two stride levels")
     rows, tokens, row_stride, token_stride = lay
-    with torch.cuda.device(out.device):
+    with _on(out.device):
         rc = lib().tq_decompress(idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, rows, tokens, table.data_ptr(),
                                  out.shape[-1], bits, out.data_ptr(), dtype_code(out.dtype), row_stride,
                                  token_stride, _stream_handle(out.device))
@@ -387,7 +411,7 @@ def _scores_into_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: t
         raise TqError("scores must be a float32 [B, Hq, S] view with a dense last dimension and evenly spaced heads")
     q_rot = q_rot.to(torch.float32).contiguous()
     stride = scores.stride(1) if Hq > 1 else (scores.stride(0) if B > 1 else max(tokens, 1))
-    with torch.cuda.device(idx_bytes.device):
+    with _on(idx_bytes.device):
         rc = lib().tq_scores(idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, rows, tokens, table.data_ptr(), D, bits,
                              q_rot.data_ptr(), group, scores.data_ptr(), stride, _stream_handle(idx_bytes.device))
     check(rc, "tq_scores")
@@ -413,7 +437,7 @@ def _weighted_values_impl(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, tabl
     L = lib()
     splits = L.tq_weighted_values_splits(rows, tokens)
     step = 8                                             # query heads per kv head and launch
-    with torch.cuda.device(idx_bytes.device):
+    with _on(idx_bytes.device):
         if group <= step:
             partial = torch.empty((rows, splits, group, head_dim), dtype=torch.float32, device=idx_bytes.device)
             rc = L.tq_weighted_values(idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, rows, tokens, table.data_ptr(),
@@ -464,7 +488,7 @@ def _attend_partials_impl(k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: tor
     L = lib()
     splits = L.tq_attend_splits(B * H, S)
     part = torch.empty((B, H, splits, group, D + 2), dtype=torch.float32, device=k_idx.device)
-    with torch.cuda.device(k_idx.device):
+    with _on(k_idx.device):
         rc = L.tq_attend_partials(k_idx.data_ptr(), k_norms.data_ptr(), v_idx.data_ptr(), v_norms.data_ptr(), prs_k,
                                   B * H, S, table_k.data_ptr(), table_v.data_ptr(), D, bits_k, bits_v,
                                   q_rot.data_ptr(), group, splits, part.data_ptr(), _stream_handle(k_idx.device))
@@ -510,7 +534,7 @@ def _attend_packed_impl(queries: torch.Tensor, k_idx: torch.Tensor, k_norms: tor
             lay_k = row_layout(k_win)
         win_stride = lay_k[2] if rows > 1 else n_w * D
     out = torch.empty((B, Hq, 1, D), dtype=queries.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = L.tq_attend_prepare(q.data_ptr(), dtype_code(q.dtype), rows, group, scale, pi_k_t.data_ptr(),
                                  k_win.data_ptr() if n_w else None, v_win.data_ptr() if n_w else None,
                                  dtype_code(k_win.dtype) if n_w else 0, n_w, win_stride, q_rot.data_ptr(),
@@ -575,13 +599,13 @@ class JobList:
         self.dev = torch.from_numpy(raw).to(self.device)
 
     def compress(self) -> None:
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             rc = lib().tq_compress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, HEAD_DIM,
                                            _stream_handle(self.device))
         check(rc, "tq_compress_batched")
 
     def decompress(self) -> None:
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             rc = lib().tq_decompress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, HEAD_DIM,
                                              _stream_handle(self.device))
         check(rc, "tq_decompress_batched")
