@@ -790,7 +790,9 @@ __global__ __launch_bounds__(256) void tq_attend_prepare_kernel(PrepareArgs a) {
     const uint32_t row = blockIdx.x, tid = threadIdx.x, G = a.group, lane = tid & 63u, wave = tid >> 6;
     const uint32_t sub = lane & 15u, tk = lane >> 4;          // key side: elements 8 sub .., token slot tk of 4
     const uint32_t sub5 = lane & 31u, tk5 = lane >> 5;        // value side: columns 4 sub5 .., token slot tk5 of 2
-    const uint32_t W = a.part_w ? a.n_win : 0u;
+    // grid.y = 2 when there is a window: blocks (row, 0) rotate the queries, blocks (row, 1) take the window, side by side
+    const bool do_rot = blockIdx.y == 0u, do_win = gridDim.y == 1u || blockIdx.y == 1u;
+    const uint32_t W = (a.part_w && do_win) ? a.n_win : 0u;
     const size_t win_base = (size_t)row * a.win_stride;
     // past the end the last token is read again and not used
     auto ktoken = [&](uint32_t trip, int k) { return 64u * trip + 16u * wave + 4u * (uint32_t)k + tk; };
@@ -838,7 +840,7 @@ __global__ __launch_bounds__(256) void tq_attend_prepare_kernel(PrepareArgs a) {
         qt[c][g] = i < G * TQ_HEAD_DIM ? tq_load_elem(a.queries, (size_t)row * G * TQ_HEAD_DIM + i, a.q_dtype) * a.scale : 0.f;
     }
     __syncthreads();
-    {   // rotated queries: q_rot[g][j] = sum_i Pi[j][i] * q[g][i]; all heads of a coordinate come with 16-byte reads
+    if (do_rot) {   // rotated queries: q_rot[g][j] = sum_i Pi[j][i] * q[g][i]; all heads of a coordinate come with 16-byte reads
         const uint32_t j = tid & 127u, half = tid >> 7;
         const TQ_GLOBAL float *pc = (const TQ_GLOBAL float *)a.pi_k_t + (size_t)half * 64u * TQ_HEAD_DIM + j;
         float s[GP];
@@ -858,9 +860,10 @@ __global__ __launch_bounds__(256) void tq_attend_prepare_kernel(PrepareArgs a) {
         for (int g = 0; g < GP; ++g) part[half][g][j] = s[g];
     }
     __syncthreads();
-    for (uint32_t o = tid; o < G * TQ_HEAD_DIM; o += 256u)
-        ((TQ_GLOBAL float *)a.q_rot)[(size_t)row * G * TQ_HEAD_DIM + o] =
-            part[0][o / TQ_HEAD_DIM][o % TQ_HEAD_DIM] + part[1][o / TQ_HEAD_DIM][o % TQ_HEAD_DIM];
+    if (do_rot)
+        for (uint32_t o = tid; o < G * TQ_HEAD_DIM; o += 256u)
+            ((TQ_GLOBAL float *)a.q_rot)[(size_t)row * G * TQ_HEAD_DIM + o] =
+                part[0][o / TQ_HEAD_DIM][o % TQ_HEAD_DIM] + part[1][o / TQ_HEAD_DIM][o % TQ_HEAD_DIM];
     if (!W) return;
     {   // scores of the window tokens
         const uint32_t trips = (W + 63u) / 64u;
@@ -1239,7 +1242,7 @@ extern "C" int tq_attend_prepare(const void *queries, int q_dtype, long long row
     const hipStream_t st = static_cast<hipStream_t>(stream);
     const int wd = n_win ? win_dtype : TQ_BF16;
     const int gp = group > 8 ? 16 : group > 4 ? 8 : group > 2 ? 4 : group;
-    const dim3 grid((unsigned)rows), block(256);
+    const dim3 grid((unsigned)rows, n_win ? 2u : 1u), block(256);
 #define TQ_PREP_CASE(WD, GP) \
     if (wd == WD && gp == GP) hipLaunchKernelGGL((tq_attend_prepare_kernel<WD, GP>), grid, block, 0, st, a)
     TQ_PREP_CASE(TQ_F32, 1); TQ_PREP_CASE(TQ_F32, 2); TQ_PREP_CASE(TQ_F32, 4); TQ_PREP_CASE(TQ_F32, 8); TQ_PREP_CASE(TQ_F32, 16);
