@@ -474,18 +474,20 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
     uint32_t kraw_buf[2][SUB][2][NWK];
     tq_u4 vpiece_buf[2][NVP];
     uint16_t kn_buf[2] = {0, 0}, vn_buf[2] = {0, 0};
-    auto issue_loads = [&](auto bsel, uint32_t t0) __attribute__((always_inline)) {
+    // FULL: the run has all its tokens, so no address is clamped and the arithmetic folds into constants
+    auto issue_loads = [&](auto bsel, auto full_tag, uint32_t t0) __attribute__((always_inline)) {
         constexpr int B = decltype(bsel)::value;
+        constexpr bool FULL = decltype(full_tag)::value;
         auto &kraw_next = kraw_buf[B];
         auto &vpiece_next = vpiece_buf[B];
         uint16_t &kn_next = kn_buf[B], &vn_next = vn_buf[B];
-        const uint32_t n_tok = min((uint32_t)RUN, t_end - t0);
+        const uint32_t n_tok = FULL ? (uint32_t)RUN : min((uint32_t)RUN, t_end - t0);
 #pragma unroll
         for (int u = 0; u < SUB; ++u)
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
                 const uint32_t tl = 32u * u + 16u * b + n16;
-                const uint8_t *src = a.k_idx + (slot0 + t0 + (tl < n_tok ? tl : 0u)) * (4 * KB) + q4 * KB;
+                const uint8_t *src = a.k_idx + (slot0 + t0 + ((FULL || tl < n_tok) ? tl : 0u)) * (4 * KB) + q4 * KB;
                 if constexpr (KB == 4) {
                     kraw_next[u][b][0] = *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)src);
                 } else if constexpr (KB == 8) {
@@ -504,7 +506,7 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
 #pragma unroll
         for (int p = 0; p < NVP; ++p) {
             const uint32_t piece = p * 64u + lane;
-            const bool ok = piece < VPIECES && piece * 16u < n_tok * GBV;
+            const bool ok = piece < VPIECES && (FULL || piece * 16u < n_tok * GBV);
             vpiece_next[p] = tq_gload16(vsrc + (ok ? piece : 0u) * 16u);
         }
         kn_next = lane < n_tok ? tq_gload2(a.k_norms + slot0 + t0 + lane) : (uint16_t)0;
@@ -622,16 +624,17 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
         {
             const _Float16 kh = __builtin_bit_cast(_Float16, kn_buf[B]);
             if (RUN == 64 || lane < (uint32_t)RUN) lds_kn[wave][lane] = (float)kh;     // one token per lane
-            // largest exponent field of the run's value norms: row-wise running maximum, then the four row ends
+            // does a value norm of this run exceed the reference exponent?  (a vote; a handful of times per wave)
             uint32_t e = ((uint32_t)vn_buf[B] >> 10) & 31u;
-            e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x111, 0xf, 0xf, true));
-            e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x112, 0xf, 0xf, true));
-            e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x114, 0xf, 0xf, true));
-            e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x118, 0xf, 0xf, true));
-            const uint32_t emax = max(max((uint32_t)__builtin_amdgcn_readlane((int)e, 15), (uint32_t)__builtin_amdgcn_readlane((int)e, 31)),
-                                      max((uint32_t)__builtin_amdgcn_readlane((int)e, 47), (uint32_t)__builtin_amdgcn_readlane((int)e, 63)));
-            const int ev = (int)max(emax, 1u) - 15;
-            if (ev > ev_ref) {                       // uniform; a handful of times per wave
+            if (__any((int)max(e, 1u) - 15 > ev_ref)) {
+                // largest exponent field of the run: row-wise running maximum, then the four row ends
+                e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x111, 0xf, 0xf, true));
+                e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x112, 0xf, 0xf, true));
+                e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x114, 0xf, 0xf, true));
+                e = max(e, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e, 0x118, 0xf, 0xf, true));
+                const uint32_t emax = max(max((uint32_t)__builtin_amdgcn_readlane((int)e, 15), (uint32_t)__builtin_amdgcn_readlane((int)e, 31)),
+                                          max((uint32_t)__builtin_amdgcn_readlane((int)e, 47), (uint32_t)__builtin_amdgcn_readlane((int)e, 63)));
+                const int ev = (int)max(emax, 1u) - 15;
                 const float f = ldexpf(1.f, ev_ref - ev);
 #pragma unroll
                 for (int c = 0; c < 8; ++c) acc[c] *= f;
@@ -642,7 +645,8 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
             if (RUN == 64 || lane < (uint32_t)RUN) lds_vn[wave][lane] = __builtin_bit_cast(uint16_t, vs);
         }
         const uint32_t t_next = t0 + RUN * AT_WAVES;
-        if (t_next < t_end) issue_loads(std::integral_constant<int, 1 - B>{}, t_next);
+        if (t_next + RUN <= t_end) issue_loads(std::integral_constant<int, 1 - B>{}, std::true_type{}, t_next);
+        else if (t_next < t_end) issue_loads(std::integral_constant<int, 1 - B>{}, std::false_type{}, t_next);
         asm volatile("" ::: "memory");    // staged with one access width, read back with others (LDS serves a wave in order)
         __builtin_amdgcn_wave_barrier();
         if (n_tok == RUN) run(std::true_type{}, kraw_buf[B], n_tok);
@@ -654,7 +658,7 @@ __global__ __launch_bounds__(AT_WAVES *TQ_WAVE, AT_WAVES / 4) void tq_attend_ker
     {
         uint32_t t0 = t_begin + RUN * wave;
         if (t0 < t_end) {
-            issue_loads(std::integral_constant<int, 0>{}, t0);
+            issue_loads(std::integral_constant<int, 0>{}, std::false_type{}, t0);
             for (;;) {
                 t0 = trip(std::integral_constant<int, 0>{}, t0);
                 if (t0 >= t_end) break;
