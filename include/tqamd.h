@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define TQ_ABI_VERSION 2
+#define TQ_ABI_VERSION 3
 
 /* element types of K/V tensors */
 enum { TQ_F32 = 0, TQ_F16 = 1, TQ_BF16 = 2 };
@@ -120,12 +120,25 @@ int tq_compress(const void *states, int dtype, long long rows, long long tokens,
  *   (n / tokens) * row_stride + (n % tokens) * token_stride   of `out`
  * and read from packed slot (n / tokens) * packed_row_stride + (n % tokens) (0 = dense), which
  * also covers the loop over stored chunks of generation_test_v2.py:131-135.
+ *
+ *   workspace   device memory of tq_workspace_bytes(1) bytes, 64-byte aligned, or NULL.  It holds the
+ *               counter from which the kernel's blocks draw their tiles in the order in which they
+ *               become free, which keeps the output addresses written at any moment close together
+ *               (measurably faster than a fixed assignment of tiles to blocks on large jobs; the
+ *               results are the same bytes).  Contract: all zero before its first use; every launch
+ *               that completes leaves it all zero again; two launches that can overlap in time
+ *               (different streams) must not share one.  NULL selects the fixed assignment.
  */
+#define TQ_MAX_JOBS 4096               /* most jobs one batched launch takes */
+#define TQ_WORKSPACE_BYTES_PER_JOB 256
+/* bytes of workspace for a launch of n_jobs jobs (n_jobs = 1 for tq_decompress); TQ_ERR_SIZE if n_jobs < 0 or > TQ_MAX_JOBS */
+long long tq_workspace_bytes(int n_jobs);
+
 int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long packed_row_stride,
                   long long rows, long long tokens,
                   const void *table_dev, int head_dim, int bits,
                   void *out, int out_dtype, long long row_stride, long long token_stride,
-                  void *stream);
+                  void *workspace, void *stream);
 
 /*
  * Batched forms: one launch for many (layer, tensor) jobs, each with its own table.
@@ -135,6 +148,8 @@ int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long
  * `jobs_host` is read for validation and launch sizing; `jobs_dev` is a device copy of the
  * same n_jobs records that the kernel reads -- the caller uploads it once and may reuse it
  * for every call with the same buffers (nothing is allocated here).
+ * tq_decompress_batched takes a workspace of tq_workspace_bytes(n_jobs) bytes under the contract
+ * stated at tq_decompress (job i uses bytes [i * TQ_WORKSPACE_BYTES_PER_JOB, ...)), or NULL.
  */
 typedef struct tq_job {
     const void *states;        /* compress: input vectors;   decompress: output vectors   */
@@ -149,12 +164,10 @@ typedef struct tq_job {
     long long packed_row_stride; /* packed slots per row of idx_bytes / vec_norms; 0 = tokens */
 } tq_job;
 
-#define TQ_MAX_JOBS 4096
-
 int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
                         int head_dim, void *stream);
 int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
-                          int head_dim, void *stream);
+                          int head_dim, void *workspace, void *stream);
 
 /*
  * Decode-time attention on the packed cache, without de-quantising it.  Replaces, for single-token

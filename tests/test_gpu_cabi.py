@@ -48,9 +48,16 @@ def test_raw_binding_round_trip(tq, oracle, bits, dtype):
     rc = lib.tq_compress(_p(x), DT[dtype], ll(1), ll(B * H * S), ll(0), ll(D), _p(table), D, bits, _p(idx), _p(nrm), ll(0), stream)
     assert rc == 0, lib.tq_status_string(rc)
     out = torch.empty(B, H, S, D, dtype=torch.float32, device=DEV)
-    rc = lib.tq_decompress(_p(idx), _p(nrm), ll(0), ll(1), ll(B * H * S), _p(table), D, bits, _p(out), 0, ll(0), ll(D), stream)
+    rc = lib.tq_decompress(_p(idx), _p(nrm), ll(0), ll(1), ll(B * H * S), _p(table), D, bits, _p(out), 0, ll(0), ll(D), None, stream)
+    assert rc == 0, lib.tq_status_string(rc)
+    # with a workspace (zero before, zero after) the same bytes come out
+    lib.tq_workspace_bytes.restype = ctypes.c_longlong
+    ws = torch.zeros(lib.tq_workspace_bytes(1), dtype=torch.uint8, device=DEV)
+    out_ws = torch.empty_like(out)
+    rc = lib.tq_decompress(_p(idx), _p(nrm), ll(0), ll(1), ll(B * H * S), _p(table), D, bits, _p(out_ws), 0, ll(0), ll(D), _p(ws), stream)
     assert rc == 0, lib.tq_status_string(rc)
     torch.cuda.synchronize()
+    assert torch.equal(out, out_ws) and int(ws.sum()) == 0
     orc = oracle.COracle(pi, cent, bits, accum_double=True)
     ref = orc.compress(x.float().cpu().numpy().reshape(-1, D))
     got = idx.cpu().numpy().reshape(-1, G)

@@ -379,6 +379,91 @@ def test_batched_jobs_equal_single_calls(pkg):
         assert torch.equal(o, want)
 
 
+def _raw_decompress(native, c, idx, nrm, out, rows, tokens, row_stride, token_stride, prs, workspace):
+    rc = native.lib().tq_decompress(idx.data_ptr(), nrm.data_ptr(), prs, rows, tokens, c.table().data_ptr(), 128, c.bits,
+                                    out.data_ptr(), native.dtype_code(out.dtype), row_stride, token_stride,
+                                    workspace.data_ptr() if workspace is not None else None,
+                                    torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, native.lib().tq_status_string(rc)
+
+
+@pytest.mark.parametrize("bits,out_dtype", [(4, torch.bfloat16), (2, torch.float16), (8, torch.float16), (3, torch.float32)])
+def test_decompress_tickets_give_the_same_bytes(pkg, bits, out_dtype):
+    """Jobs large enough for the kernel to draw its tiles from the workspace counter: the output is byte for
+    byte what the fixed assignment of tiles writes, the counters are zero again after every launch, and a
+    second, smaller launch on the same workspace is right too."""
+    native = pkg._native
+    c = pkg.MSECompressor(128, bits, seed=7 + bits, device=DEV)
+    n = 300_000 + 17                                     # a ragged last tile
+    x = outlier_kv((1, 1, n, 128), seed=bits, dtype=torch.bfloat16).to(DEV)
+    packed = c.compress(x)
+    idx, nrm = packed["idx_bytes"], packed["vec_norms"]
+    ws = torch.zeros(int(native.lib().tq_workspace_bytes(1)), dtype=torch.uint8, device=DEV)
+    for tokens in (n, 270_001):
+        fixed = torch.full((tokens + 8, 128), 7.0, dtype=out_dtype, device=DEV)
+        drawn = torch.full((tokens + 8, 128), 7.0, dtype=out_dtype, device=DEV)
+        _raw_decompress(native, c, idx, nrm, fixed, 1, tokens, 0, 128, 0, None)
+        _raw_decompress(native, c, idx, nrm, drawn, 1, tokens, 0, 128, 0, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(fixed, drawn)
+        assert bool((drawn[tokens:] == 7.0).all())       # nothing written past the job
+        assert int(ws.sum()) == 0
+    # rows with their own stride in the output and in the packed store (the streaming cache's layout)
+    rows, tokens, cap = 6, 45_000, 50_000
+    fixed = torch.zeros(rows, cap, 128, dtype=out_dtype, device=DEV)
+    drawn = torch.zeros(rows, cap, 128, dtype=out_dtype, device=DEV)
+    G = idx.shape[-1]
+    store_idx = idx.reshape(-1, G)[: rows * cap].reshape(rows, cap, G)
+    store_nrm = nrm.reshape(-1)[: rows * cap].reshape(rows, cap)
+    _raw_decompress(native, c, store_idx, store_nrm, fixed, rows, tokens, cap * 128, 128, cap, None)
+    _raw_decompress(native, c, store_idx, store_nrm, drawn, rows, tokens, cap * 128, 128, cap, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(fixed, drawn) and int(ws.sum()) == 0
+    assert bool((drawn[:, tokens:] == 0).all())
+
+
+def test_decompress_tickets_batched_and_on_two_streams(pkg):
+    """One launch over jobs of very different sizes (each job has its own counter), and two launches that
+    overlap on two streams, each with the workspace the host side keeps for its stream."""
+    native = pkg._native
+    sizes = [280_000, 100, 70_003, 31, 150_000]
+    comps = [pkg.MSECompressor(128, 4, seed=42 + 1000 * l, device=DEV) for l in range(len(sizes))]
+    xs = [outlier_kv((1, 1, n, 128), seed=50 + l, dtype=torch.float16).to(DEV) for l, n in enumerate(sizes)]
+    packed = [c.compress(x) for c, x in zip(comps, xs)]
+    outs = [torch.zeros_like(x) for x in xs]
+    jobs = [{"states": o, "idx_bytes": p["idx_bytes"], "vec_norms": p["vec_norms"], "table": c.table(), "bits": 4}
+            for o, p, c in zip(outs, packed, comps)]
+    jl = native.JobList(jobs, DEV)
+    for _ in range(2):
+        for o in outs:
+            o.zero_()
+        jl.decompress()
+        torch.cuda.synchronize()
+        assert int(jl.workspace.sum()) == 0
+        for c, p, o, n in zip(comps, packed, outs, sizes):
+            want = torch.empty_like(o)
+            _raw_decompress(native, c, p["idx_bytes"], p["vec_norms"], want, 1, n, 0, 128, 0, None)
+            torch.cuda.synchronize()
+            assert torch.equal(o, want)
+    # two streams at once through the host mirror
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    got = [torch.empty_like(xs[0]), torch.empty_like(xs[4])]
+    for _ in range(3):
+        with torch.cuda.stream(s1):
+            comps[0].decompress_into(packed[0], got[0])
+        with torch.cuda.stream(s2):
+            comps[4].decompress_into(packed[4], got[1])
+    torch.cuda.synchronize()
+    keys = [k for k in native._workspaces if k[1] in (s1.cuda_stream, s2.cuda_stream)]
+    assert len(keys) == 2 and all(int(native._workspaces[k].sum()) == 0 for k in keys)
+    for i, j in ((0, 0), (1, 4)):
+        want = torch.empty_like(got[i])
+        _raw_decompress(native, comps[j], packed[j]["idx_bytes"], packed[j]["vec_norms"], want, 1, sizes[j], 0, 128, 0, None)
+        torch.cuda.synchronize()
+        assert torch.equal(got[i], want)
+
+
 def test_round_trip_properties_at_scale(pkg):
     """Size-independent properties on a Llama-3-8B-shaped layer slice (bf16, 8 heads x 8192 tokens):
     re-compressing the de-quantised tensor reproduces (almost) the same codes; scaling the input by 2

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol(pkg):
     for name in declared:
         assert hasattr(lib, name), name
     assert sorted(pkg._native.EXPORTS) == declared
-    assert lib.tq_abi_version() == 2
+    assert lib.tq_abi_version() == 3
     assert lib.tq_status_string(0) == b"ok"
     assert b"bits" in lib.tq_status_string(-2)
 
@@ -283,10 +283,18 @@ def test_c_abi_argument_errors(pkg):
     assert call(None, 1, 4, 128, tokens=0) == 0          # empty input: nothing to do, not an error
     assert call(p, 1, 4, 128, rows=2, rs=1024, prs=3) == E["SIZE"]   # packed rows shorter than the token count
     assert call(p, 1, 4, 128, rows=2, rs=1024, prs=1 << 31) == E["SIZE"]
-    assert lib.tq_decompress(p, p, 0, 1, 4, p, 128, 9, p, 0, 0, 128, None) == E["BITS"]
-    assert lib.tq_decompress(p, p, 0, 1, 4, p, 128, 4, None, 0, 0, 128, None) == E["NULL"]
-    assert lib.tq_decompress(p, p, 0, 1, 0, p, 128, 4, None, 0, 0, 128, None) == 0
-    assert lib.tq_decompress(p, p, 2, 2, 4, p, 128, 4, p, 1, 1024, 128, None) == E["SIZE"]
+    assert lib.tq_decompress(p, p, 0, 1, 4, p, 128, 9, p, 0, 0, 128, None, None) == E["BITS"]
+    assert lib.tq_decompress(p, p, 0, 1, 4, p, 128, 4, None, 0, 0, 128, None, None) == E["NULL"]
+    assert lib.tq_decompress(p, p, 0, 1, 0, p, 128, 4, None, 0, 0, 128, None, None) == 0
+    assert lib.tq_decompress(p, p, 2, 2, 4, p, 128, 4, p, 1, 1024, 128, None, None) == E["SIZE"]
+    p64 = buf.ctypes.data + (-buf.ctypes.data) % 64
+    assert lib.tq_decompress(p, p, 0, 1, 4, p, 128, 4, p, 0, 0, 128, p64 + 16, None) == E["ALIGN"]   # workspace: 64-byte aligned
+    assert lib.tq_decompress(p, p, 0, 1, 0, p, 128, 4, None, 0, 0, 128, p64, None) == 0
+    assert lib.tq_workspace_bytes(0) == 256 and lib.tq_workspace_bytes(1) == 256 and lib.tq_workspace_bytes(24) == 24 * 256
+    assert lib.tq_workspace_bytes(-1) == E["SIZE"] and lib.tq_workspace_bytes(4097) == E["SIZE"]
+    assert lib.tq_decompress_batched(None, None, 0, 128, None, None) == 0
+    assert lib.tq_decompress_batched(None, None, 3, 128, None, None) == E["NULL"]
+    assert lib.tq_decompress_batched(p, p, 3, 128, p64 + 32, None) == E["ALIGN"]
     assert lib.tq_compress_batched(None, None, 0, 128, None) == 0
     assert lib.tq_compress_batched(None, None, 3, 128, None) == E["NULL"]
     # the decode-step ends: (queries, q_dtype, rows, group, scale, pi_k_t, k_win, v_win, win_dtype, n_win, win_stride, q_rot, part_w)

@@ -12,7 +12,7 @@ import ctypes
 import os
 import shutil
 import subprocess
-from typing import List, Optional, Sequence, Tuple
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -86,7 +86,7 @@ class TqJob(ctypes.Structure):
 EXPORTS = (
     "tq_abi_version", "tq_status_string", "tq_device_count", "tq_bytes_per_vector",
     "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_quantize_host",
-    "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched",
+    "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched", "tq_workspace_bytes",
     "tq_scores", "tq_weighted_values", "tq_weighted_values_splits", "tq_attend_partials", "tq_attend_splits",
     "tq_attend_prepare", "tq_attend_merge",
 )
@@ -116,7 +116,9 @@ def lib() -> ctypes.CDLL:
     L.tq_table_build.argtypes = [vp, vp, ci, ci, vp, ctypes.c_size_t]
     L.tq_table_quantize_host.argtypes = [vp, vp, ll, vp]
     L.tq_compress.argtypes = [vp, ci, ll, ll, ll, ll, vp, ci, ci, vp, vp, ll, vp]
-    L.tq_decompress.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, ll, ll, vp]
+    L.tq_decompress.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, ll, ll, vp, vp]
+    L.tq_workspace_bytes.restype = ll
+    L.tq_workspace_bytes.argtypes = [ci]
     L.tq_compress_batched.argtypes = [vp, vp, ci, ci, vp]
     L.tq_scores.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, vp, ll, vp]
     L.tq_weighted_values_splits.argtypes = [ll, ll]
@@ -125,9 +127,9 @@ def lib() -> ctypes.CDLL:
     L.tq_attend_merge.argtypes = [vp, ci, vp, vp, ll, ci, vp, ci, vp]
     L.tq_attend_partials.argtypes = [vp, vp, vp, vp, ll, ll, ll, vp, vp, ci, ci, ci, vp, ci, ci, vp, vp]
     L.tq_weighted_values.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ll, ci, vp, ci, vp, vp]
-    L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp]
+    L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp, vp]
     for name in EXPORTS:
-        if name not in ("tq_status_string", "tq_table_bytes"):
+        if name not in ("tq_status_string", "tq_table_bytes", "tq_workspace_bytes"):
             getattr(L, name).restype = ci
     _lib = L
     return L
@@ -282,6 +284,24 @@ def _on(device: torch.device):
     return torch.cuda.device(device)
 
 
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, stream: int) -> int:
+    """Address of the ticket counters tq_decompress draws its tiles from, or 0 (fixed assignment of tiles).
+    One zero-filled buffer per (device, stream): launches on one stream run one after the other and each
+    leaves the counters at zero, launches on different streams never share.  While a graph is being
+    captured the answer is 0: the graph may be replayed on any stream, next to eager launches on this one."""
+    if torch.cuda.is_current_stream_capturing():
+        return 0
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.zeros(int(lib().tq_workspace_bytes(1)), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws.data_ptr()
+
+
 def compress_into(states: torch.Tensor, table: torch.Tensor, bits: int,
                   idx_bytes: torch.Tensor, vec_norms: torch.Tensor) -> None:
     """Launch tq_compress on `states` ([B,H,S,128], any supported float type, last dim dense).
@@ -318,9 +338,10 @@ def decompress_into(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: tor
                       "two stride levels")
     rows, tokens, row_stride, token_stride = lay
     with _on(out.device):
+        stream = _stream_handle(out.device)
         rc = lib().tq_decompress(idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, rows, tokens, table.data_ptr(),
                                  out.shape[-1], bits, out.data_ptr(), dtype_code(out.dtype), row_stride,
-                                 token_stride, _stream_handle(out.device))
+                                 token_stride, _workspace(out.device, stream), stream)
     check(rc, "tq_decompress")
 
 
@@ -597,6 +618,9 @@ class JobList:
             self._keep.append((t, j["idx_bytes"], j["vec_norms"], j["table"]))
         raw = np.frombuffer(bytes(self.host), dtype=np.uint8).copy()
         self.dev = torch.from_numpy(raw).to(self.device)
+        # ticket counters of the decompress launch, one record per job; zero now, and every launch leaves them zero.
+        # Launches of one list write the same outputs, so they never overlap and can share the counters.
+        self.workspace = torch.zeros(int(lib().tq_workspace_bytes(self.n)), dtype=torch.uint8, device=self.device)
 
     def compress(self) -> None:
         with _on(self.device):
@@ -607,7 +631,7 @@ class JobList:
     def decompress(self) -> None:
         with _on(self.device):
             rc = lib().tq_decompress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, HEAD_DIM,
-                                             _stream_handle(self.device))
+                                             self.workspace.data_ptr(), _stream_handle(self.device))
         check(rc, "tq_decompress_batched")
 
 

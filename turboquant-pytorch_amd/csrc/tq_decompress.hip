@@ -11,6 +11,16 @@
 // v_mfma_f32_32x32x16_f16; the A operand is Pi^T in fp16, fp32 accumulate.  The 32x128 result
 // tile is transposed through a wave-private, XOR-swizzled LDS buffer so that every store
 // instruction writes 1 KiB of consecutive memory.
+//
+// Which tiles a block works on.  A block draws "tickets": one ticket = WAVES consecutive tiles,
+// one per wave.  With a workspace the tickets of a job come from a counter in device memory
+// (atomicAdd), so the blocks walk through the job in the order in which they become free and the
+// addresses being written at any moment stay within a few MiB of each other; on this part that
+// write pattern reaches 10-15 % more bandwidth than a fixed assignment (block b takes tickets
+// b, b + grid, ...), under which fast and slow blocks drift apart.  Without a workspace, and for
+// jobs too small to matter, the fixed assignment is used.  Thread 0 draws one ticket ahead and
+// hands it to the block through LDS; one barrier per ticket.  The last block of a job to finish
+// sets the job's counters back to zero, so a workspace that was zero before a launch is zero after it.
 #include <type_traits>
 
 #include "tq_device.h"
@@ -35,7 +45,7 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
 }
 
 template <int DTYPE, int IPB>
-__global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompress_kernel(TqDevJob job0, const tq_job *jobs) {
+__global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t *workspace) {
     using T = OutTraits<DTYPE>;
     constexpr int ELEM = T::ELEM;
     constexpr int VEC_BYTES = TQ_HEAD_DIM * ELEM;   // 256 or 512
@@ -55,7 +65,6 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     const uint32_t lane = tid & 63u;
     const uint32_t wave = tid >> 6;
     const uint32_t n_tiles = (job.n_vec + 31u) / 32u;
-    if (blockIdx.x * T::WAVES >= n_tiles) return;
 
     const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
     uint8_t *lds_a = lds;
@@ -64,10 +73,26 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
 
     tq_copy_to_lds(lds_a, job.table + hd->off_at_f16, TQ_OPERAND_BYTES, tid, T::WAVES * TQ_WAVE);
     tq_copy_to_lds(lds_lut, job.table + hd->off_lut, 256u * 2u * IPB, tid, T::WAVES * TQ_WAVE);
+
+    // tickets: counter[0] = next tile to hand out, counter[1] = blocks of this job that are done
+    __shared__ uint32_t tk[2];
+    uint32_t *counter = workspace ? workspace + blockIdx.y * (TQ_WORKSPACE_BYTES_PER_JOB / 4) : nullptr;
+    uint32_t fixed_next = blockIdx.x * T::WAVES;
+    auto draw = [&]() -> uint32_t {     // thread 0 only
+        if (counter) return atomicAdd(counter, (uint32_t)T::WAVES);
+        const uint32_t t = fixed_next < n_tiles ? fixed_next : n_tiles;   // saturates: no wrap-around on huge grids
+        fixed_next = t + gridDim.x * T::WAVES;
+        return t;
+    };
+    if (tid == 0) {
+        const uint32_t t0 = draw(), t1 = draw();
+        tk[0] = t0;
+        tk[1] = t1;
+    }
     __syncthreads();
 
-    const uint32_t tile_stride = gridDim.x * T::WAVES;
-    uint32_t tile = blockIdx.x * T::WAVES + wave;
+    uint32_t base = tk[0];             // first tile of the block's current ticket (the same in every wave)
+    uint32_t tile = base + wave;
     const uint32_t n = lane & 31u, hk = lane >> 5;
     const uint32_t st_vec = lane / PIECES, st_piece = lane % PIECES;
 
@@ -211,16 +236,24 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     // Tiles whose 32 vectors all exist: the loads of the next tile are always issued (past the end: the
     // current tile again, never used) and nothing is predicated, so loads -> stores -> wait for the loads
     // leaves the stores in flight (s_waitcnt vmcnt(#stores)) instead of draining them every iteration.
+    // The loop runs once per ticket of the block, the same number of times in every wave (the barrier).
     const uint32_t n_full = job.n_vec / 32u;
     auto run = [&](auto fast_tag) {
+        uint32_t cur[NW];
+        float nrm = 0.f;
         if (tile < n_full) {
-            uint32_t cur[NW];
             issue_loads(std::true_type{}, fast_tag, tile);
 #pragma unroll
             for (int i = 0; i < NW; ++i) cur[i] = raw[i];
-            float nrm = half_bits_to_float(norm_bits);
-            while (tile < n_full) {
-                const uint32_t next = tile + tile_stride;
+            nrm = half_bits_to_float(norm_bits);
+        }
+        uint32_t it = 0;
+        while (base < n_tiles) {
+            uint32_t fresh = 0;
+            if (tid == 0) fresh = draw();                 // the ticket after next; its latency hides behind the tile
+            const uint32_t nbase = tk[(it + 1u) & 1u];     // written before the previous barrier
+            const uint32_t next = nbase + wave;
+            if (tile < n_full) {
                 issue_loads(std::true_type{}, fast_tag, next < n_full ? next : tile);
                 asm volatile("" ::: "memory");          // the prefetch stays ahead of the tile's work
                 process(std::true_type{}, fast_tag, tile, cur, nrm);
@@ -234,19 +267,32 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
                 uint32_t nb = norm_bits;
                 asm volatile("" : "+v"(nb));
                 nrm = half_bits_to_float((uint16_t)nb);
-                tile = next;
-            }
-        }
-        // the partial last tile of the job, for the wave whose turn it is
-        if (tile == n_full && n_full < n_tiles) {
-            issue_loads(std::false_type{}, fast_tag, tile);
-            uint32_t cur[NW];
+            } else if (tile == n_full && n_full < n_tiles) {   // the partial last tile of the job
+                issue_loads(std::false_type{}, fast_tag, tile);
+                uint32_t part[NW];
 #pragma unroll
-            for (int i = 0; i < NW; ++i) cur[i] = raw[i];
-            process(std::false_type{}, fast_tag, tile, cur, half_bits_to_float(norm_bits));
+                for (int i = 0; i < NW; ++i) part[i] = raw[i];
+                process(std::false_type{}, fast_tag, tile, part, half_bits_to_float(norm_bits));
+            }
+            if (tid == 0) tk[it & 1u] = fresh;             // everyone read this slot before the previous barrier
+            __syncthreads();
+            base = nbase;
+            tile = next;
+            ++it;
         }
     };
     if (fast) run(std::true_type{}); else run(std::false_type{});
+
+    // Every ticket this block drew has been answered (the values went through LDS) before it reports itself
+    // done, so the block that finds all others done knows that nobody touches the counters again in this
+    // launch.  All accesses to the counters are device-scope atomics, which are performed in one place;
+    // no fence is needed, and a release fence here would write back the L2's share of the output first.
+    if (counter && tid == 0) {
+        if (atomicAdd(counter + 1, 1u) == gridDim.x - 1u) {
+            atomicExch(counter, 0u);
+            atomicExch(counter + 1, 0u);
+        }
+    }
 }
 
 // ---- host side --------------------------------------------------------------------------
@@ -268,7 +314,8 @@ int device_cus(int &cus) {
 }
 
 template <int DTYPE, int IPB>
-int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t stream) {
+int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *workspace,
+                      hipStream_t stream) {
     using T = OutTraits<DTYPE>;
     int cus = 0;
     int rc = device_cus(cus);
@@ -286,26 +333,28 @@ int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, u
     const uint32_t want = (max_tiles + T::WAVES - 1) / T::WAVES;
     const uint32_t bx = tq_blocks_per_job(want, cus, n_jobs);
     dim3 grid(bx, (unsigned)n_jobs, 1), block(T::WAVES * TQ_WAVE, 1, 1);
-    hipLaunchKernelGGL((tq_decompress_kernel<DTYPE, IPB>), grid, block, lds, stream, job, jobs_dev);
+    // tickets pay off once every block has several to draw; below that the fixed assignment starts sooner
+    uint32_t *counters = want >= 4u * bx ? static_cast<uint32_t *>(workspace) : nullptr;
+    hipLaunchKernelGGL((tq_decompress_kernel<DTYPE, IPB>), grid, block, lds, stream, job, jobs_dev, counters);
     return (int)hipGetLastError();
 }
 
 template <int DTYPE>
-int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t s) {
+int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, hipStream_t s) {
     switch (8 / bits) {
-        case 8: return launch_decompress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, s);
-        case 4: return launch_decompress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, s);
-        case 2: return launch_decompress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, s);
-        case 1: return launch_decompress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, s);
+        case 8: return launch_decompress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case 4: return launch_decompress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case 2: return launch_decompress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case 1: return launch_decompress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, ws, s);
         default: return TQ_ERR_BITS;
     }
 }
 
-int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t s) {
+int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, hipStream_t s) {
     switch (dtype) {
-        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, s);
-        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, s);
-        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, s);
+        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
         default: return TQ_ERR_DTYPE;
     }
 }
@@ -338,11 +387,13 @@ int check_job(const void *out, int dtype, long long rows, long long tokens, long
 extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long packed_row_stride,
                              long long rows, long long tokens,
                              const void *table_dev, int head_dim, int bits, void *out, int out_dtype,
-                             long long row_stride, long long token_stride, void *stream) {
+                             long long row_stride, long long token_stride, void *workspace, void *stream) {
     long long n_vec = 0;
     const int rc = check_job(out, out_dtype, rows, tokens, row_stride, token_stride, table_dev, head_dim, bits,
                              idx_bytes, vec_norms, packed_row_stride, &n_vec);
-    if (rc || n_vec == 0) return rc;
+    if (rc) return rc;
+    if ((uintptr_t)workspace & 63u) return TQ_ERR_ALIGN;
+    if (n_vec == 0) return TQ_OK;
     TqDevJob job;
     job.states = static_cast<const uint8_t *>(out);
     job.idx_bytes = const_cast<uint8_t *>(idx_bytes);
@@ -353,14 +404,20 @@ extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms
     job.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     job.row_stride = row_stride * elem_bytes(out_dtype);
     job.token_stride = token_stride * elem_bytes(out_dtype);
-    return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), static_cast<hipStream_t>(stream));
+    return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), workspace, static_cast<hipStream_t>(stream));
+}
+
+extern "C" long long tq_workspace_bytes(int n_jobs) {
+    if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
+    return (long long)TQ_WORKSPACE_BYTES_PER_JOB * (n_jobs > 0 ? n_jobs : 1);
 }
 
 extern "C" int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
-                                     int head_dim, void *stream) {
+                                     int head_dim, void *workspace, void *stream) {
     if (n_jobs == 0) return TQ_OK;
     if (!jobs_host || !jobs_dev) return TQ_ERR_NULL;
     if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
+    if ((uintptr_t)workspace & 63u) return TQ_ERR_ALIGN;
     long long max_vec = 0;
     for (int i = 0; i < n_jobs; ++i) {
         const tq_job &j = jobs_host[i];
@@ -376,5 +433,5 @@ extern "C" int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs
     if (max_vec == 0) return TQ_OK;
     TqDevJob none{};
     return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec + 31) / 32),
-                    static_cast<hipStream_t>(stream));
+                    workspace, static_cast<hipStream_t>(stream));
 }
