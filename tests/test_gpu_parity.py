@@ -426,7 +426,7 @@ def test_decompress_tickets_batched_and_on_two_streams(pkg):
     """One launch over jobs of very different sizes (each job has its own counter), and two launches that
     overlap on two streams, each with the workspace the host side keeps for its stream."""
     native = pkg._native
-    sizes = [280_000, 100, 70_003, 31, 150_000]
+    sizes = [280_000, 100, 70_003, 0, 31, 150_000]
     comps = [pkg.MSECompressor(128, 4, seed=42 + 1000 * l, device=DEV) for l in range(len(sizes))]
     xs = [outlier_kv((1, 1, n, 128), seed=50 + l, dtype=torch.float16).to(DEV) for l, n in enumerate(sizes)]
     packed = [c.compress(x) for c, x in zip(comps, xs)]
@@ -448,16 +448,16 @@ def test_decompress_tickets_batched_and_on_two_streams(pkg):
     # two streams at once through the host mirror
     s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
     torch.cuda.synchronize()
-    got = [torch.empty_like(xs[0]), torch.empty_like(xs[4])]
+    got = [torch.empty_like(xs[0]), torch.empty_like(xs[5])]
     for _ in range(3):
         with torch.cuda.stream(s1):
             comps[0].decompress_into(packed[0], got[0])
         with torch.cuda.stream(s2):
-            comps[4].decompress_into(packed[4], got[1])
+            comps[5].decompress_into(packed[5], got[1])
     torch.cuda.synchronize()
     keys = [k for k in native._workspaces if k[1] in (s1.cuda_stream, s2.cuda_stream)]
     assert len(keys) == 2 and all(int(native._workspaces[k].sum()) == 0 for k in keys)
-    for i, j in ((0, 0), (1, 4)):
+    for i, j in ((0, 0), (1, 5)):
         want = torch.empty_like(got[i])
         _raw_decompress(native, comps[j], packed[j]["idx_bytes"], packed[j]["vec_norms"], want, 1, sizes[j], 0, 128, 0, None)
         torch.cuda.synchronize()

@@ -65,6 +65,7 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     const uint32_t lane = tid & 63u;
     const uint32_t wave = tid >> 6;
     const uint32_t n_tiles = (job.n_vec + 31u) / 32u;
+    if (n_tiles == 0u) return;   // an empty job of a batch: its table may be NULL, and its counters stay untouched (zero)
 
     const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
     uint8_t *lds_a = lds;
