@@ -231,6 +231,38 @@ int tq_attend_partials(const uint8_t *k_idx, const uint16_t *k_norms, const uint
                        const void *table_k, const void *table_v, int head_dim, int bits_k, int bits_v,
                        const float *q_rot, int group, int splits, float *partial, void *stream);
 
+/*
+ * One decode step of a streaming cache layer as two calls (each chains the entry points above; for hosts
+ * that pay per call).  Replaces the bookkeeping of V3Cache.update for one new token per sequence,
+ * generation_test_v2.py:96-126, on a cache kept as one packed store [rows, capacity] plus a window buffer
+ * [rows, win_cap, 128] per tensor.
+ *
+ * tq_append_token: if evict >= 0, window token `evict` of every row is compressed into packed slot
+ * `packed_slot` of the row (tq_compress with rows x 1 token; k_idx .. v_norms are the bases of the stores,
+ * packed_row_stride their capacity); then the new key / value vector of every row (row r at element
+ * r * k_new_stride / r * v_new_stride) is written to window token `put`.  dtype is the element type of the
+ * new vectors and of the window; win_stride = elements between rows of the window buffers.  Pointers are
+ * 16-byte aligned, strides multiples of 16 bytes.
+ *
+ * tq_attend_step: tq_attend_prepare, tq_attend_partials (if tokens > 0, with `splits` splits) and
+ * tq_attend_merge in a row; q_rot [rows, group, 128], part_w [rows, group, 130] and
+ * partial [rows, splits, group, 130] are float32 scratch of the caller.  k_win / v_win point at the first
+ * of the n_win window tokens.  tokens = 0 and n_win = 0 together: TQ_ERR_SIZE.
+ */
+int tq_append_token(const void *k_new, const void *v_new, int dtype, long long k_new_stride, long long v_new_stride,
+                    void *k_win, void *v_win, long long win_stride, long long evict, long long put,
+                    const void *table_k, const void *table_v, int head_dim, int bits_k, int bits_v,
+                    uint8_t *k_idx, uint16_t *k_norms, uint8_t *v_idx, uint16_t *v_norms,
+                    long long packed_row_stride, long long packed_slot, long long rows, void *stream);
+int tq_attend_step(const void *queries, int q_dtype, long long rows, int group, float scale,
+                   const float *pi_k_t, const float *pi_v,
+                   const void *k_win, const void *v_win, int win_dtype, long long n_win, long long win_stride,
+                   const uint8_t *k_idx, const uint16_t *k_norms, const uint8_t *v_idx, const uint16_t *v_norms,
+                   long long packed_row_stride, long long tokens,
+                   const void *table_k, const void *table_v, int head_dim, int bits_k, int bits_v,
+                   float *q_rot, float *part_w, float *partial, int splits,
+                   void *out, int out_dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

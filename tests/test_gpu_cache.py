@@ -553,3 +553,144 @@ def test_attend_with_sixteen_query_heads_per_kv_head(pkg, oracle):
     e2 = float((out.float() - ref).norm() / ref.norm())
     print(f"[attend] 16 heads per kv head: vs three-step {e1:.2e}, vs attention over update() tensors {e2:.2e}")
     assert e1 < 4e-3 and e2 < 1.5e-2
+
+
+@pytest.mark.parametrize("dtype,layout", [(torch.bfloat16, "bhsd"), (torch.float16, "bshd"), (torch.float32, "bhsd")])
+def test_single_call_decode_step_equals_the_general_path(pkg, dtype, layout):
+    """Steady-state decode steps go through tq_append_token / tq_attend_step (one library call each).  Two
+    caches fed the same tokens, one of them forced onto the general path, must hold the same bytes after every
+    step and give the same attention output; the run crosses several compactions of the window buffer and a
+    growth of the packed store."""
+    kvc = pkg.kv_cache
+    B, H, G, D, rw = 2, 3, 4, 128, 16
+    fast = pkg.V3Cache(4, 2, residual_window=rw, n_layers=4)
+    slow = pkg.V3Cache(4, 2, residual_window=rw, n_layers=4)
+    g = torch.Generator().manual_seed(5)
+
+    def tokens(n):
+        if layout == "bshd":                      # what a model's projections give: [B,S,H,D] storage
+            return (torch.randn(B, n, H, D, generator=g) * 1.5).to(dtype).to(DEV).transpose(1, 2)
+        return (torch.randn(B, H, n, D, generator=g) * 1.5).to(dtype).to(DEV)
+
+    calls = {"append": 0, "attend": 0}
+    real_append, real_attend = kvc._LayerStore.append_one, kvc.V3Cache._attend_step
+
+    def counted_append(self, k, v):
+        done = real_append(self, k, v)
+        calls["append"] += bool(done)
+        return done
+
+    def counted_attend(st, q, G_, scale):
+        out = real_attend(st, q, G_, scale)
+        calls["attend"] += out is not None
+        return out
+
+    k0, v0 = tokens(40), tokens(40)
+    for c in (fast, slow):
+        c.append(k0, v0, 1)
+    steps = 300
+    for i in range(steps):
+        k, v = tokens(1), tokens(1)
+        q = (torch.randn(B, H * G, 1, D, generator=g)).to(dtype).to(DEV)
+        kvc._LayerStore.append_one, kvc.V3Cache._attend_step = counted_append, staticmethod(counted_attend)
+        try:
+            fast.append(k, v, 1)
+            a = fast.attend(q, 1)
+        finally:
+            kvc._LayerStore.append_one, kvc.V3Cache._attend_step = real_append, staticmethod(real_attend)
+        kvc._LayerStore.append_one = lambda self, k_, v_: False
+        kvc.V3Cache._attend_step = staticmethod(lambda st, q_, G_, s_: None)
+        try:
+            slow.append(k, v, 1)
+            b = slow.attend(q, 1)
+        finally:
+            kvc._LayerStore.append_one, kvc.V3Cache._attend_step = real_append, staticmethod(real_attend)
+        assert torch.equal(a, b), i
+    sf, ss = fast._stores[1], slow._stores[1]
+    assert (sf.n_compressed, sf.n_recent, sf.total_seq) == (ss.n_compressed, ss.n_recent, ss.total_seq) == (40 + steps - rw, rw, 40 + steps)
+    n = sf.n_compressed
+    for name in ("k_idx", "k_nrm", "v_idx", "v_nrm"):
+        assert torch.equal(getattr(sf, name)[:, :, :n], getattr(ss, name)[:, :, :n]), name
+    for x, y in zip(sf.window(), ss.window()):
+        assert torch.equal(x, y)
+    # the single-call path really ran: every step attends through it, and every append except those that
+    # first have to move the window back to the front of its buffer or to grow the packed store
+    assert calls["attend"] == steps and calls["append"] >= steps - steps // rw - 6, calls
+
+
+def test_append_token_and_attend_step_through_the_c_abi(pkg, oracle):
+    """The two per-step entry points called by hand: the evicted window token lands in the packed slot with the
+    bytes tq_compress gives, the new token in the window slot, and tq_attend_step returns what the three
+    separate calls return."""
+    nat = pkg._native
+    L = nat.lib()
+    rows, D, G, win_cap, cap = 6, 128, 4, 32, 64
+    kc, vc = pkg.MSECompressor(D, 4, seed=1, device=DEV), pkg.MSECompressor(D, 2, seed=2, device=DEV)
+    g = torch.Generator().manual_seed(9)
+    k_win = torch.randn(rows, win_cap, D, generator=g).to(torch.bfloat16).to(DEV)
+    v_win = torch.randn(rows, win_cap, D, generator=g).to(torch.bfloat16).to(DEV)
+    k_new = torch.randn(rows, 2, D, generator=g).to(torch.bfloat16).to(DEV)[:, 1]      # rows 2*D elements apart
+    v_new = torch.randn(rows, D, generator=g).to(torch.bfloat16).to(DEV)
+    k_idx = torch.full((rows, cap, 64), 0xEE, dtype=torch.uint8, device=DEV)
+    v_idx = torch.full((rows, cap, 32), 0xEE, dtype=torch.uint8, device=DEV)
+    k_nrm = torch.full((rows, cap), -3.0, dtype=torch.float16, device=DEV)
+    v_nrm = torch.full((rows, cap), -3.0, dtype=torch.float16, device=DEV)
+    want_k, want_v = k_win.clone(), v_win.clone()
+    stream = torch.cuda.current_stream().cuda_stream
+    evict, put, slot = 5, 21, 7
+    rc = L.tq_append_token(k_new.data_ptr(), v_new.data_ptr(), 2, 2 * D, D, k_win.data_ptr(), v_win.data_ptr(), win_cap * D,
+                           evict, put, kc.table().data_ptr(), vc.table().data_ptr(), D, 4, 2,
+                           k_idx.data_ptr(), k_nrm.data_ptr(), v_idx.data_ptr(), v_nrm.data_ptr(), cap, slot, rows, stream)
+    assert rc == 0, L.tq_status_string(rc)
+    torch.cuda.synchronize()
+    want_k[:, put], want_v[:, put] = k_new, v_new
+    assert torch.equal(k_win, want_k) and torch.equal(v_win, want_v)
+    ck = kc.compress(want_k[:, evict].reshape(1, rows, 1, D))
+    cv = vc.compress(want_v[:, evict].reshape(1, rows, 1, D))
+    assert torch.equal(k_idx[:, slot], ck["idx_bytes"].reshape(rows, 64)) and torch.equal(k_nrm[:, slot], ck["vec_norms"].reshape(rows))
+    assert torch.equal(v_idx[:, slot], cv["idx_bytes"].reshape(rows, 32)) and torch.equal(v_nrm[:, slot], cv["vec_norms"].reshape(rows))
+    untouched = torch.ones(cap, dtype=torch.bool)
+    untouched[slot] = False
+    assert bool((k_idx[:, untouched] == 0xEE).all()) and bool((v_nrm[:, untouched] == -3).all())
+    # evict = -1: only the window is written
+    rc = L.tq_append_token(k_new.data_ptr(), v_new.data_ptr(), 2, 2 * D, D, k_win.data_ptr(), v_win.data_ptr(), win_cap * D,
+                           -1, 0, None, None, D, 4, 2, None, None, None, None, cap, 0, rows, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(k_win[:, 0], k_new) and bool((k_idx[:, untouched] == 0xEE).all())
+    # attend over 40 packed tokens + 9 window tokens: one call against three
+    x = outlier_kv((1, rows, 40, D), seed=3, dtype=torch.bfloat16).to(DEV)
+    pk, pv = kc.compress(x), vc.compress(x * 0.7)
+    q = torch.randn(rows, G, D, generator=g).to(torch.bfloat16).to(DEV)
+    n_w, splits, scale = 9, 2, D ** -0.5
+    outs = []
+    for single in (True, False):
+        q_rot = torch.empty(rows, G, D, device=DEV)
+        part_w = torch.empty(rows, G, D + 2, device=DEV)
+        part = torch.empty(rows, splits, G, D + 2, device=DEV)
+        out = torch.empty(rows, G, D, dtype=torch.bfloat16, device=DEV)
+        kw, vw = k_win[:, 3:], v_win[:, 3:]
+        packed = (pk["idx_bytes"].data_ptr(), pk["vec_norms"].data_ptr(), pv["idx_bytes"].data_ptr(), pv["vec_norms"].data_ptr())
+        if single:
+            rc = L.tq_attend_step(q.data_ptr(), 2, rows, G, scale, kc.pi_transposed().data_ptr(), vc.Pi.data_ptr(),
+                                  kw.data_ptr(), vw.data_ptr(), 2, n_w, win_cap * D, *packed, 0, 40,
+                                  kc.table().data_ptr(), vc.table().data_ptr(), D, 4, 2,
+                                  q_rot.data_ptr(), part_w.data_ptr(), part.data_ptr(), splits, out.data_ptr(), 2, stream)
+            assert rc == 0, L.tq_status_string(rc)
+        else:
+            assert L.tq_attend_prepare(q.data_ptr(), 2, rows, G, scale, kc.pi_transposed().data_ptr(), kw.data_ptr(), vw.data_ptr(),
+                                       2, n_w, win_cap * D, q_rot.data_ptr(), part_w.data_ptr(), stream) == 0
+            assert L.tq_attend_partials(*packed, 0, rows, 40, kc.table().data_ptr(), vc.table().data_ptr(), D, 4, 2,
+                                        q_rot.data_ptr(), G, splits, part.data_ptr(), stream) == 0
+            assert L.tq_attend_merge(part.data_ptr(), splits, part_w.data_ptr(), vc.Pi.data_ptr(), rows, G, out.data_ptr(), 2, stream) == 0
+        torch.cuda.synchronize()
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    # and against float64 attention over the de-quantised history and the window
+    kd = kc.decompress(pk).double().reshape(rows, 40, D)
+    vd = vc.decompress(pv).double().reshape(rows, 40, D)
+    K = torch.cat([kd, k_win[:, 3:3 + n_w].double()], 1)
+    V = torch.cat([vd, v_win[:, 3:3 + n_w].double()], 1)
+    ref = torch.softmax(torch.einsum("rgd,rtd->rgt", q.double(), K) * scale, -1) @ V
+    err = float((outs[0].double() - ref).norm() / ref.norm())
+    assert err < 6e-3, err

@@ -307,6 +307,18 @@ def test_c_abi_argument_errors(pkg):
     assert prep(kw=None) == E["NULL"] and prep(pw=None) == E["NULL"]
     assert prep(ws=512) == E["SIZE"]                       # rows of the window overlap
     assert prep(kw=p + 2) == E["ALIGN"] and prep(ws=1028) == E["ALIGN"]
+    # the per-step calls: (k_new, v_new, dtype, strides, windows, win_stride, evict, put, tables, head_dim, bits, stores, prs, slot, rows)
+    app = lambda kn=p, vn=p, dt=2, ks=128, vs=128, kw=p, vw=p, ws=4096, ev=0, put=16, tk=p, tv=p, hd=128, bk=4, bv=2, ki=p, kr=p, vi=p, vr=p, prs=64, slot=3, rows=2: \
+        lib.tq_append_token(kn, vn, dt, ks, vs, kw, vw, ws, ev, put, tk, tv, hd, bk, bv, ki, kr, vi, vr, prs, slot, rows, None)
+    assert app(dt=7) == E["DTYPE"] and app(hd=64) == E["HEAD_DIM"] and app(put=-1) == E["SIZE"] and app(ev=16) == E["SIZE"]
+    assert app(put=32) == E["SIZE"] and app(slot=64) == E["SIZE"] and app(ks=64) == E["SIZE"] and app(rows=0) == 0
+    assert app(kn=None) == E["NULL"] and app(ki=None) == E["NULL"] and app(bk=9) == E["BITS"]
+    assert app(kw=p + 4) == E["ALIGN"] and app(ws=4100) == E["ALIGN"] and app(vs=132) == E["ALIGN"]
+    att = lambda q=p, tokens=8, nw=4, splits=1, part=p, out=p, od=2, piv=p: lib.tq_attend_step(
+        q, 2, 1, 4, 0.5, p, piv, p, p, 2, nw, 1024, p, p, p, p, 0, tokens, p, p, 128, 4, 2, p, p, part, splits, out, od, None)
+    assert att(tokens=0, nw=0) == E["SIZE"] and att(tokens=-1) == E["SIZE"] and att(od=5) == E["DTYPE"]
+    assert att(out=None) == E["NULL"] and att(piv=None) == E["NULL"] and att(splits=0) == E["SIZE"] and att(part=None) == E["NULL"]
+    assert att(q=None) == E["NULL"]
     merge = lambda part=p, s=1, pw=p, piv=p, rows=1, g=4, out=p, od=2: lib.tq_attend_merge(part, s, pw, piv, rows, g, out, od, None)
     assert merge(g=17) == E["SIZE"] and merge(s=-1) == E["SIZE"] and merge(od=4) == E["DTYPE"] and merge(rows=0) == 0
     assert merge(piv=None) == E["NULL"] and merge(out=None) == E["NULL"] and merge(part=None) == E["NULL"]

@@ -88,7 +88,7 @@ EXPORTS = (
     "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_quantize_host",
     "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched", "tq_workspace_bytes",
     "tq_scores", "tq_weighted_values", "tq_weighted_values_splits", "tq_attend_partials", "tq_attend_splits",
-    "tq_attend_prepare", "tq_attend_merge",
+    "tq_attend_prepare", "tq_attend_merge", "tq_append_token", "tq_attend_step",
 )
 
 _lib = None
@@ -128,6 +128,9 @@ def lib() -> ctypes.CDLL:
     L.tq_attend_partials.argtypes = [vp, vp, vp, vp, ll, ll, ll, vp, vp, ci, ci, ci, vp, ci, ci, vp, vp]
     L.tq_weighted_values.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ll, ci, vp, ci, vp, vp]
     L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp, vp]
+    L.tq_append_token.argtypes = [vp, vp, ci, ll, ll, vp, vp, ll, ll, ll, vp, vp, ci, ci, ci, vp, vp, vp, vp, ll, ll, ll, vp]
+    L.tq_attend_step.argtypes = [vp, ci, ll, ci, ctypes.c_float, vp, vp, vp, vp, ci, ll, ll, vp, vp, vp, vp, ll, ll,
+                                 vp, vp, ci, ci, ci, vp, vp, vp, ci, vp, ci, vp]
     for name in EXPORTS:
         if name not in ("tq_status_string", "tq_table_bytes", "tq_workspace_bytes"):
             getattr(L, name).restype = ci
@@ -182,6 +185,9 @@ def quantize_host(table: np.ndarray, r: np.ndarray) -> np.ndarray:
 def _require_gpu(t: torch.Tensor, what: str) -> None:
     if not t.is_cuda:
         raise TqError(f"{what} must live on a HIP device (got {t.device}); this package has no CPU path")
+
+
+ERR_ALIGN = -8      # TQ_ERR_ALIGN of include/tqamd.h
 
 
 def dtype_code(dt: torch.dtype) -> int:
@@ -300,6 +306,19 @@ def _workspace(device: torch.device, stream: int) -> int:
         ws = torch.zeros(int(lib().tq_workspace_bytes(1)), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws.data_ptr()
+
+
+_step_scratch: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def step_scratch(device: torch.device, stream: int, floats: int) -> torch.Tensor:
+    """float32 scratch of a decode step (rotated queries, window record, split records), one buffer per
+    (device, stream), grown on demand: the steps of all layers on a stream run one after the other."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    buf = _step_scratch.get(key)
+    if buf is None or buf.numel() < floats:
+        buf = _step_scratch[key] = torch.empty(max(floats, 1 << 16), dtype=torch.float32, device=device)
+    return buf
 
 
 def compress_into(states: torch.Tensor, table: torch.Tensor, bits: int,

@@ -1185,7 +1185,10 @@ extern "C" int tq_attend_splits(long long rows, long long tokens) {
     if (rows <= 0 || tokens <= 0) return 1;
     int cus = 0;
     if (device_cus(cus)) cus = 256;
-    long long splits = ((long long)cus * 2 + rows - 1) / rows;       // one resident eight-wave block per compute unit, twice over
+    // One eight-wave block is resident per compute unit.  Few rows: as many splits as fill the chip once (a
+    // second generation of blocks would stage its tables again: 17 instead of 23 us for 8 rows x 32K tokens).
+    // Many rows: two generations, which balances blocks of unequal speed better than one.
+    long long splits = rows * 2 <= cus ? cus / rows : ((long long)cus * 2 + rows - 1) / rows;
     const long long most = (tokens + AT_RUN * AT_WAVES - 1) / (AT_RUN * AT_WAVES);
     if (splits > most) splits = most;
     if (splits > 4096) splits = 4096;
@@ -1267,4 +1270,92 @@ extern "C" int tq_attend_merge(const float *partial, int splits, const float *pa
     a.group = (uint32_t)group; a.splits = (uint32_t)splits; a.out_dtype = out_dtype;
     hipLaunchKernelGGL(tq_attend_merge_kernel, dim3((unsigned)(rows * group)), dim3(512), 0, static_cast<hipStream_t>(stream), a);
     return (int)hipGetLastError();
+}
+
+// ---- one decode step of a streaming cache layer, as two calls -----------------------------------------
+// Each call chains entry points declared above; a host that pays per call (an interpreter binding) makes two
+// calls per layer and step instead of nine.
+
+namespace {
+// window slot `put` of every row <- the row's new key and value vector (16-byte pieces)
+__global__ __launch_bounds__(256) void tq_window_put_kernel(const uint8_t *__restrict__ k_new, const uint8_t *__restrict__ v_new,
+                                                            long long k_new_stride, long long v_new_stride,
+                                                            uint8_t *__restrict__ k_win, uint8_t *__restrict__ v_win,
+                                                            long long win_stride, uint32_t pieces, uint32_t rows) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;      // (row, tensor, piece)
+    if (i >= rows * 2u * pieces) return;
+    const uint32_t piece = i % pieces, tensor = (i / pieces) & 1u, row = i / (2u * pieces);
+    const uint8_t *src = tensor ? v_new + (long long)row * v_new_stride : k_new + (long long)row * k_new_stride;
+    uint8_t *dst = (tensor ? v_win : k_win) + (long long)row * win_stride;
+    tq_gstore16(dst + piece * 16u, tq_gload16(src + piece * 16u));
+}
+
+inline int elem_size(int dtype) { return dtype == TQ_F32 ? 4 : (dtype == TQ_F16 || dtype == TQ_BF16) ? 2 : 0; }
+}  // namespace
+
+extern "C" int tq_append_token(const void *k_new, const void *v_new, int dtype, long long k_new_stride, long long v_new_stride,
+                               void *k_win, void *v_win, long long win_stride, long long evict, long long put,
+                               const void *table_k, const void *table_v, int head_dim, int bits_k, int bits_v,
+                               uint8_t *k_idx, uint16_t *k_norms, uint8_t *v_idx, uint16_t *v_norms,
+                               long long packed_row_stride, long long packed_slot, long long rows, void *stream) {
+    const int eb = elem_size(dtype);
+    if (!eb) return TQ_ERR_DTYPE;
+    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
+    if (rows < 0 || rows > (1 << 24) || put < 0 || evict < -1 || packed_slot < 0) return TQ_ERR_SIZE;
+    if (win_stride < (put + 1) * TQ_HEAD_DIM || win_stride < (evict + 1) * TQ_HEAD_DIM || evict == put) return TQ_ERR_SIZE;
+    if (rows > 1 && (k_new_stride < TQ_HEAD_DIM || v_new_stride < TQ_HEAD_DIM)) return TQ_ERR_SIZE;
+    if (rows == 0) return TQ_OK;
+    if (!k_new || !v_new || !k_win || !v_win) return TQ_ERR_NULL;
+    if (((uintptr_t)k_new & 15u) || ((uintptr_t)v_new & 15u) || ((uintptr_t)k_win & 15u) || ((uintptr_t)v_win & 15u) ||
+        ((win_stride * eb) & 15) || (rows > 1 && (((k_new_stride * eb) & 15) || ((v_new_stride * eb) & 15))))
+        return TQ_ERR_ALIGN;
+    if (evict >= 0) {
+        // the oldest window token of every row leaves the window: one vector per row, rows win_stride apart
+        if (packed_slot >= (packed_row_stride ? packed_row_stride : 1)) return TQ_ERR_SIZE;
+        const int gk = tq_bytes_per_vector(head_dim, bits_k), gv = tq_bytes_per_vector(head_dim, bits_v);
+        if (gk < 0) return gk;
+        if (gv < 0) return gv;
+        if (!k_idx || !k_norms || !v_idx || !v_norms) return TQ_ERR_NULL;
+        const uint8_t *kw = static_cast<const uint8_t *>(k_win) + evict * TQ_HEAD_DIM * eb;
+        const uint8_t *vw = static_cast<const uint8_t *>(v_win) + evict * TQ_HEAD_DIM * eb;
+        int rc = tq_compress(kw, dtype, rows, 1, win_stride, TQ_HEAD_DIM, table_k, head_dim, bits_k,
+                             k_idx + packed_slot * gk, k_norms + packed_slot, packed_row_stride, stream);
+        if (rc) return rc;
+        rc = tq_compress(vw, dtype, rows, 1, win_stride, TQ_HEAD_DIM, table_v, head_dim, bits_v,
+                         v_idx + packed_slot * gv, v_norms + packed_slot, packed_row_stride, stream);
+        if (rc) return rc;
+    }
+    const uint32_t pieces = (uint32_t)(TQ_HEAD_DIM * eb / 16);
+    const uint32_t n = (uint32_t)rows * 2u * pieces;
+    hipLaunchKernelGGL(tq_window_put_kernel, dim3((n + 255u) / 256u), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t *>(k_new), static_cast<const uint8_t *>(v_new),
+                       k_new_stride * eb, v_new_stride * eb,
+                       static_cast<uint8_t *>(k_win) + put * TQ_HEAD_DIM * eb, static_cast<uint8_t *>(v_win) + put * TQ_HEAD_DIM * eb,
+                       win_stride * eb, pieces, (uint32_t)rows);
+    return (int)hipGetLastError();
+}
+
+extern "C" int tq_attend_step(const void *queries, int q_dtype, long long rows, int group, float scale,
+                              const float *pi_k_t, const float *pi_v,
+                              const void *k_win, const void *v_win, int win_dtype, long long n_win, long long win_stride,
+                              const uint8_t *k_idx, const uint16_t *k_norms, const uint8_t *v_idx, const uint16_t *v_norms,
+                              long long packed_row_stride, long long tokens,
+                              const void *table_k, const void *table_v, int head_dim, int bits_k, int bits_v,
+                              float *q_rot, float *part_w, float *partial, int splits,
+                              void *out, int out_dtype, void *stream) {
+    if (tokens < 0 || n_win < 0 || (tokens == 0 && n_win == 0)) return TQ_ERR_SIZE;      // nothing to attend to
+    if (out_dtype != TQ_F32 && out_dtype != TQ_F16 && out_dtype != TQ_BF16) return TQ_ERR_DTYPE;
+    if (!out || !pi_v) return TQ_ERR_NULL;
+    if (tokens && splits < 1) return TQ_ERR_SIZE;
+    if (tokens && !partial) return TQ_ERR_NULL;
+    int rc = tq_attend_prepare(queries, q_dtype, rows, group, scale, pi_k_t, k_win, v_win, win_dtype, n_win, win_stride,
+                               q_rot, part_w, stream);
+    if (rc || rows == 0) return rc;
+    if (tokens) {
+        rc = tq_attend_partials(k_idx, k_norms, v_idx, v_norms, packed_row_stride, rows, tokens, table_k, table_v,
+                                head_dim, bits_k, bits_v, q_rot, group, splits, partial, stream);
+        if (rc) return rc;
+    }
+    return tq_attend_merge(tokens ? partial : nullptr, tokens ? splits : 0, n_win ? part_w : nullptr, pi_v, rows, group,
+                           out, out_dtype, stream);
 }

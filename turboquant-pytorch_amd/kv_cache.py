@@ -48,6 +48,7 @@ class _LayerStore:
         self.w0 = 0
         self.n_recent = 0
         self.total_seq = 0
+        self._consts = None
         self.reserve(capacity)
 
     @staticmethod
@@ -73,6 +74,49 @@ class _LayerStore:
             new.append(buf)
         self.k_idx, self.k_nrm, self.v_idx, self.v_nrm = new
         self.capacity = cap
+        self._consts = None
+
+    def consts(self) -> tuple:
+        """Addresses and sizes that the per-token calls pass on every step; rebuilt when the packed store moves."""
+        c = self._consts
+        if c is None:
+            kc, vc = self.comp.key_compressor, self.comp.val_compressor
+            c = self._consts = (self.k_win.data_ptr(), self.v_win.data_ptr(), self.win_cap * self.D,
+                                kc.table().data_ptr(), vc.table().data_ptr(), kc.bits, vc.bits,
+                                self.k_idx.data_ptr(), self.k_nrm.data_ptr(), self.v_idx.data_ptr(), self.v_nrm.data_ptr(),
+                                kc.pi_transposed().data_ptr(), vc.Pi.data_ptr(), _native.dtype_code(self.dtype),
+                                self.D * self.k_win.element_size())
+        return c
+
+    def append_one(self, keys: torch.Tensor, values: torch.Tensor) -> bool:
+        """The steady-state decode step in one library call: the window is full, its oldest token is compressed
+        into the next packed slot and the new token takes the next window slot.  False (nothing done) when the
+        step is not of that kind or the tensors are not laid out for it; the general path then runs."""
+        rw = self.window_tokens
+        if (rw == 0 or self.n_recent != rw or self.w0 + rw + 1 > self.win_cap or self.n_compressed + 1 > self.capacity
+                or keys.dtype != self.dtype or values.dtype != self.dtype or torch.compiler.is_compiling()):
+            return False
+        rows = self.B * self.H
+        strides = []
+        for t in (keys, values):
+            s0, s1, _, s3 = t.stride()
+            if s3 != 1 or (self.B > 1 and self.H > 1 and s0 != self.H * s1):
+                return False
+            strides.append(s1 if self.H > 1 else s0)
+        c = self.consts()
+        dev = self.device
+        with _native._on(dev):
+            rc = _native.lib().tq_append_token(keys.data_ptr(), values.data_ptr(), c[13], strides[0], strides[1],
+                                               c[0], c[1], c[2], self.w0, self.w0 + rw, c[3], c[4], self.D, c[5], c[6],
+                                               c[7], c[8], c[9], c[10], self.capacity, self.n_compressed, rows,
+                                               _native._stream_handle(dev))
+        if rc == _native.ERR_ALIGN:
+            return False
+        _native.check(rc, "tq_append_token")
+        self.n_compressed += 1
+        self.w0 += 1
+        self.total_seq += 1
+        return True
 
     def append_compressed(self, keys: torch.Tensor, values: torch.Tensor) -> None:
         """Compress [B,H,n,D] views of keys / values into packed slots [n_compressed, n_compressed + n)."""
@@ -154,6 +198,8 @@ class V3Cache:
         """Bookkeeping of generation_test_v2.py:96-126: the uncompressed tokens are (window ++ new); all but
         the last `residual_window` of them are compressed for good, the rest is the new window."""
         S_new = key_states.shape[2]
+        if S_new == 1 and st.append_one(key_states, value_states):
+            return
         st.total_seq += S_new
         rw = self.residual_window
         recent = st.n_recent + S_new
@@ -217,6 +263,10 @@ class V3Cache:
         kc, vc = st.comp.key_compressor, st.comp.val_compressor
         if fused is None:
             fused = G <= 16
+        if fused and n_w <= 512 and not torch.compiler.is_compiling():
+            out = self._attend_step(st, query_states, G, float(scale))
+            if out is not None:
+                return out
         kw, vw = st.window()
         if fused and n_w <= 512:
             # three launches: rotate the queries + window statistics, one pass over the packed history,
@@ -249,6 +299,35 @@ class V3Cache:
         if n_w:
             out = out + torch.matmul(probs[:, :, n_c:total].reshape(B, st.H, G, n_w), vw.to(torch.float32)).reshape(B, Hq, D)
         return out.to(query_states.dtype).reshape(B, Hq, 1, D)
+
+    @staticmethod
+    def _attend_step(st: _LayerStore, query_states: torch.Tensor, G: int, scale: float) -> Optional[torch.Tensor]:
+        """The fused path of `attend` in one library call (rotate + window, packed history, merge), with the
+        scratch kept per stream.  None when the queries are not laid out for it."""
+        B, Hq, _, D = query_states.shape
+        if not query_states.is_contiguous() or query_states.dtype not in _native._DTYPE_CODE or st.k_idx is None:
+            return None
+        n_c, n_w = st.n_compressed, st.n_recent
+        rows = B * st.H
+        L = _native.lib()
+        dev = st.device
+        c = st.consts()
+        splits = L.tq_attend_splits(rows, n_c) if n_c else 0
+        rec = D + 2
+        n_q, n_pw, n_p = rows * G * D, rows * G * rec, rows * splits * G * rec
+        with _native._on(dev):
+            stream = _native._stream_handle(dev)
+            scratch = _native.step_scratch(dev, stream, n_q + n_pw + n_p)
+            base = scratch.data_ptr()
+            out = torch.empty_like(query_states)
+            code = _native.dtype_code(query_states.dtype)
+            win_off = st.w0 * c[14]
+            rc = L.tq_attend_step(query_states.data_ptr(), code, rows, G, scale, c[11], c[12],
+                                  c[0] + win_off, c[1] + win_off, c[13], n_w, c[2],
+                                  c[7], c[8], c[9], c[10], st.capacity, n_c, c[3], c[4], D, c[5], c[6],
+                                  base, base + 4 * n_q, base + 4 * (n_q + n_pw), splits, out.data_ptr(), code, stream)
+        _native.check(rc, "tq_attend_step")
+        return out
 
     def get_seq_length(self, layer_idx: int = 0) -> int:
         st = self._stores.get(layer_idx)
