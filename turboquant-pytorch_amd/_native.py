@@ -311,12 +311,16 @@ def _workspace(device: torch.device, stream: int) -> int:
 _step_scratch: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
-def step_scratch(device: torch.device, stream: int, floats: int) -> torch.Tensor:
+def step_scratch(device: torch.device, stream: int, floats: int) -> Optional[torch.Tensor]:
     """float32 scratch of a decode step (rotated queries, window record, split records), one buffer per
-    (device, stream), grown on demand: the steps of all layers on a stream run one after the other."""
+    (device, stream), grown on demand: the steps of all layers on a stream run one after the other.
+    None when it would have to be allocated while a graph is being captured (the memory would belong to
+    the graph's pool, not to this table)."""
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     buf = _step_scratch.get(key)
     if buf is None or buf.numel() < floats:
+        if torch.cuda.is_current_stream_capturing():
+            return None
         buf = _step_scratch[key] = torch.empty(max(floats, 1 << 16), dtype=torch.float32, device=device)
     return buf
 
