@@ -20,12 +20,31 @@ subclass when transformers is importable.
 """
 from __future__ import annotations
 
-from typing import Dict, Optional, Tuple
+from typing import Dict, NamedTuple, Optional, Tuple
 
 import torch
 
 from . import _native
 from .compressors_v3 import TurboQuantV3
+
+
+class _StepConsts(NamedTuple):
+    """What the per-token library calls of one layer pass on every step: device addresses and sizes."""
+    k_win: int
+    v_win: int
+    win_stride: int        # elements between rows of the window buffers
+    table_k: int
+    table_v: int
+    bits_k: int
+    bits_v: int
+    k_idx: int
+    k_nrm: int
+    v_idx: int
+    v_nrm: int
+    pi_k_t: int
+    pi_v: int
+    dtype: int
+    vec_bytes: int         # bytes of one window token
 
 
 class _LayerStore:
@@ -82,16 +101,17 @@ class _LayerStore:
         self.capacity = cap
         self._consts = None
 
-    def consts(self) -> tuple:
-        """Addresses and sizes that the per-token calls pass on every step; rebuilt when the packed store moves."""
+    def consts(self) -> _StepConsts:
+        """Rebuilt when the packed store moves (`reserve`)."""
         c = self._consts
         if c is None:
             kc, vc = self.comp.key_compressor, self.comp.val_compressor
-            c = self._consts = (self.k_win.data_ptr(), self.v_win.data_ptr(), self.win_cap * self.D,
-                                kc.table().data_ptr(), vc.table().data_ptr(), kc.bits, vc.bits,
-                                self.k_idx.data_ptr(), self.k_nrm.data_ptr(), self.v_idx.data_ptr(), self.v_nrm.data_ptr(),
-                                kc.pi_transposed().data_ptr(), vc.Pi.data_ptr(), _native.dtype_code(self.dtype),
-                                self.D * self.k_win.element_size())
+            c = self._consts = _StepConsts(
+                self.k_win.data_ptr(), self.v_win.data_ptr(), self.win_cap * self.D,
+                kc.table().data_ptr(), vc.table().data_ptr(), kc.bits, vc.bits,
+                self.k_idx.data_ptr(), self.k_nrm.data_ptr(), self.v_idx.data_ptr(), self.v_nrm.data_ptr(),
+                kc.pi_transposed().data_ptr(), vc.Pi.data_ptr(), _native.dtype_code(self.dtype),
+                self.D * self.k_win.element_size())
         return c
 
     def append_one(self, keys: torch.Tensor, values: torch.Tensor) -> bool:
@@ -100,7 +120,8 @@ class _LayerStore:
         step is not of that kind or the tensors are not laid out for it; the general path then runs."""
         rw = self.window_tokens
         if (rw == 0 or self.n_recent != rw or self.w0 + rw + 1 > self.win_cap or self.n_compressed + 1 > self.capacity
-                or keys.dtype != self.dtype or values.dtype != self.dtype or torch.compiler.is_compiling()):
+                or keys.dtype != self.dtype or values.dtype != self.dtype or keys.device != self.device
+                or values.device != self.device or torch.compiler.is_compiling()):
             return False
         rows = self.B * self.H
         strides = []
@@ -114,9 +135,10 @@ class _LayerStore:
         c = self.consts()
         dev = self.device
         with _native._on(dev):
-            rc = _native.lib().tq_append_token(keys.data_ptr(), values.data_ptr(), c[13], strides[0], strides[1],
-                                               c[0], c[1], c[2], self.w0, self.w0 + rw, c[3], c[4], self.D, c[5], c[6],
-                                               c[7], c[8], c[9], c[10], self.capacity, self.n_compressed, rows,
+            rc = _native.lib().tq_append_token(keys.data_ptr(), values.data_ptr(), c.dtype, strides[0], strides[1],
+                                               c.k_win, c.v_win, c.win_stride, self.w0, self.w0 + rw,
+                                               c.table_k, c.table_v, self.D, c.bits_k, c.bits_v,
+                                               c.k_idx, c.k_nrm, c.v_idx, c.v_nrm, self.capacity, self.n_compressed, rows,
                                                _native._stream_handle(dev))
         if rc == _native.ERR_ALIGN:
             return False
@@ -313,7 +335,8 @@ class V3Cache:
         """The fused path of `attend` in one library call (rotate + window, packed history, merge), with the
         scratch kept per stream.  None when the queries are not laid out for it."""
         B, Hq, _, D = query_states.shape
-        if not query_states.is_contiguous() or query_states.dtype not in _native._DTYPE_CODE or st.k_idx is None:
+        if (not query_states.is_contiguous() or query_states.dtype not in _native._DTYPE_CODE or st.k_idx is None
+                or query_states.device != st.device):
             return None
         n_c, n_w = st.n_compressed, st.n_recent
         rows = B * st.H
@@ -331,10 +354,11 @@ class V3Cache:
             base = scratch.data_ptr()
             out = torch.empty_like(query_states)
             code = _native.dtype_code(query_states.dtype)
-            win_off = st.w0 * c[14]
-            rc = L.tq_attend_step(query_states.data_ptr(), code, rows, G, scale, c[11], c[12],
-                                  c[0] + win_off, c[1] + win_off, c[13], n_w, c[2],
-                                  c[7], c[8], c[9], c[10], st.capacity, n_c, c[3], c[4], D, c[5], c[6],
+            win_off = st.w0 * c.vec_bytes
+            rc = L.tq_attend_step(query_states.data_ptr(), code, rows, G, scale, c.pi_k_t, c.pi_v,
+                                  c.k_win + win_off, c.v_win + win_off, c.dtype, n_w, c.win_stride,
+                                  c.k_idx, c.k_nrm, c.v_idx, c.v_nrm, st.capacity, n_c,
+                                  c.table_k, c.table_v, D, c.bits_k, c.bits_v,
                                   base, base + 4 * n_q, base + 4 * (n_q + n_pw), splits, out.data_ptr(), code, stream)
         _native.check(rc, "tq_attend_step")
         return out
