@@ -76,7 +76,7 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     tq_copy_to_lds(lds_lut, job.table + hd->off_lut, 256u * 2u * IPB, tid, T::WAVES * TQ_WAVE);
 
     // tickets: counter[0] = next tile to hand out, counter[1] = blocks of this job that are done
-    __shared__ uint32_t tk[2];
+    __shared__ uint32_t tk[3];         // ticket k of the block sits in slot k % 3
     uint32_t *counter = workspace ? workspace + blockIdx.y * (TQ_WORKSPACE_BYTES_PER_JOB / 4) : nullptr;
     uint32_t fixed_next = blockIdx.x * T::WAVES;
     auto draw = [&]() -> uint32_t {     // thread 0 only
@@ -248,11 +248,11 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
             for (int i = 0; i < NW; ++i) cur[i] = raw[i];
             nrm = half_bits_to_float(norm_bits);
         }
-        uint32_t it = 0;
+        uint32_t s_next = 1u, s_fresh = 2u;                // slots of the next ticket and of the one drawn now
         while (base < n_tiles) {
             uint32_t fresh = 0;
             if (tid == 0) fresh = draw();                 // the ticket after next; its latency hides behind the tile
-            const uint32_t nbase = tk[(it + 1u) & 1u];     // written before the previous barrier
+            const uint32_t nbase = tk[s_next];             // written before the previous barrier
             const uint32_t next = nbase + wave;
             if (tile < n_full) {
                 issue_loads(std::true_type{}, fast_tag, next < n_full ? next : tile);
@@ -275,11 +275,12 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
                 for (int i = 0; i < NW; ++i) part[i] = raw[i];
                 process(std::false_type{}, fast_tag, tile, part, half_bits_to_float(norm_bits));
             }
-            if (tid == 0) tk[it & 1u] = fresh;             // everyone read this slot before the previous barrier
-            __syncthreads();
+            if (tid == 0) tk[s_fresh] = fresh;             // last read two barriers ago (three slots, not two: the first
+            __syncthreads();                               // ticket is read after a barrier that this write could overtake)
             base = nbase;
             tile = next;
-            ++it;
+            s_next = s_fresh;
+            s_fresh = s_fresh == 2u ? 0u : s_fresh + 1u;
         }
     };
     if (fast) run(std::true_type{}); else run(std::false_type{});
