@@ -341,15 +341,16 @@ def test_attend_with_window_only_and_without_window(pkg, oracle):
 @pytest.mark.parametrize("wdtype,qdtype,G,W,splits", [(torch.bfloat16, torch.bfloat16, 4, 128, 3), (torch.float16, torch.float16, 8, 512, 1),
                                                       (torch.float32, torch.float32, 1, 37, 2), (torch.bfloat16, torch.float32, 7, 1, 0),
                                                       (torch.float16, torch.bfloat16, 3, 0, 4), (torch.bfloat16, torch.bfloat16, 16, 300, 2), (torch.float32, torch.float16, 11, 70, 1)])
-def test_attend_prepare_and_merge_against_float64(pkg, wdtype, qdtype, G, W, splits):
+@pytest.mark.parametrize("B", [2, 50])       # 6 rows: one merge block per (row, head); 150 rows: one per row, all heads
+def test_attend_prepare_and_merge_against_float64(pkg, wdtype, qdtype, G, W, splits, B):
     """tq_attend_prepare / tq_attend_merge through the C-ABI against the same arithmetic in float64:
     rotated queries to 1e-5, window records to 1e-5, merged output to the output type's rounding."""
     nat = pkg._native
     L = nat.lib()
-    B, H, D, cap = 2, 3, 128, 520
+    H, D, cap = 3, 128, 520
     rows = B * H
     g = torch.Generator(device="cpu")
-    g.manual_seed(1000 + G * 7 + W)
+    g.manual_seed(1000 + G * 7 + W + B)
     q = (3 * torch.randn(B, H * G, 1, D, generator=g)).to(qdtype).to(DEV)
     kbuf = torch.randn(B, H, cap, D, generator=g).to(wdtype).to(DEV)
     vbuf = torch.randn(B, H, cap, D, generator=g).to(wdtype).to(DEV)
