@@ -839,9 +839,31 @@ __global__ __launch_bounds__(256) void tq_attend_prepare_kernel(PrepareArgs a) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) vload(vtoken(tr, k), vpre[tr][k]);
     }
-    for (uint32_t i = tid; i < MAXG * TQ_HEAD_DIM; i += 256u) {
-        const uint32_t g = i / TQ_HEAD_DIM, c = i % TQ_HEAD_DIM;
-        qt[c][g] = i < G * TQ_HEAD_DIM ? tq_load_elem(a.queries, (size_t)row * G * TQ_HEAD_DIM + i, a.q_dtype) * a.scale : 0.f;
+    {   // the row's queries, scaled, into `qt` (zeros for the padding heads): the element type is looked at once and
+        // the loads of a thread are issued together
+        constexpr int QG = GP < 4 ? 4 : GP;                  // heads written (the rotation reads four at a time)
+        constexpr int NQ = QG * TQ_HEAD_DIM / 256;
+        const size_t q0 = (size_t)row * G * TQ_HEAD_DIM;
+        float qraw[NQ];
+        auto load_all = [&](auto elem) __attribute__((always_inline)) {
+#pragma unroll
+            for (int n = 0; n < NQ; ++n) {
+                const uint32_t i = tid + 256u * (uint32_t)n;
+                qraw[n] = i < G * TQ_HEAD_DIM ? elem(q0 + i) : 0.f;
+            }
+        };
+        if (a.q_dtype == TQ_F32) {
+            load_all([&](size_t i) { return ((const TQ_GLOBAL float *)a.queries)[i]; });
+        } else if (a.q_dtype == TQ_F16) {
+            load_all([&](size_t i) { return (float)__builtin_bit_cast(_Float16, ((const TQ_GLOBAL uint16_t *)a.queries)[i]); });
+        } else {
+            load_all([&](size_t i) { return __uint_as_float((uint32_t)((const TQ_GLOBAL uint16_t *)a.queries)[i] << 16); });
+        }
+#pragma unroll
+        for (int n = 0; n < NQ; ++n) {
+            const uint32_t i = tid + 256u * (uint32_t)n;
+            qt[i % TQ_HEAD_DIM][i / TQ_HEAD_DIM] = qraw[n] * a.scale;
+        }
     }
     __syncthreads();
     if (do_rot) {   // rotated queries: q_rot[g][j] = sum_i Pi[j][i] * q[g][i]; all heads of a coordinate come with 16-byte reads
