@@ -8,6 +8,8 @@
 // and the value side is rotated back once per query head.  These kernels replace the pair
 // "de-quantise the whole history (generation_test_v2.py:131-135), then let the model multiply by
 // it" (score definition: validate_v3.py:87) for single-token decode steps.
+#include <atomic>
+
 #include "tq_device.h"
 
 namespace {
@@ -1086,18 +1088,19 @@ __global__ __launch_bounds__(512) void tq_attend_merge_kernel(MergeArgs a) {
 }
 
 int device_cus(int &cus) {
-    static int cache[64] = {};
+    static std::atomic<int> cache[64];   // per device; threads that race here store the same value
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
     if (dev < 0 || dev >= 64) return TQ_ERR_NO_DEVICE;
-    if (cache[dev] == 0) {
-        int c = 0;
+    int c = cache[dev].load(std::memory_order_relaxed);
+    if (c == 0) {
         e = hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev);
         if (e != hipSuccess) return (int)e;
-        cache[dev] = c > 0 ? c : 1;
+        c = c > 0 ? c : 1;
+        cache[dev].store(c, std::memory_order_relaxed);
     }
-    cus = cache[dev];
+    cus = c;
     return 0;
 }
 

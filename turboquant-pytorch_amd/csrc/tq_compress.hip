@@ -22,6 +22,7 @@
 //   * tiles whose 32 vectors all exist take a path without per-lane predicates: a fixed number
 //     of loads and stores per iteration lets the compiler wait for the prefetched loads alone
 //     (s_waitcnt vmcnt(n)) instead of draining the previous tile's stores on every iteration.
+#include <mutex>
 #include <type_traits>
 
 #include "tq_device.h"
@@ -517,22 +518,28 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
 
 // ---- host side --------------------------------------------------------------------------
 
+constexpr int MAX_DEVICES = 64;
+std::mutex host_state_mutex;   // guards the per-device tables below (filled once per device, read often)
+
 struct DeviceInfo {
+    int dev = 0;
     int cus = 0;
     int lds_optin = 0;
 };
 int query_device(DeviceInfo &info) {
-    static DeviceInfo cache[64];
+    static DeviceInfo cache[MAX_DEVICES];
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
-    if (dev < 0 || dev >= 64) return TQ_ERR_NO_DEVICE;
+    if (dev < 0 || dev >= MAX_DEVICES) return TQ_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(host_state_mutex);
     if (cache[dev].cus == 0) {
         int cus = 0, lds = 0;
         e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         if (e != hipSuccess) return (int)e;
         e = hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev);
         if (e != hipSuccess) return (int)e;
+        cache[dev].dev = dev;
         cache[dev].lds_optin = lds;
         cache[dev].cus = cus > 0 ? cus : 1;
     }
@@ -546,13 +553,18 @@ int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uin
     int rc = query_device(info);
     if (rc) return rc;
     // blocks resident per compute unit for this instantiation (registers and LDS decide): the grid
-    // is that many blocks per unit, each walking its share of the tiles
-    static int resident = 0;
-    if (resident == 0) {
-        int nb = 0;
-        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, tq_compress_kernel<DTYPE, BITS>, CTHREADS, 0);
-        if (e != hipSuccess) return (int)e;
-        resident = nb > 0 ? nb : 1;
+    // is that many blocks per unit, each walking its share of the tiles.  Asked once per device.
+    int resident;
+    {
+        static int resident_on[MAX_DEVICES] = {};
+        std::lock_guard<std::mutex> lock(host_state_mutex);
+        if (resident_on[info.dev] == 0) {
+            int nb = 0;
+            hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, tq_compress_kernel<DTYPE, BITS>, CTHREADS, 0);
+            if (e != hipSuccess) return (int)e;
+            resident_on[info.dev] = nb > 0 ? nb : 1;
+        }
+        resident = resident_on[info.dev];
     }
     const uint32_t bx = tq_blocks_per_job(max_tiles, info.cus * resident, n_jobs);
     dim3 grid(bx, (unsigned)n_jobs, 1), block(CTHREADS, 1, 1);
