@@ -5,8 +5,10 @@
  *   0            success
  *   < 0          argument error (TQ_ERR_*), nothing was launched
  *   > 0          a hipError_t reported by the HIP runtime
- * No entry point allocates or frees device memory, synchronises the device or
- * keeps state between calls; work is enqueued on the caller's stream.
+ * No entry point allocates or frees device memory or synchronises the device;
+ * work is enqueued on the caller's stream.  The library keeps no state between
+ * calls apart from per-device launch parameters it looks up once and the
+ * counters of tq_decompress_batched_noalloc (described there).
  *
  * Each declaration cites the line range of the upstream Python reference
  * (tonbistudio/turboquant-pytorch, turboquant/...) whose behaviour it replaces.
@@ -36,7 +38,8 @@ enum {
     TQ_ERR_CODEBOOK = -6,    /* centroids not finite and strictly ascending */
     TQ_ERR_TABLE = -7,       /* table blob malformed (bad magic / version) */
     TQ_ERR_ALIGN = -8,       /* pointer or stride not aligned as required */
-    TQ_ERR_NO_DEVICE = -9    /* no usable HIP device */
+    TQ_ERR_NO_DEVICE = -9,   /* no usable HIP device */
+    TQ_ERR_CAPACITY = -10    /* request larger than the fixed capacity of an entry point that allocates nothing */
 };
 
 int tq_abi_version(void);
@@ -168,6 +171,22 @@ int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_j
                         int head_dim, void *stream);
 int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
                           int head_dim, void *workspace, void *stream);
+
+/*
+ * tq_decompress_batched for callers that cannot allocate device memory and have no workspace to pass: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, checks and output bytes as tq_decompress_batched; the ticket counters live in a
+ * device array inside the library (TQ_NOALLOC_MAX_JOBS * TQ_WORKSPACE_BYTES_PER_JOB = 128 KiB on each device
+ * the library runs on, held until the process ends) and the words a call uses are cleared by a small kernel on
+ * `stream` before the launch.  More than TQ_NOALLOC_MAX_JOBS jobs: TQ_ERR_CAPACITY, nothing is launched.  The
+ * call allocates and frees nothing.  All calls on one device share the array: two calls that can overlap in
+ * time on one device (different streams, different threads) race on the counters and must be serialised by
+ * the caller.  The first call on a device looks the array's address up in the loaded code object; make that
+ * call outside graph capture.
+ */
+#define TQ_NOALLOC_MAX_JOBS 512
+int tq_decompress_batched_noalloc(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
+                                  int head_dim, void *stream);
 
 /*
  * Decode-time attention on the packed cache, without de-quantising it.  Replaces, for single-token

@@ -87,6 +87,7 @@ EXPORTS = (
     "tq_abi_version", "tq_status_string", "tq_device_count", "tq_bytes_per_vector",
     "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_quantize_host",
     "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched", "tq_workspace_bytes",
+    "tq_decompress_batched_noalloc",
     "tq_scores", "tq_weighted_values", "tq_weighted_values_splits", "tq_attend_partials", "tq_attend_splits",
     "tq_attend_prepare", "tq_attend_merge", "tq_append_token", "tq_attend_step",
 )
@@ -128,6 +129,7 @@ def lib() -> ctypes.CDLL:
     L.tq_attend_partials.argtypes = [vp, vp, vp, vp, ll, ll, ll, vp, vp, ci, ci, ci, vp, ci, ci, vp, vp]
     L.tq_weighted_values.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ll, ci, vp, ci, vp, vp]
     L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp, vp]
+    L.tq_decompress_batched_noalloc.argtypes = [vp, vp, ci, ci, vp]
     L.tq_append_token.argtypes = [vp, vp, ci, ll, ll, vp, vp, ll, ll, ll, vp, vp, ci, ci, ci, vp, vp, vp, vp, ll, ll, ll, vp]
     L.tq_attend_step.argtypes = [vp, ci, ll, ci, ctypes.c_float, vp, vp, vp, vp, ci, ll, ll, vp, vp, vp, vp, ll, ll,
                                  vp, vp, ci, ci, ci, vp, vp, vp, ci, vp, ci, vp]

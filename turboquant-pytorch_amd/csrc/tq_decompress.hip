@@ -21,9 +21,16 @@
 // jobs too small to matter, the fixed assignment is used.  Thread 0 draws one ticket ahead and
 // hands it to the block through LDS; one barrier per ticket.  The last block of a job to finish
 // sets the job's counters back to zero, so a workspace that was zero before a launch is zero after it.
+#include <mutex>
 #include <type_traits>
 
 #include "tq_device.h"
+
+// Ticket counters of tq_decompress_batched_noalloc: the workspace that tq_decompress_batched takes from its
+// caller, held by the library instead (TQ_NOALLOC_MAX_JOBS jobs x TQ_WORKSPACE_BYTES_PER_JOB bytes on every
+// device the library runs on, until the process ends).  In host code this name is only a handle for
+// hipGetSymbolAddress; launches receive the per-device address kept by static_counters().
+static __device__ __align__(256) uint32_t scratch[TQ_NOALLOC_MAX_JOBS * (TQ_WORKSPACE_BYTES_PER_JOB / 4)];
 
 namespace {
 
@@ -297,14 +304,25 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     }
 }
 
+// Sets n 32-bit words to zero.  A kernel rather than hipMemsetAsync, so that a caller may record the launch
+// into a HIP graph.
+__global__ void tq_clear_words_kernel(uint32_t *p, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
 // ---- host side --------------------------------------------------------------------------
 
+constexpr int MAX_DEVICES = 64;
+std::mutex host_state_mutex;   // guards the per-device tables below (filled once per device, read often)
+
 int device_cus(int &cus) {
-    static int cache[64] = {};
+    static int cache[MAX_DEVICES] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
-    if (dev < 0 || dev >= 64) return TQ_ERR_NO_DEVICE;
+    if (dev < 0 || dev >= MAX_DEVICES) return TQ_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(host_state_mutex);
     if (cache[dev] == 0) {
         int c = 0;
         e = hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev);
@@ -312,6 +330,26 @@ int device_cus(int &cus) {
         cache[dev] = c > 0 ? c : 1;
     }
     cus = cache[dev];
+    return 0;
+}
+
+// Address of `scratch` on the current device.  Every device holds its own copy of the array at its own
+// address, so the address is looked up once per device, with that device current, and kept.
+int static_counters(uint32_t **out) {
+    static uint32_t *address[MAX_DEVICES] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return TQ_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(host_state_mutex);
+    if (!address[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return TQ_ERR_NO_DEVICE;
+        address[dev] = static_cast<uint32_t *>(p);
+    }
+    *out = address[dev];
     return 0;
 }
 
@@ -323,14 +361,19 @@ int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, u
     int rc = device_cus(cus);
     if (rc) return rc;
     constexpr size_t lds = decompress_lds_bytes<DTYPE>();
-    static bool configured[64] = {};
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if (!configured[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&tq_decompress_kernel<DTYPE, IPB>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    {   // the kernel's LDS limit is raised once per device (one flag table per instantiation)
+        static bool configured[MAX_DEVICES] = {};
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
         if (e != hipSuccess) return (int)e;
-        configured[dev] = true;
+        if (dev < 0 || dev >= MAX_DEVICES) return TQ_ERR_NO_DEVICE;
+        std::lock_guard<std::mutex> lock(host_state_mutex);
+        if (!configured[dev]) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&tq_decompress_kernel<DTYPE, IPB>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return (int)e;
+            configured[dev] = true;
+        }
     }
     const uint32_t want = (max_tiles + T::WAVES - 1) / T::WAVES;
     const uint32_t bx = tq_blocks_per_job(want, cus, n_jobs);
@@ -414,12 +457,9 @@ extern "C" long long tq_workspace_bytes(int n_jobs) {
     return (long long)TQ_WORKSPACE_BYTES_PER_JOB * (n_jobs > 0 ? n_jobs : 1);
 }
 
-extern "C" int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
-                                     int head_dim, void *workspace, void *stream) {
-    if (n_jobs == 0) return TQ_OK;
-    if (!jobs_host || !jobs_dev) return TQ_ERR_NULL;
-    if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
-    if ((uintptr_t)workspace & 63u) return TQ_ERR_ALIGN;
+namespace {
+int decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs, int head_dim, void *workspace,
+                       void *stream) {
     long long max_vec = 0;
     for (int i = 0; i < n_jobs; ++i) {
         const tq_job &j = jobs_host[i];
@@ -436,4 +476,33 @@ extern "C" int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs
     TqDevJob none{};
     return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec + 31) / 32),
                     workspace, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+extern "C" int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
+                                     int head_dim, void *workspace, void *stream) {
+    if (n_jobs == 0) return TQ_OK;
+    if (!jobs_host || !jobs_dev) return TQ_ERR_NULL;
+    if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
+    if ((uintptr_t)workspace & 63u) return TQ_ERR_ALIGN;
+    return decompress_batched(jobs_host, jobs_dev, n_jobs, head_dim, workspace, stream);
+}
+
+extern "C" int tq_decompress_batched_noalloc(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
+                                             int head_dim, void *stream) {
+    if (n_jobs == 0) return TQ_OK;
+    if (!jobs_host || !jobs_dev) return TQ_ERR_NULL;
+    if (n_jobs < 0) return TQ_ERR_SIZE;
+    if (n_jobs > TQ_NOALLOC_MAX_JOBS) return TQ_ERR_CAPACITY;
+    uint32_t *counters = nullptr;
+    const int rc = static_counters(&counters);
+    if (rc) return rc;
+    // The array keeps what the last call left.  A launch that completed left zeros, one that failed half-way
+    // may not have: the words this call uses are cleared first, on the same stream.
+    const uint32_t words = (uint32_t)n_jobs * (TQ_WORKSPACE_BYTES_PER_JOB / 4);
+    hipLaunchKernelGGL(tq_clear_words_kernel, dim3((words + 255u) / 256u), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       counters, words);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return decompress_batched(jobs_host, jobs_dev, n_jobs, head_dim, counters, stream);
 }

@@ -131,6 +131,7 @@ const char *tq_status_string(int status) {
         case TQ_ERR_TABLE: return "malformed codec table";
         case TQ_ERR_ALIGN: return "pointer or stride not 16-byte aligned";
         case TQ_ERR_NO_DEVICE: return "no usable HIP device";
+        case TQ_ERR_CAPACITY: return "request exceeds the fixed capacity of an entry point that allocates nothing";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
