@@ -30,7 +30,14 @@
 namespace {
 
 #ifndef TQ_C16_WAVES
-#define TQ_C16_WAVES 2
+#define TQ_C16_WAVES 3
+#endif
+// tiles of 16-bit input that a block keeps in LDS or on their way there (direct-to-LDS loads)
+#ifndef TQ_RING
+#define TQ_RING 4
+#endif
+#ifndef TQ_PIN_SCHEDULE
+#define TQ_PIN_SCHEDULE 1
 #endif
 template <int DTYPE> struct InTraits;
 template <> struct InTraits<TQ_F16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = TQ_C16_WAVES; };
@@ -127,6 +134,23 @@ __device__ __forceinline__ uint32_t copy_shift_rt(uint32_t c) {
     return IPB == 1 ? 8u * c : 8u * (c / IPB) + (uint32_t)BITS * (c % IPB);
 }
 
+// s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// calls step(k) for k = FROM .. TO-1 until one of them reports the end; true = ended
+template <uint32_t FROM, uint32_t TO, typename F>
+__device__ __forceinline__ bool run_tail(F &step) {
+    if constexpr (FROM >= TO) {
+        return false;
+    } else {
+        if (step(std::integral_constant<uint32_t, FROM>{})) return true;
+        return run_tail<FROM + 1, TO>(step);
+    }
+}
+
 template <int DTYPE, int BITS>
 __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compress_kernel(TqDevJob job0, const tq_job *jobs) {
     using T = InTraits<DTYPE>;
@@ -140,11 +164,13 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     constexpr int NB = P::NB, NW = P::NW;
 
     // grid copies first, so that their LDS addresses are small compile-time immediates
+    constexpr int RING = ELEM == 2 ? TQ_RING : 2;     // staged tiles
     __shared__ __attribute__((aligned(16))) uint8_t lds_grid[TQ_GRID_LDS_BYTES];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_stage[2][STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_stage[RING][STAGE];
     __shared__ float lds_ss[2][32];   // sum of squares of the tile's vectors (16-bit inputs)
+    __shared__ __attribute__((aligned(16))) float lds_part[2][32][4];   // the same, one share per wave (pipelined path)
 
-    const TqDevJob job = tq_load_job(job0, jobs, blockIdx.y, ELEM);
+    const TqDevJob job = tq_uniform_job(tq_load_job(job0, jobs, blockIdx.y, ELEM));
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
@@ -156,7 +182,11 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
 
     const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
 
-    // ---- this wave's quarter of the rotation, resident for the whole kernel
+    // ---- this wave's quarter of the rotation, resident for the whole kernel.  Wave w walks the 16-input
+    // steps of the contraction in the order 2w, 2w+1, ... (mod 8): its first two steps then cover inputs
+    // [32w, 32w+32), the share of the vector whose squares it sums in the pipelined path.
+    // (fp32 inputs sum their squares while they walk the steps, every wave over the whole vector: same order in all waves)
+    const uint32_t step0 = ELEM == 2 ? 2u * wave : 0u;
     tq_u4 areg[T::TERMS][TQ_STEPS];
     {
         const uint8_t *src = job.table + (DTYPE == TQ_F16 ? hd->off_a_f16 : hd->off_a_bf16);
@@ -165,7 +195,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
 #pragma unroll
             for (int s = 0; s < TQ_STEPS; ++s)
                 areg[term][s] = tq_gload16(src + (size_t)term * TQ_OPERAND_BYTES +
-                                           (((size_t)wave * TQ_STEPS + s) * 64 + lane) * 16);
+                                           (((size_t)wave * TQ_STEPS + ((s + step0) & 7u)) * 64 + lane) * 16);
     }
     {   // one grid copy per code position, base pre-shifted
         const uint32_t cells = hd->grid_cells;
@@ -183,14 +213,12 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     const uint32_t n = lane & 31u, hk = lane >> 5;                    // role in the MFMA: column, half
     const bool one_row = job.tokens >= job.n_vec;
 
-    // LDS offsets that do not change from tile to tile
-    uint32_t st_off[NLOAD];
-#pragma unroll
-    for (int j = 0; j < NLOAD; ++j) {
+    // LDS offset of this lane's piece of load j (computed where it is used: these paths are not the hot one)
+    auto st_off = [&](int j) {
         const uint32_t vl = (wave * NLOAD + j) * VEC_PER_LOAD + ld_vec;
         const uint32_t swz = (ELEM == 2) ? (vl & 15u) : ((vl & 15u) << 1);
-        st_off[j] = vl * VEC_BYTES + ((ld_piece ^ swz) << 4);
-    }
+        return vl * VEC_BYTES + ((ld_piece ^ swz) << 4);
+    };
 
     tq_u4 pre[NLOAD];
     // loads of this wave's quarter of tile `tl`, generic addressing (any strides, tail clamped)
@@ -206,21 +234,27 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     };
 
     // Park this wave's quarter of the prefetched tile in LDS (swizzled: the operand reads are conflict
-    // free).  For 16-bit inputs the squares are summed here, where every element is touched once:
-    // 16 lanes hold one vector, an inclusive row scan leaves the total in the last of them.
+    // free).  For 16-bit inputs the squares are summed here, where every element is touched once: the 16
+    // lanes of a DPP row hold the 16 pieces of one vector.  The order of the additions is the one of the
+    // pipelined path below (pieces 4w + h and 4w + 2 + h as one chain, the two chains of a wave's share
+    // added, the shares added pairwise), so that a vector gets the same norm whichever path compresses it.
+    auto row_shr = [](float v, auto n_tag) {
+        constexpr int N = decltype(n_tag)::value;
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x110 + N, 0xf, 0xf, true));
+    };
     auto park = [&](uint32_t b, const tq_u4 (&src)[NLOAD]) {
         uint8_t *stage = lds_stage[b];
 #pragma unroll
-        for (int j = 0; j < NLOAD; ++j) *reinterpret_cast<tq_u4 *>(stage + st_off[j]) = src[j];
+        for (int j = 0; j < NLOAD; ++j) *reinterpret_cast<tq_u4 *>(stage + st_off(j)) = src[j];
         if constexpr (ELEM == 2) {
 #pragma unroll
             for (int j = 0; j < NLOAD; ++j) {
-                float x = sumsq8<DTYPE>(src[j], 0.f);
-                x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x111, 0xf, 0xf, true));
-                x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x112, 0xf, 0xf, true));
-                x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x114, 0xf, 0xf, true));
-                x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x118, 0xf, 0xf, true));
-                if ((lane & 15u) == 15u) lds_ss[b][(wave * NLOAD + j) * VEC_PER_LOAD + ld_vec] = x;
+                const float own = sumsq8<DTYPE>(src[j], 0.f);
+                const float chain = sumsq8<DTYPE>(src[j], row_shr(own, std::integral_constant<int, 2>{}));   // pieces p - 2, p
+                const float share = chain + row_shr(chain, std::integral_constant<int, 1>{});               // at p % 4 == 3
+                const float pair = share + row_shr(share, std::integral_constant<int, 4>{});                // at p == 7, 15
+                const float total = pair + row_shr(pair, std::integral_constant<int, 8>{});                 // at p == 15
+                if ((lane & 15u) == 15u) lds_ss[b][(wave * NLOAD + j) * VEC_PER_LOAD + ld_vec] = total;
             }
         }
     };
@@ -229,14 +263,15 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     // (1) rotation step s of the tile parked in `stage`: acc[r] += sum over 16 inputs of
     //     Pi[32w + 16h + r][k] * x_n[k]  (raw, unnormalised); fp32 inputs also sum their squares here
     auto rotate_step = [&](const uint8_t *stage, int s, tq_f16v &acc, float &ss0, float &ss1) {
+        const uint32_t sg = ((uint32_t)s + step0) & 7u;   // the step of the contraction that areg[.][s] belongs to
         if constexpr (ELEM == 2) {
-            const uint32_t piece = 2u * s + hk;
+            const uint32_t piece = 2u * sg + hk;
             const tq_u4 bop = *reinterpret_cast<const tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4));
 #pragma unroll
             for (int term = 0; term < T::TERMS; ++term)
                 acc = (DTYPE == TQ_F16) ? mfma_f16(areg[term][s], bop, acc) : mfma_bf16(areg[term][s], bop, acc);
         } else {
-            const uint32_t piece = 2u * (2u * s + hk);
+            const uint32_t piece = 2u * (2u * sg + hk);
             const uint32_t swz = (n & 15u) << 1;
             const uint8_t *row = stage + n * VEC_BYTES;
             const tq_u4 q0 = *reinterpret_cast<const tq_u4 *>(row + ((piece ^ swz) << 4));
@@ -258,14 +293,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
 
     // (2) norm of the lane's vector and the two scale factors of the code search
     struct Scale { float nrm, inv, inv_cell; };
-    auto scale_of = [&](uint32_t b, float ss0, float ss1) {
-        float ss;
-        if constexpr (ELEM == 2) {
-            ss = lds_ss[b][n];
-        } else {
-            ss = ss0 + ss1;                 // both lanes of a vector hold half of the squares
-            ss += __shfl_xor(ss, 32);
-        }
+    auto scale_from_ss = [&](float ss) {
         Scale sc;
         // sqrt: reciprocal square root plus one Newton step is correctly rounded except for a
         // vanishing fraction of inputs.  Sums below 1e-35 (norm < 1e-17: it vanishes both in
@@ -282,6 +310,16 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
         if (DTYPE == TQ_F16) sc.inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
         sc.inv_cell = sc.inv * grid_scale;   // grid_scale is a power of two: exact
         return sc;
+    };
+    auto scale_of = [&](uint32_t b, float ss0, float ss1) {
+        float ss;
+        if constexpr (ELEM == 2) {
+            ss = lds_ss[b][n];
+        } else {
+            ss = ss0 + ss1;                 // both lanes of a vector hold half of the squares
+            ss += __shfl_xor(ss, 32);
+        }
+        return scale_from_ss(ss);
     };
 
     // (3) code search + packing.  Lane (n, hk) of wave w holds coordinates 32w + 16hk + r.
@@ -362,126 +400,195 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     uint32_t buf = 0;
     uint32_t words[NW];
     float nrm;
-    if (tile < n_full && ELEM == 2 && one_row) {
+    // the pipelined path addresses a tile's vectors with 32-bit offsets from a scalar base
+    const bool dma_ok = one_row && job.token_stride < (1ll << 26);
+    if (tile < n_full && ELEM == 2 && dma_ok) {
         if constexpr (ELEM == 2) {
-            // Single-row jobs with 16-bit elements (the KV-cache case).  Software pipeline inside the
-            // wave, over this block's full tiles t_0 .. t_{m-1}: iteration j
-            //   starts the loads of t_{j+2} into the register set that t_j has just left,
-            //   passes the barrier that publishes t_j in LDS buffer j % 2,
-            //   rotates t_j on the matrix cores while searching and packing the codes of t_{j-1},
-            //   whose rotated coordinates wait in the other accumulator set: the two instruction
-            //   streams are independent, so the VALU work fills the issue slots under the MFMAs,
-            //   stores t_{j-1} and parks t_{j+1} (loaded an iteration ago) in the other LDS buffer.
-            // Loads, stores and the wait for the older loads sit in one straight line and none is
-            // predicated, so the wait is s_waitcnt vmcnt(n > 0): stores and the newer loads stay in
-            // flight.  Two tiles per wave are on their way from memory at any time.  Per-lane
-            // pointers run along the job: a handful of 64-bit adds per tile, no index arithmetic.
-            const long long jstep = (long long)VEC_PER_LOAD * job.token_stride;
-            const long long in_step = (long long)tile_stride * 32 * job.token_stride;
-            const uint8_t *ld = job.states + (long long)(tile * 32u + (wave * NLOAD) * VEC_PER_LOAD + ld_vec) * job.token_stride + ld_piece * 16u;
-            uint8_t *cd = job.idx_bytes + (size_t)(tile * 32u + n) * (8 * NB) + lane_slot;
-            uint16_t *nd = job.vec_norms + (size_t)tile * 32u + n;
-            const size_t cd_step = (size_t)tile_stride * 32u * (8 * NB), nd_step = (size_t)tile_stride * 32u;
+            // Single-row jobs with 16-bit elements (the KV-cache case): a software pipeline over this block's full
+            // tiles t_0 .. t_{m-1}.  Tiles travel from memory straight into a ring of RING LDS slots
+            // (global_load_lds_dwordx4: no registers, no LDS write instructions); iteration j
+            //   waits for its own loads of t_j (issued RING-1 iterations ago) and passes the barrier: t_j is complete
+            //   in slot j % RING, and everybody has finished reading t_{j-1};
+            //   starts the loads of t_{j+RING-1} into the slot that t_{j-1} has just left;
+            //   rotates t_j on the matrix cores while it searches and packs the codes of t_{j-1}, whose rotated
+            //   coordinates wait in the other accumulator set (two independent instruction streams: the VALU work
+            //   fills the issue slots under the MFMAs); the scale of t_{j-1} comes from the four waves' shares of
+            //   its sum of squares, written an iteration ago;
+            //   sums the squares of its own share of t_j from the first two operands it feeds to the matrix cores;
+            //   stores t_{j-1}.
+            // The loads are invisible to the compiler (inline assembly), so it never waits for them; the explicit
+            // s_waitcnt counts the younger vector-memory operations of the wave, which is fixed: 2 loads and
+            // 2 stores per iteration.
+            constexpr int P = RING;
+            static_assert(NLOAD == 2 && P >= 2 && P <= 6, "the wait counts below assume two loads per wave and tile");
             const uint32_t m = (n_full - tile + tile_stride - 1u) / tile_stride;   // this block's full tiles
-            uint32_t ahead = m - 1u;      // tiles beyond the one `ld` points at
-            uint32_t to_rotate = m;
-
-            tq_u4 set0[NLOAD], set1[NLOAD];
-            // past the block's last tile the pointer stays where it is: a harmless re-read, never used
-            auto load_next = [&](tq_u4 (&dst)[NLOAD]) {
+            const long long in_step = (long long)tile_stride * 32 * job.token_stride;
+            // lane i of load j fills bytes [16 i, 16 i + 16) of KiB (wave * NLOAD + j) of the slot: vector
+            // vl = (wave * NLOAD + j) * 4 + i / 16, position i % 16, which has to hold piece (i % 16) ^ (vl & 15)
+            uint32_t src_off[NLOAD];
 #pragma unroll
-                for (int j = 0; j < NLOAD; ++j) dst[j] = tq_gload16(ld + j * jstep);
-                ld += ahead ? in_step : 0;
+            for (int j = 0; j < NLOAD; ++j) {
+                const uint32_t vl = (wave * NLOAD + j) * VEC_PER_LOAD + ld_vec;
+                src_off[j] = vl * (uint32_t)job.token_stride + ((ld_piece ^ (vl & 15u)) << 4);
+            }
+            const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
+                (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)&lds_stage[0][0] + wave * (NLOAD * 1024u));
+            const uint8_t *src = job.states + (long long)tile * 32 * job.token_stride;   // the same in every lane
+            uint32_t ahead = m - 1u;      // tiles beyond the one `src` points at
+            // past the block's last tile the pointer stays where it is: a harmless re-read, never used
+            auto issue = [&](uint32_t slot) {
+                const uint64_t a = (uint64_t)(uintptr_t)src;
+                // (the builtin returns int: widen through uint32_t, or the low half is sign-extended into the high one)
+                const uint32_t a_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+                const uint32_t a_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)a);
+                const uint64_t base = ((uint64_t)a_hi << 32) | (uint64_t)a_lo;
+#pragma unroll
+                for (int j = 0; j < NLOAD; ++j) {
+                    const uint32_t dst = lds_wave + slot * (uint32_t)STAGE + j * 1024u;
+                    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                                 :: "s"(dst), "v"(src_off[j]), "s"(base) : "memory", "m0");
+                }
+                src += ahead ? in_step : 0;
                 ahead -= ahead ? 1u : 0u;
             };
-            // iteration j: `fresh` receives t_{j+2}, `ready` holds t_{j+1}; `acc_new` receives t_j,
-            // (`acc_old`, `sc_old`) belong to t_{j-1}
-            auto iteration = [&](auto with_search, uint32_t b, tq_u4 (&fresh)[NLOAD], const tq_u4 (&ready)[NLOAD],
-                                 tq_f16v &acc_new, Scale &sc_new, const tq_f16v &acc_old, const Scale &sc_old) {
+            // operand addresses inside a slot, in this wave's step order
+            uint32_t op_off[TQ_STEPS];
+#pragma unroll
+            for (int i = 0; i < TQ_STEPS; ++i) {
+                const uint32_t piece = 2u * ((i + step0) & 7u) + hk;
+                op_off[i] = n * VEC_BYTES + ((piece ^ (n & 15u)) << 4);
+            }
+            const uint32_t bperm_other_half = (lane ^ 32u) << 2;
+
+            // output addresses: a base that is the same in every lane, advanced per tile, plus a per-lane constant
+            uint8_t *cd = job.idx_bytes + (size_t)tile * 32u * (8 * NB);
+            uint16_t *nd = job.vec_norms + (size_t)tile * 32u;
+            const uint32_t cd_lane = n * (8 * NB) + lane_slot, nd_lane = n;
+            const size_t cd_step = (size_t)tile_stride * 32u * (8 * NB), nd_step = (size_t)tile_stride * 32u;
+
+            auto scale_from_shares = [&](uint32_t par) {
+                const float4 q = *reinterpret_cast<const float4 *>(&lds_part[par][n][0]);
+                return scale_from_ss((q.x + q.y) + (q.z + q.w));
+            };
+            // iteration j: slot = j % P; `acc_new` receives t_j, `acc_old` holds t_{j-1}
+            auto iteration = [&](auto with_search, auto slot_tag, bool warm, uint32_t par, tq_f16v &acc_new, const tq_f16v &acc_old) {
                 constexpr bool SEARCH = decltype(with_search)::value;
-                load_next(fresh);
+                constexpr uint32_t SLOT = decltype(slot_tag)::value;
+                // younger than the loads of t_j: the loads of P-2 tiles and, once the pipeline is full, the stores of P-1
+                if (warm) wait_vmcnt<2 * (P - 2) + 2 * (P - 1)>(); else wait_vmcnt<2 * (P - 2)>();
                 __syncthreads();
+                issue((SLOT + P - 1u) % P);
+                const uint8_t *stage = lds_stage[SLOT];
+                auto operand = [&](int i) { return *reinterpret_cast<const tq_u4 *>(stage + op_off[i]); };
+                auto mfma = [&](int term, int i, tq_u4 bop) {
+                    acc_new = (DTYPE == TQ_F16) ? mfma_f16(areg[term][i], bop, acc_new) : mfma_bf16(areg[term][i], bop, acc_new);
+                };
                 acc_new = tq_zero16();
                 Search z;
                 search_begin(z);
-                const uint8_t *stage = lds_stage[b];
-                auto operand = [&](int s) {
-                    const uint32_t piece = 2u * s + hk;
-                    return *reinterpret_cast<const tq_u4 *>(stage + n * VEC_BYTES + ((piece ^ (n & 15u)) << 4));
-                };
-                auto mfma = [&](int term, int s, tq_u4 bop) {
-                    acc_new = (DTYPE == TQ_F16) ? mfma_f16(areg[term][s], bop, acc_new) : mfma_bf16(areg[term][s], bop, acc_new);
-                };
-                // LDS reads run one step ahead of their use: the operand of step s + 1 and the grid
-                // cells of coordinates 2s + 2, 2s + 3 are requested before the MFMAs of step s
+                Scale sc_old{};
+                float share = 0.f;
+                // Order of the instruction stream: the first step's MFMAs come before anything that depends on the
+                // scale of t_{j-1} (an LDS read, a reciprocal square root); the search runs one step behind:
+                // coordinates 2i-2, 2i-1 are looked up in step i-1 and applied in step i.
                 tq_u4 bop = operand(0);
                 tq_u2 c0 = {0u, 0u}, c1 = {0u, 0u};
-                if constexpr (SEARCH) {
-                    c0 = search_lookup(0, acc_old, sc_old);
-                    c1 = search_lookup(1, acc_old, sc_old);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
-                }
 #pragma unroll
-                for (int s = 0; s < TQ_STEPS; ++s) {
+                for (int i = 0; i < TQ_STEPS; ++i) {
                     tq_u4 bop_next = bop;
                     tq_u2 n0 = c0, n1 = c1;
-                    if (s + 1 < TQ_STEPS) {
-                        bop_next = operand(s + 1);
-                        if constexpr (SEARCH) { n0 = search_lookup(2 * s + 2, acc_old, sc_old); n1 = search_lookup(2 * s + 3, acc_old, sc_old); }
-                    }
-                    mfma(0, s, bop);
-                    if constexpr (SEARCH) search_apply(z, 2 * s, acc_old, sc_old, c0);
-                    mfma(1, s, bop);
-                    if constexpr (SEARCH) search_apply(z, 2 * s + 1, acc_old, sc_old, c1);
+                    if (i + 1 < TQ_STEPS) bop_next = operand(i + 1);
                     if constexpr (SEARCH) {
-                        // pin the order: address arithmetic, the step's LDS reads, then each MFMA
-                        // followed by the VALU work that fills its shadow
-                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);   // VALU
-                        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);   // DS read
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
-                        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                        if (i >= 1) { n0 = search_lookup(2 * i - 2, acc_old, sc_old); n1 = search_lookup(2 * i - 1, acc_old, sc_old); }
                     }
+                    mfma(0, i, bop);
+                    if (i < 2) share = sumsq8<DTYPE>(bop, share);
+                    if constexpr (SEARCH) {
+                        if (i == 0) sc_old = scale_from_shares(par ^ 1u);
+                        if (i >= 2) search_apply(z, 2 * i - 4, acc_old, sc_old, c0);
+                    }
+                    mfma(1, i, bop);
+                    if constexpr (SEARCH) {
+                        if (i >= 2) search_apply(z, 2 * i - 3, acc_old, sc_old, c1);
+                    }
+                    if (i == 1) {
+                        share += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((int)bperm_other_half, __builtin_bit_cast(int, share)));
+                        lds_part[par][n][wave] = share;
+                    }
+#if TQ_PIN_SCHEDULE
+                    if constexpr (SEARCH) {
+                        // pin the order: address arithmetic, the step's LDS reads, then each MFMA followed by the
+                        // VALU work that fills its shadow
+                        if (i == 0) {
+                            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // DS read: next operand, shares
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+                            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);  // VALU: squares, scale
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+                        } else if (i == 1) {
+                            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        } else {
+                            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);   // VALU
+                            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);   // DS read
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+                            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                        }
+                    }
+#endif
                     bop = bop_next; c0 = n0; c1 = n1;
                 }
-                const float ss0 = 0.f, ss1 = 0.f;
-                sc_new = scale_of(b, ss0, ss1);
                 if constexpr (SEARCH) {
+                    search_apply(z, 12, acc_old, sc_old, c0);
+                    search_apply(z, 13, acc_old, sc_old, c1);
+                    search_coord(z, 14, acc_old, sc_old);
+                    search_coord(z, 15, acc_old, sc_old);
                     search_end(z, words);
-                    store(cd, nd, words, sc_old.nrm);
+                    store(cd + cd_lane, nd + nd_lane, words, sc_old.nrm);
                     cd += cd_step;
                     nd += nd_step;
                 }
-                park(b ^ 1u, ready);
             };
-            auto drain = [&](const tq_f16v &acc_old, const Scale &sc_old) {
+            auto drain = [&](uint32_t par, const tq_f16v &acc_old) {    // par: parity of the iteration that would come next
+                __syncthreads();    // the last tile's shares of the sum of squares are complete
+                const Scale sc_old = scale_from_shares(par ^ 1u);
                 Search z;
                 search_begin(z);
 #pragma unroll
                 for (int q = 0; q < 16; ++q) search_coord(z, q, acc_old, sc_old);
                 search_end(z, words);
-                store(cd, nd, words, sc_old.nrm);
+                store(cd + cd_lane, nd + nd_lane, words, sc_old.nrm);
             };
 
-            load_next(set0);
-            load_next(set1);
-            park(0u, set0);
+#pragma unroll
+            for (int p = 0; p < P - 1; ++p) issue((uint32_t)p);
             tq_f16v acc_a, acc_b;
-            Scale sc_a, sc_b;
-            iteration(std::false_type{}, 0u, set0, set1, acc_a, sc_a, acc_a, sc_a);
-            --to_rotate;
-            while (true) {
-                if (to_rotate == 0u) { drain(acc_a, sc_a); break; }
-                iteration(std::true_type{}, 1u, set1, set0, acc_b, sc_b, acc_a, sc_a);
-                --to_rotate;
-                if (to_rotate == 0u) { drain(acc_b, sc_b); break; }
-                iteration(std::true_type{}, 0u, set0, set1, acc_a, sc_a, acc_b, sc_b);
-                --to_rotate;
-            }
+            uint32_t done = 0;     // iterations finished
+            iteration(std::false_type{}, std::integral_constant<uint32_t, 0>{}, false, 0u, acc_a, acc_a);
+            ++done;
+            // unrolled by U = lcm(2 accumulator sets, P slots); iteration j runs variant j % U
+            constexpr uint32_t U = (P % 2 == 0) ? P : 2 * P;
+            auto step = [&](auto k_tag) -> bool {    // true = all tiles rotated
+                constexpr uint32_t K = decltype(k_tag)::value;
+                if (done == m) return true;
+                if constexpr (K & 1u) iteration(std::true_type{}, std::integral_constant<uint32_t, K % P>{}, done >= (uint32_t)P, 1u, acc_b, acc_a);
+                else iteration(std::true_type{}, std::integral_constant<uint32_t, K % P>{}, done >= (uint32_t)P, 0u, acc_a, acc_b);
+                ++done;
+                return false;
+            };
+            bool fin = run_tail<1, U>(step);         // the first trip starts at iteration 1
+            while (!fin) fin = run_tail<0, U>(step);
+            // the accumulator set filled last belongs to iteration done - 1
+            if (done & 1u) drain(1u, acc_a); else drain(0u, acc_b);
+            wait_vmcnt<0>();       // re-reads past the last tile may still be on their way into the ring
+            __syncthreads();
             tile += m * tile_stride;
-            buf = m & 1u;   // the buffer nobody reads while slower waves finish the last iteration
+            buf = 0u;
         }
     } else if (tile < n_full) {
         // General case (several rows with their own stride, fp32 elements).  Iteration k: start the

@@ -46,6 +46,27 @@ __device__ __forceinline__ TqDevJob tq_load_job(const TqDevJob &single, const tq
     return job;
 }
 
+// The job's fields are the same in every lane of a block, but a record fetched from the job array arrives in vector
+// registers (the compiler cannot prove that nobody writes the array).  Moving every field into scalar registers keeps
+// them out of the vector register budget and lets the address arithmetic on them run on the scalar unit.
+__device__ __forceinline__ uint32_t tq_uniform32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ uint64_t tq_uniform64(uint64_t v) {
+    return ((uint64_t)tq_uniform32((uint32_t)(v >> 32)) << 32) | (uint64_t)tq_uniform32((uint32_t)v);
+}
+__device__ __forceinline__ TqDevJob tq_uniform_job(const TqDevJob &j) {
+    TqDevJob u;
+    u.states = reinterpret_cast<const uint8_t *>((uintptr_t)tq_uniform64((uint64_t)(uintptr_t)j.states));
+    u.idx_bytes = reinterpret_cast<uint8_t *>((uintptr_t)tq_uniform64((uint64_t)(uintptr_t)j.idx_bytes));
+    u.vec_norms = reinterpret_cast<uint16_t *>((uintptr_t)tq_uniform64((uint64_t)(uintptr_t)j.vec_norms));
+    u.table = reinterpret_cast<const uint8_t *>((uintptr_t)tq_uniform64((uint64_t)(uintptr_t)j.table));
+    u.n_vec = tq_uniform32(j.n_vec);
+    u.tokens = tq_uniform32(j.tokens);
+    u.packed_row_stride = tq_uniform32(j.packed_row_stride);
+    u.row_stride = (long long)tq_uniform64((uint64_t)j.row_stride);
+    u.token_stride = (long long)tq_uniform64((uint64_t)j.token_stride);
+    return u;
+}
+
 // Byte offset of vector v inside `states`.
 __device__ __forceinline__ long long tq_vec_offset(const TqDevJob &job, uint32_t v) {
     if (job.tokens >= job.n_vec) return (long long)v * job.token_stride;  // one row
