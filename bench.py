@@ -28,6 +28,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0     # MI355X published HBM3E bandwidth, GB/s
+MFMA_PEAK_PFLOPS = 2.5    # MI355X published dense bf16 / fp16 matrix rate, PFLOP/s
+# Matrix-core work per vector: the rotation is a 128 x 128 contraction (32 768 flop).  compress runs it over the two
+# 16-bit terms of the split rotation (fp32-grade result from 16-bit operands), decompress over one.
+ROTATION_FLOP = 2 * 128 * 128
+MFMA_PASSES = {"compress": 2, "decompress": 1}
 
 WORKLOADS = {
     # name: layers, batch, kv heads, tokens, dtype, key_bits, value_bits, protected_layers
@@ -68,41 +73,73 @@ def synth_kv(torch, shape, seed, dtype, device):
     return (x * ch * tok).to(dtype)
 
 
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return platform.processor() or platform.machine()
+
+
+def _timed_sample(run, make_input, share, budget_s, probe_n=2048, cap=4_000_000):
+    """Times run(x) on a sample sized so that it takes about share * budget_s seconds; returns (vectors/s, n)."""
+    x = make_input(probe_n)
+    run(x)                                   # first call: thread pools, page faults
+    t0 = time.perf_counter()
+    run(x)
+    probe = time.perf_counter() - t0
+    n = int(min(max(probe_n * budget_s * share / max(probe, 1e-6), 2 * probe_n), cap))
+    x = make_input(n)
+    t0 = time.perf_counter()
+    run(x)
+    return n / (time.perf_counter() - t0), n
+
+
 def cpu_baseline(pkg, widths, budget_s=20.0):
-    """The C restatement of the reference algorithm (oracle/tq_oracle.c, OpenMP over vectors), timed
-    on this machine's host cores on a bounded sample: `widths` = {bits: share of vectors}."""
+    """The reference's CPU path on this machine's host cores, on a bounded sample: `widths` = {bits: share of
+    vectors}.  Primary figure: the reference's op sequence issued as torch CPU operators on all cores
+    (oracle.TorchCpuOracle: fp32 cast, norm, divide, sgemm, [n,D,L] broadcast / abs / argmin, int64 pack; unpack,
+    gather, sgemm, scale; chunks that keep the [n,D,L] temporary under 1 GiB).  Second figure ("port"): the scalar C
+    restatement of the same algorithm (oracle/tq_oracle.c, OpenMP over vectors)."""
     import numpy as np
+    import torch
     from oracle import tq_oracle as O
 
-    threads = O.COracle.threads()
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
     rng = np.random.default_rng(0)
-    per_width = {}
-    sample_desc = []
+    make = lambda n: rng.standard_normal((n, 128), dtype=np.float32)
+    seq, port, seq_desc, port_desc = {}, {}, [], []
     for bits, share in sorted(widths.items()):
         comp = pkg.MSECompressor(128, bits, seed=42, device="cpu")
-        orc = O.COracle(comp.Pi.numpy(), comp.centroids.numpy(), bits, accum_double=False)
-        n = 4096
-        x = rng.standard_normal((n, 128), dtype=np.float32)
-        t0 = time.perf_counter()
-        out = orc.compress(x, want_rotated=False)
-        orc.decompress(out["idx_bytes"], out["vec_norms"])
-        probe = time.perf_counter() - t0
-        target = budget_s * share
-        n = int(min(max(n * target / max(probe, 1e-6), 8192), 4_000_000))
-        x = rng.standard_normal((n, 128), dtype=np.float32)
-        t0 = time.perf_counter()
-        out = orc.compress(x, want_rotated=False)
-        orc.decompress(out["idx_bytes"], out["vec_norms"])
-        dt = time.perf_counter() - t0
-        per_width[bits] = n / dt
-        sample_desc.append(f"{n} x {bits}-bit")
+        pi, cent = comp.Pi.numpy(), comp.centroids.numpy()
+        tor = O.TorchCpuOracle(pi, cent, bits)
+
+        def run_seq(x):
+            b, n = tor.compress(torch.from_numpy(x))
+            tor.decompress(b, n)
+        seq[bits], n = _timed_sample(run_seq, make, share, 0.65 * budget_s, probe_n=min(2048, tor.chunk))
+        seq_desc.append(f"{n} x {bits}-bit (chunks of {tor.chunk})")
+        orc = O.COracle(pi, cent, bits, accum_double=False)
+
+        def run_port(x):
+            out = orc.compress(x, want_rotated=False)
+            orc.decompress(out["idx_bytes"], out["vec_norms"])
+        port[bits], n = _timed_sample(run_port, make, share, 0.35 * budget_s, probe_n=4096)
+        port_desc.append(f"{n} x {bits}-bit")
     # harmonic mix: time per vector of the workload = sum share_b / rate_b
-    rate = 1.0 / sum(share / per_width[b] for b, share in widths.items())
+    mix = lambda rates: 1.0 / sum(share / rates[b] for b, share in widths.items())
     return {
-        "value": rate, "unit": "vectors/s", "cores": threads, "kind": "port",
-        "sample": "compress+decompress of " + ", ".join(sample_desc) + " random fp32 vectors, mixed in the workload's width shares",
-        "per_width_vectors_per_s": {str(b): r for b, r in per_width.items()},
-        "cpu": platform.processor() or platform.machine(),
+        "value": mix(seq), "unit": "vectors/s", "cores": cores, "kind": "op-sequence",
+        "sample": "compress+decompress of " + ", ".join(seq_desc) + " random fp32 vectors through torch CPU operators "
+                  "(the reference's op sequence, compressors_v3.py:46-105), mixed in the workload's width shares",
+        "per_width_vectors_per_s": {str(b): r for b, r in seq.items()},
+        "cpu": cpu_model(), "torch": torch.__version__, "torch_threads": torch.get_num_threads(),
+        "port": {"value": mix(port), "unit": "vectors/s", "cores": O.COracle.threads(), "kind": "port",
+                 "sample": "the same on " + ", ".join(port_desc) + " vectors through the scalar C restatement (oracle/tq_oracle.c, OpenMP)",
+                 "per_width_vectors_per_s": {str(b): r for b, r in port.items()}},
     }
 
 
@@ -170,7 +207,9 @@ def run_decode(args, torch, pkg, w, dev):
                                  + (algorithmic_bytes(w["key_bits"], 2, "c") + algorithmic_bytes(w["value_bits"], 2, "c"))
                                  + 2 * rw * 256)
     result = {
-        "metric": "KV vectors/sec (compress+decompress)", "value": (deq_vec + cmp_vec) / sec, "unit": "vectors/s",
+        "metric": ("KV vectors/sec (compressed on append + attended from packed codes)" if attend
+                   else "KV vectors/sec (compress+decompress)"),
+        "value": (deq_vec + cmp_vec) / sec, "unit": "vectors/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, "layers": L, "batch": B, "kv_heads": H, "compressed_tokens": n_c,
@@ -300,21 +339,35 @@ def main():
         bytes_per_launch = jobs * n_vec * algorithmic_bytes(b, elem, direction)
         avg_ms = sum(e0.elapsed_time(e1) for e0, e1 in evs) / len(evs)
         step_bytes += bytes_per_launch
+        flop = jobs * n_vec * ROTATION_FLOP * MFMA_PASSES[direction]
         kernels[f"{direction}_b{b}"] = {
             "launches_per_step": 1, "jobs": jobs, "vectors_per_launch": jobs * n_vec,
             "algorithmic_bytes_per_launch": bytes_per_launch, "avg_ms": avg_ms,
             "achieved_GBps": bytes_per_launch / avg_ms / 1e6,
             "frac_of_hbm_peak": bytes_per_launch / avg_ms / 1e6 / HBM_PEAK_GBS,
+            "mfma_flop_per_launch": flop, "mfma_PFLOPs": flop / avg_ms / 1e12,
+            "frac_of_mfma_peak": flop / avg_ms / 1e12 / MFMA_PEAK_PFLOPS,
         }
     dominant = max(kernels, key=lambda k: kernels[k]["avg_ms"])
     dk = kernels[dominant]
-    traffic = None
+    # HBM bytes per launch of the dominant kernel as the counters saw them (FETCH_SIZE + WRITE_SIZE, calibrated against
+    # a copy kernel): a number from the committed profile run of this workload, not measured by this process
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         try:
             traffic = json.load(open(tpath)).get(args.workload, {}).get(dominant)
+            traffic_source = "profiles/hbm_traffic.json (rocprofv3 --pmc run of this workload, committed)" if traffic else None
         except Exception:
             traffic = None
+
+    def mfma_of(direction):
+        """the rotation's matrix-core rate in the slowest launch of one direction"""
+        name = max((k for k in kernels if k.startswith(direction)), key=lambda k: kernels[k]["avg_ms"])
+        k = kernels[name]
+        return {"kernel": name, "flop_per_vector": ROTATION_FLOP * MFMA_PASSES[direction],
+                "flop_per_launch": k["mfma_flop_per_launch"], "achieved": k["mfma_PFLOPs"], "peak": MFMA_PEAK_PFLOPS,
+                "unit": "PFLOP/s", "frac": k["frac_of_mfma_peak"]}
 
     widths = {}
     for b, jobs in groups.items():
@@ -336,7 +389,8 @@ def main():
         "step_GBps": step_bytes / (wall / args.steps) / 1e9,
         "step_frac_of_hbm_peak": step_bytes / (wall / args.steps) / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dk["achieved_GBps"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": dk["frac_of_hbm_peak"], "traffic": traffic},
+                     "unit": "GB/s", "frac": dk["frac_of_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source,
+                     "mfma": {"compress": mfma_of("compress"), "decompress": mfma_of("decompress")}},
         "kernels": kernels,
         "round_trip_rel_error": rel,
     }

@@ -82,6 +82,14 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
                    void *table_host, size_t table_bytes);
 
 /*
+ * Checks a table blob in host memory against the (head_dim, bits) it is about to be used with: TQ_OK, or
+ * TQ_ERR_TABLE (bad magic / version / size, or built for another head_dim or another bit width).  The launch
+ * entry points cannot make this check (the blob they get is in device memory and `bits` selects the kernel):
+ * a binding keeps `bits` next to every table pointer and calls this once per table, before the first launch.
+ */
+int tq_table_check(const void *table_host, size_t table_bytes, int head_dim, int bits);
+
+/*
  * Host emulation of the kernels' quantiser lookup, bit for bit (same fused multiply-add,
  * same grid): idx[i] = code chosen for unit-sphere coordinate r[i].  For tests of the
  * table contents; the product path never calls it.

@@ -9,8 +9,11 @@ upstream algorithm live here and check each other:
     integer pack; unpack, gather, product, scale), chunked over N.
     Follows turboquant/compressors_v3.py:46-81 (compress) and :84-105 (decompress).
   * `COracle`      -- ctypes front end of oracle/tq_oracle.c (scalar loops, OpenMP
-    over vectors): fast enough for the large parity tests and the timed CPU
-    baseline of the benchmark.
+    over vectors): fast enough for the large parity tests; the benchmark times it as a second CPU figure.
+  * `TorchCpuOracle` -- the same op sequence issued as torch CPU operators (the reference's own
+    library calls: fp32 cast, torch.norm, divide, sgemm, [n,D,L] broadcast / abs / argmin, int64
+    pack; unpack, gather, sgemm, scale), chunked over N so that the [n,D,L] temporary stays under
+    1 GiB.  This is what the benchmark times as "the reference's CPU path" on the host cores.
 
 Only tests/, the repository's smoke check and the benchmark's cpu_baseline leg
 may import this module; the shipped package never does.
@@ -145,6 +148,69 @@ class NumpyOracle:
         n = vec_norms_bits.reshape(-1, 1).view(np.float16).astype(np.float32)
         with np.errstate(invalid="ignore", over="ignore"):
             return (y @ self.Pi) * n
+
+
+# --------------------------------------------------------------------------
+# torch CPU restatement (the timed "reference CPU path")
+# --------------------------------------------------------------------------
+class TorchCpuOracle:
+    """MSECompressor.compress / decompress of turboquant/compressors_v3.py as torch CPU operators, on chunks of
+    `chunk` vectors (default: the largest power of two that keeps the [chunk, D, 2^bits] float32 intermediate of
+    :60-61 under 1 GiB; unchunked, one 8-bit layer of 262 144 vectors would need 34 GB)."""
+
+    def __init__(self, Pi: np.ndarray, centroids: np.ndarray, bits: int, chunk: int = 0):
+        import torch
+        self.torch = torch
+        self.Pi = torch.from_numpy(np.ascontiguousarray(Pi, dtype=np.float32))
+        self.centroids = torch.from_numpy(np.ascontiguousarray(centroids, dtype=np.float32))
+        self.bits = int(bits)
+        self.D = self.Pi.shape[0]
+        if not chunk:
+            chunk = 1
+            while chunk * 2 * self.D * (1 << self.bits) * 4 < (1 << 30):
+                chunk *= 2
+        self.chunk = chunk
+        ipb = indices_per_byte(self.bits)
+        self.ipb = ipb
+        self.pad = (ipb - self.D % ipb) % ipb                                                    # :65
+        self.weights = torch.tensor([2 ** (self.bits * i) for i in range(ipb - 1, -1, -1)], dtype=torch.long)   # :70-73
+        self.shifts = torch.tensor([self.bits * i for i in range(ipb - 1, -1, -1)], dtype=torch.long)           # :95-98
+
+    def compress(self, x):
+        """x: torch CPU tensor or array [..., D], any float type -> (idx_bytes u8 [N,G], vec_norms fp16 [N]) as torch tensors"""
+        torch = self.torch
+        x = torch.as_tensor(x).reshape(-1, self.D)
+        out_b, out_n = [], []
+        with torch.no_grad():
+            for s in range(0, x.shape[0], self.chunk):
+                flat = x[s:s + self.chunk].float()                                        # :52
+                norms = torch.norm(flat, dim=-1)                                           # :55
+                unit = flat / (norms.unsqueeze(-1) + 1e-8)                                 # :56
+                rotated = unit @ self.Pi.T                                                 # :59
+                codes = (rotated.unsqueeze(-1) - self.centroids).abs().argmin(dim=-1).to(torch.uint8)   # :60-61
+                wide = codes.long()                                                        # :66
+                if self.pad:
+                    wide = torch.nn.functional.pad(wide, (0, self.pad))                    # :67-68
+                groups = wide.shape[-1] // self.ipb
+                out_b.append((wide.reshape(-1, groups, self.ipb) * self.weights).sum(-1).to(torch.uint8))  # :74
+                out_n.append(norms.to(torch.float16))                                      # :78
+        return torch.cat(out_b), torch.cat(out_n)
+
+    def decompress(self, idx_bytes, vec_norms):
+        """-> float32 [N, D] torch tensor (:84-105)"""
+        torch = self.torch
+        idx_bytes = torch.as_tensor(idx_bytes).reshape(-1, bytes_per_vector(self.D, self.bits))
+        vec_norms = torch.as_tensor(vec_norms).reshape(-1, 1)
+        mask = (1 << self.bits) - 1
+        out = []
+        with torch.no_grad():
+            for s in range(0, idx_bytes.shape[0], self.chunk):
+                b = idx_bytes[s:s + self.chunk]
+                codes = ((b.long().unsqueeze(-1) >> self.shifts) & mask).reshape(b.shape[0], -1)   # :99
+                if self.pad:
+                    codes = codes[:, :self.D]                                                     # :100-101
+                out.append((self.centroids[codes] @ self.Pi) * vec_norms[s:s + self.chunk].float())   # :104
+        return torch.cat(out)
 
 
 # --------------------------------------------------------------------------

@@ -117,6 +117,65 @@ def test_v3cache_stream_equals_one_shot_codec(pkg, oracle, rw, dtype):
     assert cache.stored_bytes() == L * B * H * (n_c * (64 + 32 + 4) + 2 * (total - n_c) * D * 2)
 
 
+def test_config5_shape_decode_streaming(pkg, oracle):
+    """The decode-streaming workload at its real shape, one layer: 64 sequences x 8 KV heads, 16 384 compressed +
+    128 window tokens prefilled (bf16, K4/V2, residual_window=128), then three single-token decode steps.
+    Everything is checked on all 512 rows against the one-shot codec on the device (bit for bit), and on a sample
+    of rows (first and last sequence) against the CPU oracle: stored codes and norms, the de-quantised history
+    `update` returns, and `attend` against float64 attention over the oracle-decoded cache."""
+    B, H, D, S0, rw, G = 64, 8, 128, 16384, 128, 4
+    from test_gpu_parity import _device_kv, check_codes, check_norms
+    cache = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=rw, protected_layers=0, n_layers=32, capacity=S0 + 16)
+    total = S0 + rw + 3
+    keys = _device_kv((B, H, total, D), 5_000_000, torch.bfloat16)
+    vals = _device_kv((B, H, total, D), 5_000_001, torch.bfloat16)
+    layer = 0
+    fk, fv = cache.update(keys[:, :, :S0 + rw], vals[:, :, :S0 + rw], layer)
+    assert fk.shape == (B, H, S0 + rw, D) and cache.get_compression_info() == f"{S0} compressed, {rw} fp16, {S0 + rw} total"
+    del fk, fv
+    for t in range(S0 + rw, total):
+        fk, fv = cache.update(keys[:, :, t:t + 1], vals[:, :, t:t + 1], layer)
+        if t + 1 < total:
+            del fk, fv
+    n_c = total - rw
+    st = cache._stores[layer]
+    assert cache.get_seq_length(layer) == total and st.n_compressed == n_c == S0 + 3
+    assert fk.shape == (B, H, total, D) and fk.dtype == torch.bfloat16
+    # all rows: the window verbatim, the history equal to the one-shot codec over the same tokens
+    assert torch.equal(fk[:, :, n_c:], keys[:, :, n_c:]) and torch.equal(fv[:, :, n_c:], vals[:, :, n_c:])
+    tq = cache._get_compressor(layer, D, DEV)
+    ck, cv = tq.compress_kv(keys[:, :, :n_c], vals[:, :, :n_c])
+    assert torch.equal(st.k_idx[:, :, :n_c], ck["compressed"]["idx_bytes"]) and torch.equal(st.k_nrm[:, :, :n_c], ck["compressed"]["vec_norms"])
+    assert torch.equal(st.v_idx[:, :, :n_c], cv["compressed"]["idx_bytes"]) and torch.equal(st.v_nrm[:, :, :n_c], cv["compressed"]["vec_norms"])
+    dk, dv = tq.decompress_kv(ck, cv)
+    assert torch.equal(fk[:, :, :n_c], dk) and torch.equal(fv[:, :, :n_c], dv)
+    del dk, dv, ck, cv
+    # the query step on all rows; sampled sequences against the oracle
+    q = _device_kv((B, H * G, 1, D), 5_000_003, torch.bfloat16) * 0.05
+    out = cache.attend(q, layer)
+    assert out.shape == q.shape and bool(torch.isfinite(out.float()).all())
+    for b in (0, B - 1):
+        dec = {}
+        for comp, idx, nrm, x, full, name in ((tq.key_compressor, st.k_idx, st.k_nrm, keys, fk, "K4"),
+                                              (tq.val_compressor, st.v_idx, st.v_nrm, vals, fv, "V2")):
+            Pi, cent = comp.Pi.cpu().numpy(), comp.centroids.cpu().numpy()
+            flat = x[b, :, :n_c].float().cpu().numpy().reshape(-1, D)
+            ref, _ = check_codes(oracle, idx[b, :, :n_c].contiguous().cpu().numpy(), flat, Pi, cent, comp.bits, f"config 5 seq {b} {name}")
+            check_norms(oracle, bits16(nrm[b, :, :n_c].contiguous()), ref["vec_norms"], f"config 5 seq {b} {name}")
+            orc = oracle.COracle(Pi, cent, comp.bits, True)
+            stored = orc.decompress(idx[b, :, :n_c].contiguous().cpu().numpy().reshape(-1, idx.shape[-1]),
+                                    bits16(nrm[b, :, :n_c].contiguous()).reshape(-1))
+            err, _ = rel_l2(full[b, :, :n_c].float().cpu().numpy().reshape(-1, D), stored)
+            assert err < 4e-3, (name, err)                 # bf16 output rounding on top of the 1e-3 bar
+            dec[name] = np.concatenate([stored.reshape(H, n_c, D), x[b, :, n_c:].float().cpu().numpy()], axis=1)
+        _, want = oracle.attention_decode(q[b:b + 1, :, 0].float().cpu().numpy(), dec["K4"][None], dec["V2"][None], D ** -0.5)
+        got = out[b, :, 0].float().cpu().numpy()
+        err = float(np.linalg.norm(got - want[0]) / np.linalg.norm(want[0]))
+        print(f"[config 5] seq {b}: attend vs float64 attention over the oracle-decoded cache: {err:.2e}")
+        assert err < 6e-3, err                             # bf16 output rounding of `attend`
+    assert cache.stored_bytes() == B * H * (n_c * (64 + 32 + 4) + 2 * rw * D * 2)
+
+
 def test_v3cache_grows_and_protects_layers(pkg):
     """Capacity doubles without losing history; protected layers store 8-bit codes for K and V."""
     cache = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=8, protected_layers=1, n_layers=3)
@@ -489,7 +548,23 @@ def test_hf_model_decodes_through_packed_attention(pkg):
         cache = cls(key_bits=4, value_bits=2, residual_window=16, n_layers=3, packed_attention=True)
         gen = model.generate(ids, attention_mask=torch.ones_like(ids), past_key_values=cache, max_new_tokens=10, do_sample=False)
         assert gen.shape == (2, 80) and cache.get_seq_length() == 79
+        # a padded batch is refused in that mode: attention from the packed store counts every cached token
+        cache = cls(key_bits=4, value_bits=2, residual_window=16, n_layers=3, packed_attention=True)
+        mask = torch.ones_like(ids)
+        model(ids, attention_mask=mask, past_key_values=cache, use_cache=True)
+        mask = torch.cat([mask, torch.ones_like(steps[0])], dim=1)
+        mask[1, :3] = 0
+        with pytest.raises(RuntimeError, match="hides cached tokens"):
+            model(steps[0], attention_mask=mask, past_key_values=cache, use_cache=True)
+        # a cache in packed mode under a model whose attention is not the registered function: the step of layer 0
+        # would be attention over one token; the next call on the cache says so instead
         model.config._attn_implementation = "sdpa"
+        cache = cls(key_bits=4, value_bits=2, residual_window=16, n_layers=3, packed_attention=True)
+        mask = torch.ones_like(ids)
+        model(ids, attention_mask=mask, past_key_values=cache, use_cache=True)
+        mask = torch.cat([mask, torch.ones_like(steps[0])], dim=1)
+        with pytest.raises(RuntimeError, match="never answered"):
+            model(steps[0], attention_mask=mask, past_key_values=cache, use_cache=True)
 
 
 def test_fused_attention_over_extreme_value_norms(pkg, oracle):

@@ -561,6 +561,79 @@ def test_config3_shape_k6v4_window(pkg, oracle):
     assert mem["compressed_bytes"] == B * H * (3968 * (128 + 2 + 64 + 2) + 128 * D * 2 * 2)
 
 
+def _device_kv(shape, seed, dtype):
+    """N(0,1) x per-channel log-normal x per-token U[0.5, 2], generated on the device (the benchmark's recipe)."""
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    x = torch.randn(shape, generator=g, device=DEV, dtype=torch.float32)
+    ch = torch.exp(torch.randn(shape[-1], generator=g, device=DEV))
+    tok = 0.5 + 1.5 * torch.rand(shape[:-1] + (1,), generator=g, device=DEV)
+    return (x * ch * tok).to(dtype)
+
+
+def test_config4_shape_llama_32k(pkg, oracle):
+    """One layer of the Llama-3-8B-shaped cache at its real shape, [1,8,32768,128] bf16 with the per-token norm
+    spread, through TurboQuantV3 with the reference's protected-layer rule (n_layers=32, protected_layers=4):
+    layer 0 is protected (K8/V8), layer 16 is K4/V2.  262 144 vectors per tensor: codes and norms against the
+    oracle, the reconstruction against the oracle's decode within bf16 output rounding."""
+    shape = (1, 8, 32768, 128)
+    for layer, (kb, vb) in ((0, (8, 8)), (16, (4, 2))):
+        tq = pkg.TurboQuantV3(128, key_bits=4, value_bits=2, residual_window=0, layer_idx=layer, n_layers=32,
+                              protected_layers=4, device=DEV)
+        assert (tq.key_bits, tq.value_bits) == (kb, vb)
+        keys = outlier_kv(shape, seed=4_000_000 + 10 * layer, dtype=torch.bfloat16)
+        vals = outlier_kv(shape, seed=4_000_001 + 10 * layer, dtype=torch.bfloat16)
+        ck, cv = tq.compress_kv(keys.to(DEV), vals.to(DEV))
+        assert ck["split_at"] == 32768 and ck["fp16"].shape[2] == 0
+        rk, rv = tq.decompress_kv(ck, cv)
+        for c, x, comp, rec, name in ((ck, keys, tq.key_compressor, rk, f"K{kb}"), (cv, vals, tq.val_compressor, rv, f"V{vb}")):
+            Pi, cent = comp.Pi.cpu().numpy(), comp.centroids.cpu().numpy()
+            # bf16 inputs meet the rotation as two bf16 terms (2^-17): a few hundred coordinates per million sit
+            # within 1e-6 of a boundary at 8 bits, where boundaries are densest; all inside the 1e-5 window
+            ref, _ = check_codes(oracle, c["compressed"]["idx_bytes"].cpu().numpy(), x.float().numpy().reshape(-1, 128), Pi, cent,
+                                 comp.bits, f"config 4 layer {layer} {name}", max_frac=6e-4 if comp.bits == 8 else 2e-4)
+            check_norms(oracle, bits16(c["compressed"]["vec_norms"]), ref["vec_norms"], f"config 4 layer {layer} {name}")
+            want = oracle.COracle(Pi, cent, comp.bits, True).decompress(ref["idx_bytes"], ref["vec_norms"])
+            err, _ = rel_l2(rec.float().cpu().numpy().reshape(-1, 128), want)
+            assert rec.dtype == torch.bfloat16 and err < 4e-3, (name, err)   # bf16 output rounding (2^-9) on top of 1e-3
+        mem = tq.memory_bytes(*shape[:3])
+        assert mem["compressed_bytes"] == 8 * 32768 * ((128 if kb == 8 else 64) + 2 + (128 if vb == 8 else 32) + 2)
+
+
+def test_config4_batched_launches_equal_per_layer_calls(pkg):
+    """The launches the benchmark times: all 32 layers of the Llama-3-8B-shaped cache (K and V, [1,8,32768,128]
+    bf16 each) as three compress and three decompress launches grouped by width (24 K4 jobs, 24 V2 jobs, 16
+    eight-bit jobs of the 8 protected layers).  Every job's packed bytes, norms and de-quantised tensor equal,
+    bit for bit, what a call on that tensor alone produces."""
+    native = pkg._native
+    L, shape = 32, (1, 8, 32768, 128)
+    groups = {}
+    for l in range(L):
+        tq = pkg.TurboQuantV3(128, key_bits=4, value_bits=2, residual_window=0, layer_idx=l, n_layers=L,
+                              protected_layers=4, device=DEV)
+        for which, comp in ((0, tq.key_compressor), (1, tq.val_compressor)):
+            G = 128 // (8 // comp.bits)
+            groups.setdefault(comp.bits, []).append({
+                "comp": comp, "states": _device_kv(shape, 4_100_000 + 10 * l + which, torch.bfloat16),
+                "idx_bytes": torch.zeros(shape[:3] + (G,), dtype=torch.uint8, device=DEV),
+                "vec_norms": torch.zeros(shape[:3], dtype=torch.float16, device=DEV),
+                "out": torch.zeros(shape, dtype=torch.bfloat16, device=DEV), "table": comp.table(), "bits": comp.bits})
+    assert {b: len(j) for b, j in groups.items()} == {8: 16, 4: 24, 2: 24}
+    for b, jobs in groups.items():
+        native.JobList(jobs, DEV).compress()
+    for b, jobs in groups.items():
+        native.JobList([dict(j, states=j["out"]) for j in jobs], DEV).decompress()
+    torch.cuda.synchronize()
+    for b, jobs in groups.items():
+        for j in jobs:
+            one = j["comp"].compress(j["states"])
+            assert torch.equal(one["idx_bytes"], j["idx_bytes"]) and torch.equal(one["vec_norms"], j["vec_norms"]), b
+            alone = torch.empty_like(j["out"])
+            j["comp"].decompress_into(one, alone)
+            assert torch.equal(alone, j["out"]), b
+            del one, alone
+
+
 def test_operators_trace_under_a_compiler(pkg):
     """The registered operators carry schemas and fake implementations: `torch.library.opcheck` accepts them, and a
     compiled function (aot_eager backend: traced with fake tensors, executed with the real kernels) that goes
@@ -573,6 +646,16 @@ def test_operators_trace_under_a_compiler(pkg):
     idx, nrm = torch.ops.tqamd.compress(x, table, 4)
     torch.library.opcheck(torch.ops.tqamd.decompress.default, (idx, nrm, table, 4, 128, torch.bfloat16),
                           test_utils=("test_schema", "test_faketensor"))
+
+    # the one-pass attention operator: its fake implementation has to predict the split count of the real one
+    kc = pkg.MSECompressor(128, 4, seed=6, device=DEV)
+    vc = pkg.MSECompressor(128, 2, seed=7, device=DEV)
+    kv = outlier_kv((2, 2, 3000, 128), seed=92, dtype=torch.bfloat16).to(DEV)
+    pk, pv = kc.compress(kv), vc.compress(kv)
+    q_rot = torch.randn(2, 8, 128, device=DEV)
+    args = (pk["idx_bytes"], pk["vec_norms"], pv["idx_bytes"], pv["vec_norms"], kc.table(), vc.table(), 4, 2, q_rot)
+    torch.library.opcheck(torch.ops.tqamd.attend_partials.default, args, test_utils=("test_schema", "test_faketensor"))
+    assert torch.ops.tqamd.attend_partials(*args).shape[2] == pkg._native.lib().tq_attend_splits(4, 3000) > 1
 
     def round_trip(t):
         c = comp.compress(t)

@@ -243,6 +243,46 @@ def test_passthrough_and_errors_without_gpu(pkg):
         wide.compress(torch.randn(1, 1, 4, 128))
 
 
+def test_table_and_width_must_agree(pkg):
+    """A table blob is checked against the (head_dim, bits) it is used with before anything is launched: by
+    tq_table_check on the host copy, and by the registry of uploaded tables at every launch of this package."""
+    native = pkg._native
+    lib = native.lib()
+    pi = pkg.generate_rotation_matrix(128, seed=3)
+    blob = native.build_table(pi, pkg.LloydMaxCodebook(128, 4).centroids, 4)
+    assert lib.tq_table_check(blob.ctypes.data, blob.size, 128, 4) == 0
+    assert lib.tq_table_check(blob.ctypes.data, blob.size, 128, 2) == -7          # built for another width
+    assert lib.tq_table_check(blob.ctypes.data, blob.size, 64, 4) == -7
+    assert lib.tq_table_check(blob.ctypes.data, blob.size - 1, 128, 4) == -7      # truncated
+    assert lib.tq_table_check(blob.ctypes.data, blob.size, 128, 9) == -2
+    broken = blob.copy()
+    broken[0] ^= 0xFF
+    assert lib.tq_table_check(broken.ctypes.data, broken.size, 128, 4) == -7
+    assert lib.tq_table_check(None, 0, 128, 4) == -1
+    # the launch-side check: a tensor registered as a 4-bit table cannot be launched as a 2-bit one
+    fake = torch.zeros(16, dtype=torch.uint8)
+    native._table_widths[fake.data_ptr()] = (128, 4)
+    try:
+        native.check_table(fake, 128, 4)
+        with pytest.raises(native.TqError, match="4 bits used with head_dim 128, 2 bits"):
+            native.check_table(fake, 128, 2)
+        native.check_table(torch.zeros(16, dtype=torch.uint8), 128, 2)             # unknown tables pass
+    finally:
+        del native._table_widths[fake.data_ptr()]
+
+
+def test_workspace_is_dropped_after_a_failed_call(pkg):
+    """The ticket counters kept per (device, stream) are only trusted while every call on them succeeded."""
+    native = pkg._native
+    dev = torch.device("cuda:0")
+    native._workspaces[(0, 12345)] = torch.zeros(1)
+    native._workspaces[(0, 777)] = torch.zeros(1)
+    native._drop_workspace(dev, 12345)
+    assert (0, 12345) not in native._workspaces and (0, 777) in native._workspaces
+    native._drop_workspace(dev, 12345)                                             # nothing to drop: fine
+    del native._workspaces[(0, 777)]
+
+
 def test_c_abi_argument_errors(pkg):
     lib = pkg._native.lib()
     E = {k: v for k, v in (("NULL", -1), ("BITS", -2), ("HEAD_DIM", -3), ("DTYPE", -4), ("SIZE", -5),

@@ -40,6 +40,36 @@ def test_roundtrip_fixtures_numpy_bit_exact(golden, oracle):
     assert n == 20
 
 
+def test_roundtrip_fixtures_torch_cpu_op_sequence(golden, oracle):
+    """The torch CPU op sequence that the benchmark times as the reference's CPU path: the reference's bytes and
+    norms on every fixture (a tiny chunk size, so that the chunk loop is what is tested), fp32 reconstruction to
+    rounding (sgemm blocks its sums by the row count, so the last bits move with the chunk size)."""
+    fx = golden["mse_roundtrip"]
+    for b, dn in _cases(golden):
+        cent = fx[f"centroids_b{b}"]
+        x = torch.from_numpy(oracle.widen(fx[f"b{b}_{dn}_x"], dn))
+        ref_bytes = fx[f"b{b}_{dn}_idx_bytes"]
+        ref_bytes = ref_bytes.reshape(-1, ref_bytes.shape[-1])
+        ref_norms = fx[f"b{b}_{dn}_vec_norms"].reshape(-1)
+        for chunk in (0, 7):
+            orc = oracle.TorchCpuOracle(fx[f"Pi_b{b}"], cent, b, chunk=chunk)
+            with np.errstate(over="ignore", invalid="ignore"):
+                got_b, got_n = orc.compress(x)
+            got_b = got_b.numpy()
+            if not np.array_equal(got_b, ref_bytes):      # only a coordinate on a decision boundary may move
+                rot = oracle.NumpyOracle(fx[f"Pi_b{b}"], cent, b).rotate(x.numpy())[1]
+                rep = oracle.code_mismatch_report(got_b, ref_bytes, rot, cent, b)
+                assert rep["outside_window"] == 0 and rep["differ"] <= 2, (b, dn, chunk, rep)
+            assert oracle.fp16_ulp_distance(got_n.view(torch.int16).numpy().view(np.uint16), ref_norms).max() <= 1
+            rec = orc.decompress(torch.from_numpy(ref_bytes), torch.from_numpy(ref_norms.view(np.float16))).numpy()
+            ref = fx[f"b{b}_{dn}_recon"].reshape(-1, 128)
+            fin = np.isfinite(ref).all(-1)
+            assert np.array_equal(np.isfinite(rec).all(-1), fin)
+            assert np.abs(rec[fin] - ref[fin]).max() <= 1e-5 * max(1.0, np.abs(ref[fin]).max())
+    assert oracle.TorchCpuOracle(fx["Pi_b8"], fx["centroids_b8"], 8).chunk == 4096       # 4096 x 128 x 256 x 4 B = 512 MiB
+    assert oracle.TorchCpuOracle(fx["Pi_b2"], fx["centroids_b2"], 2).chunk == 262144
+
+
 @pytest.mark.parametrize("accum_double", [False, True])
 def test_roundtrip_fixtures_c(golden, oracle, accum_double):
     """The scalar C restatement: same codes except inside the 1e-5 boundary window (none seen),

@@ -86,7 +86,7 @@ class TqJob(ctypes.Structure):
 
 EXPORTS = (
     "tq_abi_version", "tq_status_string", "tq_device_count", "tq_bytes_per_vector",
-    "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_quantize_host",
+    "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_check", "tq_table_quantize_host",
     "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched", "tq_workspace_bytes",
     "tq_decompress_batched_noalloc",
     "tq_scores", "tq_weighted_values", "tq_weighted_values_splits", "tq_attend_partials", "tq_attend_splits",
@@ -116,6 +116,7 @@ def lib() -> ctypes.CDLL:
     L.tq_table_bytes.restype = ll
     L.tq_table_bytes.argtypes = [ci, ci]
     L.tq_table_build.argtypes = [vp, vp, ci, ci, vp, ctypes.c_size_t]
+    L.tq_table_check.argtypes = [vp, ctypes.c_size_t, ci, ci]
     L.tq_table_quantize_host.argtypes = [vp, vp, ll, vp]
     L.tq_compress.argtypes = [vp, ci, ll, ll, ll, ll, vp, ci, ci, vp, vp, ll, vp]
     L.tq_decompress.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, ll, ll, vp, vp]
@@ -172,6 +173,28 @@ def build_table(Pi: torch.Tensor, centroids: torch.Tensor, bits: int) -> np.ndar
     blob = np.zeros(nbytes, dtype=np.uint8)
     check(lib().tq_table_build(pi.ctypes.data, cent.ctypes.data, d, bits, blob.ctypes.data, blob.size), "tq_table_build")
     return blob
+
+
+# The launch entry points take a table in device memory and a bit width that selects the kernel; nothing on the
+# device side can tell them apart when they disagree (the codes would be garbage, silently).  Every table this
+# module uploads is therefore remembered with the width it was built for, and every launch checks its pair.
+_table_widths: Dict[int, Tuple[int, int]] = {}     # device address of an uploaded table -> (head_dim, bits)
+
+
+def upload_table(blob: np.ndarray, head_dim: int, bits: int, device: torch.device) -> torch.Tensor:
+    """Device copy of a blob from build_table, after tq_table_check(blob, head_dim, bits)."""
+    check(lib().tq_table_check(blob.ctypes.data, blob.size, head_dim, bits), "tq_table_check")
+    t = torch.from_numpy(blob).to(device)
+    _table_widths[t.data_ptr()] = (head_dim, bits)
+    return t
+
+
+def check_table(table: torch.Tensor, head_dim: int, bits: int) -> None:
+    """Raises if `table` was uploaded for another (head_dim, bits).  Tables this module never saw (a caller's own
+    upload) pass: their owner has to make the check, with tq_table_check on the host copy."""
+    known = _table_widths.get(table.data_ptr())
+    if known is not None and known != (head_dim, 8 if bits > 8 else bits):
+        raise TqError(f"codec table built for head_dim {known[0]}, {known[1]} bits used with head_dim {head_dim}, {bits} bits")
 
 
 def quantize_host(table: np.ndarray, r: np.ndarray) -> np.ndarray:
@@ -311,19 +334,26 @@ def _workspace(device: torch.device, stream: int) -> int:
     return ws.data_ptr()
 
 
+def _drop_workspace(device: torch.device, stream: int) -> None:
+    """Forget the counters kept for (device, stream) after a call that reported an error: the contract "zero before,
+    zero after" only holds for launches that complete, so the next call gets fresh zeroed counters."""
+    _workspaces.pop((device.index if device.index is not None else torch.cuda.current_device(), stream), None)
+
+
 _step_scratch: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
 def step_scratch(device: torch.device, stream: int, floats: int) -> Optional[torch.Tensor]:
     """float32 scratch of a decode step (rotated queries, window record, split records), one buffer per
-    (device, stream), grown on demand: the steps of all layers on a stream run one after the other.
-    None when it would have to be allocated while a graph is being captured (the memory would belong to
-    the graph's pool, not to this table)."""
+    (device, stream), grown on demand: the steps of all layers on a stream run one after the other.  One entry per
+    stream that ever ran a decode step, kept for the life of the process (a few hundred KiB each).
+    None while a graph is being captured: the caller then takes the general path, whose scratch comes from the
+    graph's own memory pool."""
+    if torch.cuda.is_current_stream_capturing():
+        return None      # a captured step may be replayed on any stream, next to eager steps that use this buffer
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     buf = _step_scratch.get(key)
     if buf is None or buf.numel() < floats:
-        if torch.cuda.is_current_stream_capturing():
-            return None
         buf = _step_scratch[key] = torch.empty(max(floats, 1 << 16), dtype=torch.float32, device=device)
     return buf
 
@@ -342,6 +372,7 @@ def compress_into(states: torch.Tensor, table: torch.Tensor, bits: int,
         states = states.contiguous()
         lay = row_layout(states) if prs else vector_layout(states)
     rows, tokens, row_stride, token_stride = lay
+    check_table(table, states.shape[-1], bits)
     with _on(states.device):
         rc = lib().tq_compress(states.data_ptr(), dtype_code(states.dtype), rows, tokens, row_stride, token_stride,
                                table.data_ptr(), states.shape[-1], bits,
@@ -363,11 +394,14 @@ def decompress_into(idx_bytes: torch.Tensor, vec_norms: torch.Tensor, table: tor
         raise TqError("decompress output must have a dense last dimension, 16-byte aligned rows and at most "
                       "two stride levels")
     rows, tokens, row_stride, token_stride = lay
+    check_table(table, out.shape[-1], bits)
     with _on(out.device):
         stream = _stream_handle(out.device)
         rc = lib().tq_decompress(idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, rows, tokens, table.data_ptr(),
                                  out.shape[-1], bits, out.data_ptr(), dtype_code(out.dtype), row_stride,
                                  token_stride, _workspace(out.device, stream), stream)
+    if rc:
+        _drop_workspace(out.device, stream)
     check(rc, "tq_decompress")
 
 
@@ -549,7 +583,10 @@ attend_partials_op = torch.library.custom_op("tqamd::attend_partials", _attend_p
 
 @attend_partials_op.register_fake
 def _(k_idx, k_norms, v_idx, v_norms, table_k, table_v, bits_k, bits_v, q_rot):
-    return q_rot.new_empty((q_rot.shape[0], q_rot.shape[1], 1, q_rot.shape[2] + 2), dtype=torch.float32)
+    # the split count depends on shapes and on the device's compute-unit count only: ask the library, as the real op does
+    B, H, S, _ = k_idx.shape
+    splits = int(lib().tq_attend_splits(int(B) * int(H), int(S)))
+    return q_rot.new_empty((q_rot.shape[0], q_rot.shape[1], max(splits, 1), q_rot.shape[2] + 2), dtype=torch.float32)
 
 
 def _attend_packed_impl(queries: torch.Tensor, k_idx: torch.Tensor, k_norms: torch.Tensor, v_idx: torch.Tensor,
@@ -638,6 +675,7 @@ class JobList:
                 raise TqError("batched jobs need tensors with a dense last dimension and at most two stride "
                               "levels, and packed buffers that are contiguous or slices of a per-row store")
             rows, tokens, row_stride, token_stride = lay
+            check_table(j["table"], t.shape[-1], int(j["bits"]))
             self.host[i] = TqJob(t.data_ptr(), j["idx_bytes"].data_ptr(), j["vec_norms"].data_ptr(),
                                  j["table"].data_ptr(), rows, tokens, row_stride, token_stride,
                                  int(j["bits"]), dtype_code(t.dtype), prs)
@@ -658,6 +696,8 @@ class JobList:
         with _on(self.device):
             rc = lib().tq_decompress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, HEAD_DIM,
                                              self.workspace.data_ptr(), _stream_handle(self.device))
+        if rc:
+            self.workspace.zero_()      # counters of a launch that did not complete are not trusted
         check(rc, "tq_decompress_batched")
 
 

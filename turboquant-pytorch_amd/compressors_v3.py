@@ -86,7 +86,7 @@ class MSECompressor:
             dev = torch.device(self.device)
             if dev.type != "cuda":
                 raise _native.TqError(f"MSECompressor(device={self.device!r}): the codec runs on HIP devices only")
-            self._table = torch.from_numpy(self._table_host).to(dev)
+            self._table = _native.upload_table(self._table_host, self.head_dim, self.bits, dev)
         return self._table
 
     @torch.no_grad()

@@ -299,6 +299,18 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     return TQ_OK;
 }
 
+int tq_table_check(const void *table_host, size_t table_bytes, int head_dim, int bits) {
+    if (!table_host) return TQ_ERR_NULL;
+    if (bits < 1 || bits > 8) return TQ_ERR_BITS;
+    if (table_bytes < sizeof(TqTableHeader)) return TQ_ERR_TABLE;
+    TqTableHeader hd;
+    std::memcpy(&hd, table_host, sizeof(hd));
+    if (hd.magic != TQ_TABLE_MAGIC || hd.version != TQ_TABLE_VERSION) return TQ_ERR_TABLE;
+    if (hd.total_bytes > table_bytes || (long long)hd.total_bytes != tq_table_bytes((int)hd.head_dim, (int)hd.bits)) return TQ_ERR_TABLE;
+    if ((int)hd.head_dim != head_dim || (int)hd.bits != bits) return TQ_ERR_TABLE;
+    return TQ_OK;
+}
+
 int tq_table_quantize_host(const void *table_host, const float *r, long long n, uint8_t *idx) {
     if (!table_host || (n > 0 && (!r || !idx))) return TQ_ERR_NULL;
     TqTableHeader hd;

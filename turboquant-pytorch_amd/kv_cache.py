@@ -413,11 +413,28 @@ def hf_cache_class():
             DynamicCache.__init__(self)
             V3Cache.__init__(self, *args, **kwargs)
             self.packed_attention = packed_attention
+            # A packed decode step hands the model only the new token's K / V.  Until `packed_attention_forward` has
+            # answered it from the packed store the step is "pending"; anything else that touches the cache first
+            # means the model's attention ran over one token (another attention implementation is selected, or the
+            # tag on the key tensor was lost on the way), and that must not pass silently.
+            self._pending_layer = None
+            self._mask_checked = None      # (address, version) of the last attention mask found free of padding
+
+        def _no_pending(self, what: str) -> None:
+            if self._pending_layer is not None:
+                layer, self._pending_layer = self._pending_layer, None
+                raise RuntimeError(
+                    f"packed_attention: the decode step appended to layer {layer} was never answered by "
+                    f"packed_attention_forward (next cache call: {what}).  The model's attention ran over the new token "
+                    "alone.  Select the registered implementation (register_packed_attention(), "
+                    "model.config._attn_implementation = 'tq_packed') or create the cache with packed_attention=False.")
 
         def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
+            self._no_pending(f"update(layer {layer_idx})")
             if self.packed_attention and key_states.shape[2] == 1 and V3Cache.get_seq_length(self, layer_idx) > 0:
                 V3Cache.append(self, key_states, value_states, layer_idx)
                 key_states._tq_packed = (self, layer_idx)       # read by packed_attention_forward
+                self._pending_layer = layer_idx
                 out = (key_states, value_states)
             else:
                 out = V3Cache.update(self, key_states, value_states, layer_idx, cache_kwargs)
@@ -429,6 +446,7 @@ def hf_cache_class():
             return out
 
         def get_seq_length(self, layer_idx=0):
+            self._no_pending("get_seq_length")
             return V3Cache.get_seq_length(self, layer_idx)
 
         def get_mask_sizes(self, query_length, layer_idx=0):
@@ -438,15 +456,32 @@ def hf_cache_class():
     return HFV3Cache
 
 
+def _mask_hides_nothing(mask: torch.Tensor) -> bool:
+    """True if an attention mask (boolean: True = attend; additive: 0 = attend) lets every key through."""
+    if mask.dtype == torch.bool:
+        return bool(mask.all())
+    return bool((mask == 0).all())
+
+
 def packed_attention_forward(module, query, key, value, attention_mask, scaling=None, dropout=0.0, **kwargs):
     """Attention function for transformers' AttentionInterface.  A decode step whose keys come tagged from a
     cache in packed-attention mode is answered by `V3Cache.attend` (scores, softmax and value sum computed from
-    the packed codes; the mask is not consulted: all cached tokens count).  Everything else is passed to the
-    library's scaled-dot-product implementation unchanged."""
+    the packed codes).  `attend` counts every cached token, so a mask that hides one (a padded batch) is refused;
+    the mask of a step is inspected once, not once per layer.  Everything else is passed to the library's
+    scaled-dot-product implementation unchanged."""
     tag = getattr(key, "_tq_packed", None)
     if tag is not None and query.shape[2] == 1:
         cache, layer_idx = tag
+        if attention_mask is not None:
+            ident = (attention_mask.data_ptr(), attention_mask._version, tuple(attention_mask.shape))
+            if cache._mask_checked != ident:
+                if not _mask_hides_nothing(attention_mask):
+                    raise RuntimeError("packed_attention: the attention mask hides cached tokens (padded batch?); attention from "
+                                       "the packed store counts every cached token.  Use packed_attention=False for such batches.")
+                cache._mask_checked = ident
         out = cache.attend(query, layer_idx, scale=scaling)           # [B, Hq, 1, D]
+        if cache._pending_layer == layer_idx:
+            cache._pending_layer = None
         return out.transpose(1, 2).contiguous(), None
     from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
     return ALL_ATTENTION_FUNCTIONS["sdpa"](module, query, key, value, attention_mask, dropout=dropout, scaling=scaling, **kwargs)
@@ -454,7 +489,15 @@ def packed_attention_forward(module, query, key, value, attention_mask, scaling=
 
 def register_packed_attention(name: str = "tq_packed") -> str:
     """Register `packed_attention_forward` under `name`; select it with
-    `model.config._attn_implementation = name` (or `model.set_attn_implementation(name)`)."""
+    `model.config._attn_implementation = name` (or `model.set_attn_implementation(name)`).
+    The library's scaled-dot-product mask builder is registered under the same name: without one, transformers
+    hands a custom attention function no mask at all, and a padded batch would be attended to in full with no way
+    for the function to notice."""
     from transformers import AttentionInterface
     AttentionInterface.register(name, packed_attention_forward)
+    try:
+        from transformers.masking_utils import AttentionMaskInterface, sdpa_mask
+        AttentionMaskInterface.register(name, sdpa_mask)
+    except ImportError:          # releases that build masks inside the model: they pass them to every attention function
+        pass
     return name
