@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define TQ_ABI_VERSION 3
+#define TQ_ABI_VERSION 4
 
 /* element types of K/V tensors */
 enum { TQ_F32 = 0, TQ_F16 = 1, TQ_BF16 = 2 };
@@ -179,6 +179,34 @@ int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_j
                         int head_dim, void *stream);
 int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
                           int head_dim, void *workspace, void *stream);
+
+/*
+ * V2 key path: MSE codes of (bits - 1) bits plus one QJL sign bit per coordinate of the quantisation residual, for the
+ * unbiased inner-product estimate  <q, k> ~ <q, k_mse> + ||r|| * sqrt(pi/2) / D * <S q, sign(S r)>.
+ * Replaces TurboQuantCompressorV2.compress / asymmetric_attention_scores, turboquant/compressors.py:84-158 (and the
+ * two-stage quantiser TurboQuantProd.quantize / inner_product, turboquant/turboquant.py:134-192, whose arithmetic it is).
+ * Stored per vector, as the reference's own memory accounting counts it (validate.py:121-127): packed MSE codes and
+ * fp16 norm (tq_compress with mse_bits and the table of tq_table_build), 16 bytes of sign bits, fp16 residual norm.
+ *
+ *   tq_qjl_table_bytes / tq_qjl_table_build
+ *                   host blob with Pi^T and S as MFMA operand tiles and the codebook, from Pi (row-major, as
+ *                   tq_table_build takes it), S [head_dim * head_dim] row-major (projected = residual @ S^T,
+ *                   compressors.py:49-52 and :116) and the 2^mse_bits centroids; upload it 256-byte aligned.
+ *   tq_qjl_signs    second stage of compress (:107-117): from the input vectors (n_vec of them, token_stride elements
+ *                   apart, 16-byte aligned) and the codes tq_compress wrote for them (dense [n_vec, G]):
+ *                   residual = x - (centroids[codes] @ Pi) * ||x||  in float32,
+ *                   sign_bytes[v][b] bit 7-k = (residual @ S^T)[8b + k] >= 0  (the 1-bit code packing of tq_compress),
+ *                   residual_norm[v] = fp16(||residual||).
+ * Scores need no entry point of their own: term 1 is tq_scores on the MSE codes with q_rot = Pi q, term 2 is tq_scores
+ * on sign_bytes / residual_norm as a 1-bit store whose table was built from the identity rotation and the codebook
+ * (-1, +1), with q_rot = sqrt(pi/2) / head_dim * S q.
+ */
+long long tq_qjl_table_bytes(int head_dim, int mse_bits);
+int tq_qjl_table_build(const float *Pi, const float *S, const float *centroids, int head_dim, int mse_bits,
+                       void *table_host, size_t table_bytes);
+int tq_qjl_signs(const void *states, int dtype, long long n_vec, long long token_stride,
+                 const uint8_t *idx_bytes, const void *qjl_table_dev, int head_dim, int mse_bits,
+                 uint8_t *sign_bytes, uint16_t *residual_norm, void *stream);
 
 /*
  * tq_decompress_batched for callers that cannot allocate device memory and have no workspace to pass: code

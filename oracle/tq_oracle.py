@@ -151,6 +151,56 @@ class NumpyOracle:
 
 
 # --------------------------------------------------------------------------
+# V2 key path: MSE codes plus 1-bit QJL signs of the residual
+# --------------------------------------------------------------------------
+class QjlOracle:
+    """TurboQuantCompressorV2 of turboquant/compressors.py:84-158 in float32 numpy: `bits` is the total budget, the
+    codebook `centroids` has 2^max(bits-1, 1) levels (:33), S is the [D, D] Gaussian projection (:49-52).
+    Pinned by tests/golden/v2_qjl.npz (outputs of the reference class on seeded inputs)."""
+
+    def __init__(self, Pi: np.ndarray, S: np.ndarray, centroids: np.ndarray):
+        self.Pi = np.ascontiguousarray(Pi, dtype=np.float32)
+        self.S = np.ascontiguousarray(S, dtype=np.float32)
+        self.centroids = np.ascontiguousarray(centroids, dtype=np.float32)
+        self.D = self.Pi.shape[0]
+        self.mse = NumpyOracle(self.Pi, self.centroids, int(np.log2(self.centroids.size)))
+
+    def compress(self, x: np.ndarray) -> dict:
+        """x [..., D] float32 -> codes [N,D], norms fp32 [N], k_mse fp32 [N,D] (and its fp16 bits), residual norm fp32
+        (and fp16 bits), projected residual fp32 [N,D], signs int8 [N,D] in {-1,+1}"""
+        flat = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.D)
+        norms, rotated = self.mse.rotate(flat)                                   # :96-103
+        codes = self.mse.nearest(rotated)                                        # :104-105
+        with np.errstate(invalid="ignore", over="ignore"):
+            k_mse = (self.centroids[codes] @ self.Pi) * norms[:, None]           # :108-109, fp32 norms
+            residual = flat - k_mse                                              # :112
+            rnorm = np.sqrt(np.sum(residual * residual, axis=-1, dtype=np.float32)).astype(np.float32)   # :113
+            projected = residual @ self.S.T                                      # :116
+        signs = np.where(projected >= 0, 1, -1).astype(np.int8)                  # :117 (a projection of 0 counts as +1)
+        return {"codes": codes, "norms_f32": norms, "rotated": rotated, "k_mse": k_mse,
+                "k_mse_f16": k_mse.astype(np.float16).view(np.uint16), "residual_norm_f32": rnorm,
+                "residual_norm": rnorm.astype(np.float16).view(np.uint16), "projected": projected, "signs": signs}
+
+    def scores(self, q: np.ndarray, k_mse_f16: np.ndarray, signs: np.ndarray, residual_norm_f16: np.ndarray) -> np.ndarray:
+        """asymmetric_attention_scores (:124-158): q [R, Sq, D]; stored fp16 k_mse [R, Sk, D], signs [R, Sk, D],
+        fp16 residual norms [R, Sk] -> float32 [R, Sq, Sk]"""
+        k = k_mse_f16.view(np.float16).astype(np.float32)
+        rn = residual_norm_f16.view(np.float16).astype(np.float32)
+        q = np.ascontiguousarray(q, dtype=np.float32)
+        term1 = q @ np.swapaxes(k, -1, -2)                                       # :144
+        ip = (q @ self.S.T) @ np.swapaxes(signs.astype(np.float32), -1, -2)      # :149-152
+        scale = np.float32(np.sqrt(np.pi / 2) / self.S.shape[0])                 # :155-156
+        return term1 + scale * ip * rn[..., None, :]                             # :158
+
+
+def pack_signs(signs: np.ndarray) -> np.ndarray:
+    """{-1,+1} [N, D] -> [N, D/8] bytes, coordinate 8b+k in bit 7-k of byte b (the 1-bit code packing of
+    compressors_v3.py:64-74 applied to the bit (sign >= 0))."""
+    bits = (np.asarray(signs) > 0).astype(np.uint8)
+    return np.packbits(bits.reshape(bits.shape[0], -1, 8), axis=-1, bitorder="big").reshape(bits.shape[0], -1)
+
+
+# --------------------------------------------------------------------------
 # torch CPU restatement (the timed "reference CPU path")
 # --------------------------------------------------------------------------
 class TorchCpuOracle:

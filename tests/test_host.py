@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol(pkg):
     for name in declared:
         assert hasattr(lib, name), name
     assert sorted(pkg._native.EXPORTS) == declared
-    assert lib.tq_abi_version() == 3
+    assert lib.tq_abi_version() == 4
     assert lib.tq_status_string(0) == b"ok"
     assert b"bits" in lib.tq_status_string(-2)
 

@@ -281,3 +281,36 @@ def test_attention_decode_oracle_is_textbook_attention(oracle):
         assert np.abs(scores[b, hq] - s).max() < 1e-12
         p = np.exp(s - s.max()); p /= p.sum()
         assert np.abs(out[b, hq] - (p[:, None] * V[b, h].astype(np.float64)).sum(0)).max() < 1e-12
+
+
+def test_v2_qjl_oracle_against_reference_vectors(oracle):
+    """The numpy restatement of the V2 key path against outputs of the reference class (tests/golden/v2_qjl.npz):
+    stored fp16 reconstruction and residual norms to one fp16 unit, signs identical except where the projection is
+    within 1e-5 * |S row| * |residual| of zero (none, or a handful), scores to float32 rounding."""
+    import os
+    fx = np.load(os.path.join(os.path.dirname(__file__), "golden", "v2_qjl.npz"))
+    seen = 0
+    for bits in (2, 3, 4, 5):
+        orc = oracle.QjlOracle(fx[f"b{bits}_Pi"], fx[f"b{bits}_S"], fx[f"b{bits}_centroids"])
+        assert orc.centroids.size == 1 << max(bits - 1, 1)
+        srow = np.linalg.norm(orc.S, axis=1)
+        for dn in ("f16", "bf16", "f32"):
+            tag = f"b{bits}_{dn}"
+            x = oracle.widen(fx[tag + "_x"], dn).reshape(-1, 128)
+            out = orc.compress(x)
+            assert oracle.fp16_ulp_distance(out["k_mse_f16"].reshape(-1), fx[tag + "_k_mse"].reshape(-1)).max() <= 1
+            assert oracle.fp16_ulp_distance(out["residual_norm"], fx[tag + "_residual_norm"].reshape(-1)).max() <= 1
+            ref_signs = fx[tag + "_qjl_signs"].reshape(-1, 128)
+            diff = out["signs"] != ref_signs
+            margin = np.abs(out["projected"]) / (srow[None, :] * np.maximum(out["residual_norm_f32"][:, None], 1e-30))
+            assert diff.sum() <= 4 and (margin[diff] < 1e-5).all(), (tag, int(diff.sum()))
+            assert (out["signs"][0] == 1).all()                       # the all-zero vector: projection 0 -> +1
+            q = fx[tag + "_q"].reshape(2, 5, 128)
+            sc = orc.scores(q, fx[tag + "_k_mse"].reshape(2, 80, 128), ref_signs.reshape(2, 80, 128),
+                            fx[tag + "_residual_norm"].reshape(2, 80))
+            ref = fx[tag + "_scores"].reshape(2, 5, 80)
+            assert np.abs(sc - ref).max() <= 2e-5 * np.abs(ref).max(), tag
+            seen += 1
+    assert seen == 12
+    s = np.array([[1, -1, -1, -1, -1, -1, -1, 1] + [1] * 8])
+    assert oracle.pack_signs(s).tolist() == [[0x81, 0xFF]]

@@ -20,7 +20,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(CSRC, "libtqamd.so")
-SOURCES = ("tq_host.cpp", "tq_compress.hip", "tq_decompress.hip", "tq_attend.hip")
+SOURCES = ("tq_host.cpp", "tq_compress.hip", "tq_decompress.hip", "tq_attend.hip", "tq_qjl.hip")
 HEADERS = ("tq_table.h", "tq_device.h", os.path.join("..", "..", "include", "tqamd.h"))
 GPU_ARCH = "gfx950"
 
@@ -88,7 +88,7 @@ EXPORTS = (
     "tq_abi_version", "tq_status_string", "tq_device_count", "tq_bytes_per_vector",
     "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_check", "tq_table_quantize_host",
     "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched", "tq_workspace_bytes",
-    "tq_decompress_batched_noalloc",
+    "tq_decompress_batched_noalloc", "tq_qjl_table_bytes", "tq_qjl_table_build", "tq_qjl_signs",
     "tq_scores", "tq_weighted_values", "tq_weighted_values_splits", "tq_attend_partials", "tq_attend_splits",
     "tq_attend_prepare", "tq_attend_merge", "tq_append_token", "tq_attend_step",
 )
@@ -132,11 +132,15 @@ def lib() -> ctypes.CDLL:
     L.tq_weighted_values.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ll, ci, vp, ci, vp, vp]
     L.tq_decompress_batched.argtypes = [vp, vp, ci, ci, vp, vp]
     L.tq_decompress_batched_noalloc.argtypes = [vp, vp, ci, ci, vp]
+    L.tq_qjl_table_bytes.restype = ll
+    L.tq_qjl_table_bytes.argtypes = [ci, ci]
+    L.tq_qjl_table_build.argtypes = [vp, vp, vp, ci, ci, vp, ctypes.c_size_t]
+    L.tq_qjl_signs.argtypes = [vp, ci, ll, ll, vp, vp, ci, ci, vp, vp, vp]
     L.tq_append_token.argtypes = [vp, vp, ci, ll, ll, vp, vp, ll, ll, ll, vp, vp, ci, ci, ci, vp, vp, vp, vp, ll, ll, ll, vp]
     L.tq_attend_step.argtypes = [vp, ci, ll, ci, ctypes.c_float, vp, vp, vp, vp, ci, ll, ll, vp, vp, vp, vp, ll, ll,
                                  vp, vp, ci, ci, ci, vp, vp, vp, ci, vp, ci, vp]
     for name in EXPORTS:
-        if name not in ("tq_status_string", "tq_table_bytes", "tq_workspace_bytes"):
+        if name not in ("tq_status_string", "tq_table_bytes", "tq_workspace_bytes", "tq_qjl_table_bytes"):
             getattr(L, name).restype = ci
     _lib = L
     return L

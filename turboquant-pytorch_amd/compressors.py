@@ -1,0 +1,182 @@
+"""
+The V2 compressors of the reference (turboquant/compressors.py) on the MI355X kernels: `TurboQuantCompressorV2`
+(keys: MSE codes of bits-1 bits plus one QJL sign bit per coordinate of the residual, scores straight from the
+compressed form, compressors.py:25-158) and `TurboQuantCompressorMSE` (values, compressors.py:161-221).
+
+Same constructor arguments, method names and score definition.  What `compress` returns for keys is the packed form
+the reference's own memory accounting describes (validate.py:121-127: indices, sign bits, residual norm, vector
+norm): packed MSE codes, fp16 norms, 16 bytes of sign bits and an fp16 residual norm per vector, 4.5x to 9x smaller than
+the fp16 reconstruction plus int8 signs the reference materialises.  `asymmetric_attention_scores` takes that dict;
+`reference_format` expands it into the reference's keys ("k_mse", "qjl_signs") for callers that look inside.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _native
+from .compressors_v3 import MSECompressor, _cached_centroids, _cached_rotation
+
+
+def _qjl_matrix(head_dim: int, seed: int) -> torch.Tensor:
+    """The Gaussian projection of compressors.py:49-52 (CPU generator, seed + 10000)."""
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(seed + 10000)
+    return torch.randn(head_dim, head_dim, generator=gen)
+
+
+class TurboQuantCompressorV2:
+    """Keys for asymmetric attention: interface of compressors.py:25-158."""
+
+    def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cuda"):
+        self.head_dim = head_dim
+        self.bits = bits
+        self.mse_bits = max(bits - 1, 1)
+        self.device = device
+        pi_host = _cached_rotation(head_dim, seed)
+        cent_host = _cached_centroids(head_dim, self.mse_bits)
+        self._setup(pi_host, _qjl_matrix(head_dim, seed), cent_host)
+
+    @classmethod
+    def from_tensors(cls, Pi: torch.Tensor, S: torch.Tensor, centroids: torch.Tensor, bits: int, device: str = "cuda"):
+        """A compressor over explicit matrices and codebook (parity tests pass the reference's own through here)."""
+        self = cls.__new__(cls)
+        self.head_dim = Pi.shape[0]
+        self.bits = bits
+        self.mse_bits = max(bits - 1, 1)
+        self.device = device
+        self._setup(Pi.detach().cpu().float(), S.detach().cpu().float(), centroids.detach().cpu().float())
+        return self
+
+    def _setup(self, pi_host: torch.Tensor, s_host: torch.Tensor, cent_host: torch.Tensor) -> None:
+        import numpy as np
+        dev = self.device
+        self.Pi = pi_host.to(dev).contiguous()
+        self.PiT = self.Pi.T.contiguous()
+        self.S = s_host.to(dev).contiguous()
+        self.centroids = cent_host.to(dev)
+        self._mse = MSECompressor.from_tensors(pi_host, cent_host, self.mse_bits, device=dev)
+        # the sign bits are a 1-bit store over the codebook (-1, +1) in an un-rotated space: the score kernels read them as such
+        self._sign = MSECompressor.from_tensors(torch.eye(self.head_dim), torch.tensor([-1.0, 1.0]), 1, device=dev)
+        L = _native.lib()
+        n = L.tq_qjl_table_bytes(self.head_dim, self.mse_bits)
+        if n < 0:
+            _native.check(int(n), "tq_qjl_table_bytes")
+        blob = np.zeros(n, dtype=np.uint8)
+        pi = np.ascontiguousarray(pi_host.numpy(), dtype=np.float32)
+        s = np.ascontiguousarray(s_host.numpy(), dtype=np.float32)
+        c = np.ascontiguousarray(cent_host.numpy(), dtype=np.float32)
+        _native.check(L.tq_qjl_table_build(pi.ctypes.data, s.ctypes.data, c.ctypes.data, self.head_dim, self.mse_bits,
+                                           blob.ctypes.data, blob.size), "tq_qjl_table_build")
+        self._qjl_host = blob
+        self._qjl_table = None
+
+    def _table(self) -> torch.Tensor:
+        if self._qjl_table is None:
+            dev = torch.device(self.device)
+            if dev.type != "cuda":
+                raise _native.TqError(f"TurboQuantCompressorV2(device={self.device!r}): the codec runs on HIP devices only")
+            self._qjl_table = torch.from_numpy(self._qjl_host).to(dev)
+        return self._qjl_table
+
+    @torch.no_grad()
+    def compress(self, states: torch.Tensor) -> dict:
+        """(B, H, S, D) -> {"idx_bytes" u8 [B,H,S,G], "vec_norms" f16 [B,H,S], "sign_bytes" u8 [B,H,S,D/8],
+        "residual_norm" f16 [B,H,S], "shape"}.  Two launches: MSE codes and norms, then residual signs and norms."""
+        B, H, S, D = states.shape
+        _native._require_gpu(states, "states")
+        if not states.is_contiguous() or states.data_ptr() % 16:
+            states = states.contiguous()
+        first = self._mse.compress(states)
+        sign_bytes = torch.empty((B, H, S, D // 8), dtype=torch.uint8, device=states.device)
+        residual_norm = torch.empty((B, H, S), dtype=torch.float16, device=states.device)
+        n_vec = B * H * S
+        if n_vec:
+            with _native._on(states.device):
+                rc = _native.lib().tq_qjl_signs(states.data_ptr(), _native.dtype_code(states.dtype), n_vec, D,
+                                                first["idx_bytes"].data_ptr(), self._table().data_ptr(), D, self.mse_bits,
+                                                sign_bytes.data_ptr(), residual_norm.data_ptr(),
+                                                _native._stream_handle(states.device))
+            _native.check(rc, "tq_qjl_signs")
+        return {"idx_bytes": first["idx_bytes"], "vec_norms": first["vec_norms"], "sign_bytes": sign_bytes,
+                "residual_norm": residual_norm, "shape": (B, H, S, D)}
+
+    @torch.no_grad()
+    def reference_format(self, compressed: dict) -> dict:
+        """The dictionary the reference's compress returns (:119-124): "k_mse" fp16 [B,H,S,D], "qjl_signs" int8 in
+        {-1,+1} [B,H,S,D], "residual_norm", "shape", expanded from the packed form."""
+        B, H, S, D = compressed["shape"]
+        k_mse = self._mse.decompress({"idx_bytes": compressed["idx_bytes"], "vec_norms": compressed["vec_norms"],
+                                      "shape": (B, H, S, D), "idx_pad": 0}).to(torch.float16)
+        shifts = torch.arange(7, -1, -1, device=compressed["sign_bytes"].device, dtype=torch.uint8)
+        bits = (compressed["sign_bytes"].unsqueeze(-1) >> shifts) & 1
+        signs = (bits.to(torch.int8) * 2 - 1).reshape(B, H, S, D)
+        return {"k_mse": k_mse, "qjl_signs": signs, "residual_norm": compressed["residual_norm"], "shape": (B, H, S, D)}
+
+    @torch.no_grad()
+    def asymmetric_attention_scores(self, queries: torch.Tensor, compressed: dict) -> torch.Tensor:
+        """<q, k> ~ <q, k_mse> + ||r|| sqrt(pi/2)/m <S q, sign(S r)>  (:124-158): queries (B, H, S_q, D) against a dict
+        from compress -> float32 (B, H, S_q, S_k).  Both terms are computed from the packed bytes (the query is
+        rotated by Pi for the first and projected by S for the second; neither the reconstruction nor the signs are
+        expanded).  A dict in the reference's format (`reference_format`) is accepted too and takes plain matrix
+        products."""
+        m = self.S.shape[0]
+        corr = math.sqrt(math.pi / 2) / m
+        if "idx_bytes" not in compressed:
+            k_mse = compressed["k_mse"].float()
+            term1 = torch.matmul(queries.float(), k_mse.transpose(-2, -1))
+            ip = torch.matmul(torch.matmul(queries.float(), self.S.T), compressed["qjl_signs"].float().transpose(-2, -1))
+            return term1 + corr * ip * compressed["residual_norm"].float().unsqueeze(-2)
+        B, H, S_k, D = compressed["shape"]
+        S_q = queries.shape[2]
+        out = torch.empty((B, H, S_q, S_k), dtype=torch.float32, device=queries.device)
+        if out.numel() == 0:
+            return out
+        q = queries.float()
+        q_sign = torch.matmul(q, self.S.T) * corr
+        step = 32                                   # query tokens per key row and launch
+        for lo in range(0, S_q, step):
+            hi = min(lo + step, S_q)
+            n = hi - lo
+            first = self._mse.packed_scores(compressed["idx_bytes"], compressed["vec_norms"], q[:, :, lo:hi].reshape(B, H * n, D))
+            second = self._sign.packed_scores(compressed["sign_bytes"], compressed["residual_norm"],
+                                              q_sign[:, :, lo:hi].reshape(B, H * n, D))
+            out[:, :, lo:hi] = (first + second).reshape(B, H, n, S_k)
+        return out
+
+
+class TurboQuantCompressorMSE:
+    """Values: MSE codes only, interface of compressors.py:161-221.  `compress` returns the reference's keys
+    ("indices" one code per byte [N, D], "vec_norms" fp16 [N], "shape") next to the packed bytes the kernels wrote;
+    `decompress` reads the packed bytes when they are there and packs the indices otherwise."""
+
+    def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cuda"):
+        self.head_dim = head_dim
+        self.bits = bits
+        self.device = device
+        self._mse = MSECompressor(head_dim, bits, seed, device=device)
+        self.Pi = self._mse.Pi
+        self.centroids = self._mse.centroids
+
+    @torch.no_grad()
+    def compress(self, states: torch.Tensor) -> dict:
+        B, H, S, D = states.shape
+        packed = self._mse.compress(states)
+        ipb = 8 // self.bits
+        shifts = torch.arange(ipb - 1, -1, -1, device=states.device, dtype=torch.uint8) * self.bits
+        codes = (packed["idx_bytes"].reshape(B * H * S, -1, 1) >> shifts) & ((1 << self.bits) - 1)
+        return {"indices": codes.reshape(B * H * S, -1)[:, :D].contiguous(), "vec_norms": packed["vec_norms"].reshape(-1),
+                "shape": (B, H, S, D), "idx_bytes": packed["idx_bytes"]}
+
+    @torch.no_grad()
+    def decompress(self, compressed: dict) -> torch.Tensor:
+        B, H, S, D = compressed["shape"]
+        idx_bytes = compressed.get("idx_bytes")
+        if idx_bytes is None:
+            ipb = 8 // self.bits
+            codes = compressed["indices"].reshape(B * H * S, D // ipb, ipb).to(torch.int32)
+            weights = torch.tensor([1 << (self.bits * i) for i in range(ipb - 1, -1, -1)], device=codes.device, dtype=torch.int32)
+            idx_bytes = (codes * weights).sum(-1).to(torch.uint8).reshape(B, H, S, -1)
+        return self._mse.decompress({"idx_bytes": idx_bytes, "vec_norms": compressed["vec_norms"].reshape(B, H, S),
+                                     "shape": (B, H, S, D), "idx_pad": 0})

@@ -299,6 +299,65 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     return TQ_OK;
 }
 
+long long tq_qjl_table_bytes(int head_dim, int mse_bits) {
+    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
+    if (mse_bits < 1 || mse_bits > 7) return TQ_ERR_BITS;
+    return (long long)sizeof(TqQjlHeader) + 5ll * TQ_OPERAND_BYTES + 1024;
+}
+
+int tq_qjl_table_build(const float *Pi, const float *S, const float *centroids, int head_dim, int mse_bits,
+                       void *table_host, size_t table_bytes) {
+    if (!Pi || !S || !centroids || !table_host) return TQ_ERR_NULL;
+    const long long need = tq_qjl_table_bytes(head_dim, mse_bits);
+    if (need < 0) return (int)need;
+    if (table_bytes < (size_t)need) return TQ_ERR_SIZE;
+    const int D = head_dim, levels = 1 << mse_bits;
+    if (!valid_codebook(centroids, levels)) return TQ_ERR_CODEBOOK;
+    for (int i = 0; i < D * D; ++i)
+        if (!std::isfinite(Pi[i]) || !std::isfinite(S[i])) return TQ_ERR_SIZE;
+    uint8_t *blob = static_cast<uint8_t *>(table_host);
+    std::memset(blob, 0, (size_t)need);
+    TqQjlHeader hd{};
+    hd.magic = TQ_QJL_MAGIC;
+    hd.version = TQ_QJL_VERSION;
+    hd.head_dim = (uint32_t)D;
+    hd.mse_bits = (uint32_t)mse_bits;
+    hd.levels = (uint32_t)levels;
+    hd.off_pit = sizeof(TqQjlHeader);
+    hd.off_s = hd.off_pit + 3 * TQ_OPERAND_BYTES;
+    hd.off_centroids = hd.off_s + 2 * TQ_OPERAND_BYTES;
+    hd.total_bytes = (uint32_t)need;
+    uint16_t *pit = reinterpret_cast<uint16_t *>(blob + hd.off_pit);
+    uint16_t *sm = reinterpret_cast<uint16_t *>(blob + hd.off_s);
+    const size_t term = TQ_OPERAND_BYTES / 2;
+    for (int t = 0; t < TQ_TILES; ++t)
+        for (int s = 0; s < TQ_STEPS; ++s)
+            for (int l = 0; l < 64; ++l) {
+                const int m = l % 32, hk = l / 32;
+                const int a = m / 8, h = (m / 4) % 2, b = m % 4;
+                const int out = 32 * t + 16 * h + 4 * a + b;
+                for (int i = 0; i < 8; ++i) {
+                    const size_t o = (((size_t)t * TQ_STEPS + s) * 64 + l) * 8 + i;
+                    const int k = 16 * s + 8 * hk + i;
+                    float v = Pi[k * D + out];                 // Pi^T[out][k]
+                    for (int q = 0; q < 3; ++q) {
+                        const uint16_t h16 = to_bf16(v);
+                        pit[q * term + o] = h16;
+                        v -= from_bf16(h16);
+                    }
+                    v = S[out * D + k];
+                    for (int q = 0; q < 2; ++q) {
+                        const uint16_t h16 = to_bf16(v);
+                        sm[q * term + o] = h16;
+                        v -= from_bf16(h16);
+                    }
+                }
+            }
+    std::memcpy(blob + hd.off_centroids, centroids, (size_t)levels * 4);
+    std::memcpy(blob, &hd, sizeof(hd));
+    return TQ_OK;
+}
+
 int tq_table_check(const void *table_host, size_t table_bytes, int head_dim, int bits) {
     if (!table_host) return TQ_ERR_NULL;
     if (bits < 1 || bits > 8) return TQ_ERR_BITS;
