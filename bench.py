@@ -47,6 +47,9 @@ WORKLOADS = {
     # (32 query heads over 8 kv heads) computed from the packed store, nothing de-quantised to memory
     "decode-attend-64x16k": dict(layers=32, batch=64, heads=8, tokens=16384, dtype="bf16", key_bits=4, value_bits=2,
                                  protected=0, window=128, decode=True, attend=True, q_heads=32),
+    # the V2 key path (MSE codes + 1-bit QJL signs of the residual): a step compresses every layer's keys (two launches
+    # per layer) and scores one query per head against them from the packed bytes
+    "v2-keys-32k": dict(layers=8, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=3, value_bits=0, protected=0, v2=True),
     # one sequence with a long context: the latency-bound end of the same path
     "decode-attend-1x32k": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2,
                                 protected=0, window=128, decode=True, attend=True, q_heads=32),
@@ -141,6 +144,65 @@ def cpu_baseline(pkg, widths, budget_s=20.0):
                  "sample": "the same on " + ", ".join(port_desc) + " vectors through the scalar C restatement (oracle/tq_oracle.c, OpenMP)",
                  "per_width_vectors_per_s": {str(b): r for b, r in port.items()}},
     }
+
+
+def run_v2(args, torch, pkg, w, dev):
+    """TurboQuantCompressorV2 on synthetic keys: compress (codes + norms, then residual signs + norms) and
+    asymmetric_attention_scores for one query token per head, every layer with its own rotation and projection."""
+    L, B, H, S, bits = w["layers"], w["batch"], w["heads"], w["tokens"], w["key_bits"]
+    comps = [pkg.TurboQuantCompressorV2(128, bits, seed=1000 * l, device=str(dev)) for l in range(L)]
+    keys = [synth_kv(torch, (B, H, S, 128), seed=6_000_000 + l, dtype=torch.bfloat16, device=dev) for l in range(L)]
+    q = synth_kv(torch, (B, H, 1, 128), seed=6_000_100, dtype=torch.float32, device=dev)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    marks = [[(ev(), ev(), ev()) for _ in range(L)] for _ in range(args.steps)]
+
+    def step(ms=None):
+        out = None
+        for l in range(L):
+            if ms:
+                ms[l][0].record()
+            packed = comps[l].compress(keys[l])
+            if ms:
+                ms[l][1].record()
+            out = comps[l].asymmetric_attention_scores(q, packed)
+            if ms:
+                ms[l][2].record()
+        return out, packed
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        scores, packed = step(marks[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    sec = wall / args.steps
+    c_ms = sum(m[0].elapsed_time(m[1]) for ms in marks for m in ms) / args.steps
+    s_ms = sum(m[1].elapsed_time(m[2]) for ms in marks for m in ms) / args.steps
+    # sanity: the estimate tracks the true inner products of the last layer
+    true = torch.matmul(q.float(), keys[-1].float().transpose(-2, -1))
+    cos = float(torch.nn.functional.cosine_similarity(scores.flatten(), true.flatten(), dim=0))
+    if not cos > 0.8:       # (3 bits, random query: noise of the estimate ~0.04 |q||k| against signals ~0.09 |q||k|)
+        sys.exit(f"bench.py: V2 scores do not follow the true inner products (cosine {cos})")
+    n_vec = L * B * H * S
+    mse_bits = max(bits - 1, 1)
+    stored = packed_bytes(mse_bits) + 2 + 16 + 2
+    comp_bytes = n_vec * (256 + stored)                 # one pass over the keys, the packed form written once
+    score_bytes = n_vec * (stored + 4)                  # the packed form read once, one float32 score per key written
+    result = {
+        "metric": "KV vectors/sec (V2 keys: compress + scores from the packed form)", "value": n_vec / sec, "unit": "vectors/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "layers": L, "batch": B, "kv_heads": H, "tokens": S, "head_dim": 128,
+                   "bits": bits, "mse_bits": mse_bits, "stored_bytes_per_vector": stored, "queries_per_head": 1},
+        "compress_ms_per_step": c_ms, "scores_ms_per_step": s_ms,
+        "step_algorithmic_GB": (comp_bytes + score_bytes) / 1e9, "step_GBps": (comp_bytes + score_bytes) / sec / 1e9,
+        "roofline": {"bound": "hbm", "kernel": "compress (tq_compress + tq_qjl_signs, per layer)", "achieved": comp_bytes / c_ms / 1e6,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": comp_bytes / c_ms / 1e6 / HBM_PEAK_GBS, "traffic": None},
+        "score_cosine_vs_true": cos,
+    }
+    print(json.dumps(result))
 
 
 def run_decode(args, torch, pkg, w, dev):
@@ -252,6 +314,8 @@ def main():
     w = WORKLOADS[args.workload]
     if w.get("decode"):
         return run_decode(args, torch, pkg, w, dev)
+    if w.get("v2"):
+        return run_v2(args, torch, pkg, w, dev)
     L, B, H, S = w["layers"], w["batch"], w["heads"], w["tokens"]
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16}[w["dtype"]]
     n_vec = B * H * S
