@@ -13,6 +13,10 @@ window.  `--workload llama3-8b-32k-k4v2` runs the same shape with every layer at
 `--workload qwen2.5-3b-8k` is the small Qwen2.5-3B-shaped cache (36 layers x [1, 2, 8192, 128] fp16); `--workload decode-64x16k` is the streaming
 decode case (config 5): a step is one generated token through `V3Cache.update` on every layer.
 
+Order of a run: W warm-up steps; an untimed pass with every launch between its own HIP events (the per-kernel table, and
+which launch is the slowest); then the timed region of exactly K steps, with events around that slowest launch only (its
+duration in `roofline` is the one measured there).
+
 Prints ONE JSON line: metric, value (vectors/s), ms_per_step, config.workload, roofline (dominant kernel) and cpu_baseline.
 """
 import argparse
@@ -350,24 +354,45 @@ def main():
         if any(launches.index(("compress", b)) > launches.index(("decompress", b)) for b in order):
             raise SystemExit("--launch-order: a width group is de-quantised before it is compressed")
 
-    def step(evs=None):
-        """One pass over the cache.  `evs`: pre-created (start, stop) event pairs, one per launch."""
+    def step(evs=None, only=None):
+        """One pass over the cache.  `evs`: pre-created (start, stop) event pairs, one per launch; `only`: the
+        index of the single launch that is bracketed (all of them when None)."""
         for i, (direction, b) in enumerate(launches):
-            if evs is not None:
+            timed = evs is not None and (only is None or only == i)
+            if timed:
                 evs[i][0].record()
             (comp_lists[b].compress if direction == "compress" else deco_lists[b].decompress)()
-            if evs is not None:
+            if timed:
                 evs[i][1].record()
 
-    # HIP events are created (and recorded once, which is what allocates them) before the timed region
-    step_events = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in launches]
-                   for _ in range(args.steps)]
+    def make_events(n_steps):
+        # HIP events are created and recorded once (which is what allocates them) outside any timed region
+        evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in launches]
+               for _ in range(n_steps)]
+        for row in evs:
+            for e0, e1 in row:
+                e0.record()
+                e1.record()
+        return evs
+
     for _ in range(args.warmup):
         step()
-    for evs in step_events:
-        for e0, e1 in evs:
-            e0.record()
-            e1.record()
+    # ---- per-kernel pass (untimed): every launch between its own pair of events.  An event record between two
+    # kernels keeps the second from starting under the tail of the first (about 3 us each, 12 of them a step), so the
+    # timed region below brackets one launch only, the slowest one of this pass.  The pass also brings the clocks to
+    # the state of a running job: the first tens of milliseconds after an idle period run slower.
+    table_steps = max(args.steps, 10)
+    table_events = make_events(table_steps)
+    torch.cuda.synchronize()
+    for evs in table_events:
+        step(evs)
+    torch.cuda.synchronize()
+    table_ms = {}
+    for li, launch in enumerate(launches):
+        table_ms[launch] = sum(evs[li][0].elapsed_time(evs[li][1]) for evs in table_events) / table_steps
+    dominant_launch = max(table_ms, key=table_ms.get)
+    dominant_index = launches.index(dominant_launch)
+    step_events = make_events(args.steps)
     torch.cuda.synchronize()
 
     # ---- timed region: exactly `steps` steps ----------------------------------------------------
@@ -376,16 +401,13 @@ def main():
     t0 = time.perf_counter()
     start.record()
     for k in range(args.steps):
-        step(step_events[k])
+        step(step_events[k], only=dominant_index)
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     gpu_ms = start.elapsed_time(stop)
     ms_per_step = wall * 1000.0 / args.steps
-    events = {}
-    for evs in step_events:
-        for launch, pair in zip(launches, evs):
-            events.setdefault(launch, []).append(pair)
+    live_ms = sum(evs[dominant_index][0].elapsed_time(evs[dominant_index][1]) for evs in step_events) / args.steps
 
     # ---- sanity: what was timed is a real round trip ----------------------------------------------
     j = groups[order[0]][0]
@@ -398,21 +420,24 @@ def main():
     total_vec = 2 * L * n_vec                       # K and V counted separately
     kernels = {}
     step_bytes = 0
-    for (direction, b), evs in events.items():
+    for (direction, b), table_avg in table_ms.items():
         jobs = len(groups[b])
         bytes_per_launch = jobs * n_vec * algorithmic_bytes(b, elem, direction)
-        avg_ms = sum(e0.elapsed_time(e1) for e0, e1 in evs) / len(evs)
+        live = (direction, b) == dominant_launch
+        avg_ms = live_ms if live else table_avg          # the dominant launch: measured inside the timed region
         step_bytes += bytes_per_launch
         flop = jobs * n_vec * ROTATION_FLOP * MFMA_PASSES[direction]
         kernels[f"{direction}_b{b}"] = {
             "launches_per_step": 1, "jobs": jobs, "vectors_per_launch": jobs * n_vec,
             "algorithmic_bytes_per_launch": bytes_per_launch, "avg_ms": avg_ms,
+            "timed": "events inside the timed region" if live else f"events in the {table_steps} untimed steps before it",
+            "avg_ms_untimed_pass": table_avg,
             "achieved_GBps": bytes_per_launch / avg_ms / 1e6,
             "frac_of_hbm_peak": bytes_per_launch / avg_ms / 1e6 / HBM_PEAK_GBS,
             "mfma_flop_per_launch": flop, "mfma_PFLOPs": flop / avg_ms / 1e12,
             "frac_of_mfma_peak": flop / avg_ms / 1e12 / MFMA_PEAK_PFLOPS,
         }
-    dominant = max(kernels, key=lambda k: kernels[k]["avg_ms"])
+    dominant = f"{dominant_launch[0]}_b{dominant_launch[1]}"
     dk = kernels[dominant]
     # HBM bytes per launch of the dominant kernel as the counters saw them (FETCH_SIZE + WRITE_SIZE, calibrated against
     # a copy kernel): a number from the committed profile run of this workload, not measured by this process
@@ -444,6 +469,7 @@ def main():
         "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w["dtype"], "data": "synthetic",
+        "untimed_steps_after_warmup": table_steps,
         "config": {"workload": args.workload, "layers": L, "batch": B, "kv_heads": H, "tokens": S, "head_dim": 128,
                    "key_bits": w["key_bits"], "value_bits": w["value_bits"], "protected_layers": w["protected"],
                    "residual_window": 0, "width_groups": {str(b): len(groups[b]) for b in order},

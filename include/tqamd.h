@@ -32,7 +32,7 @@ enum {
     TQ_OK = 0,
     TQ_ERR_NULL = -1,        /* a required pointer is NULL */
     TQ_ERR_BITS = -2,        /* bits outside 1..8 */
-    TQ_ERR_HEAD_DIM = -3,    /* head_dim the kernels do not support (only 128) */
+    TQ_ERR_HEAD_DIM = -3,    /* head_dim the kernels do not support (see tq_compress) */
     TQ_ERR_DTYPE = -4,       /* unknown element type */
     TQ_ERR_SIZE = -5,        /* negative / inconsistent size, stride or buffer too small */
     TQ_ERR_CODEBOOK = -6,    /* centroids not finite and strictly ascending */
@@ -102,10 +102,14 @@ int tq_table_quantize_host(const void *table_host, const float *r, long long n, 
  *
  *   states      device pointer, `dtype` elements; vector n (0 <= n < rows*tokens) starts at
  *               element  (n / tokens) * row_stride + (n % tokens) * token_stride
- *               and its head_dim (=128) elements are contiguous.  A contiguous
- *               [B,H,S,D] tensor is rows=1, tokens=B*H*S, token_stride=128; a slice
- *               [:, :, :s, :] of one is rows=B*H, tokens=s, row_stride=S*128.
+ *               and its head_dim elements are contiguous.  A contiguous
+ *               [B,H,S,D] tensor is rows=1, tokens=B*H*S, token_stride=D; a slice
+ *               [:, :, :s, :] of one is rows=B*H, tokens=s, row_stride=S*D.
  *               Base address and strides must keep every vector 16-byte aligned.
+ *   head_dim    128 runs the tuned kernels; tq_compress, tq_decompress and their batched forms also take
+ *               every other multiple of 32 from 32 to 256 (compressors_v3.py:37-43 accepts any head_dim),
+ *               through one pair of kernels that reads the dimension at run time.  Everything else in this
+ *               header (scores, weighted values, attention, token append, QJL signs) is 128 only.
  *   table_dev   device copy of the blob from tq_table_build
  *   idx_bytes   device, uint8, bytes_per_vector per packed slot
  *   vec_norms   device, one IEEE fp16 bit pattern per packed slot (norm of the fp32-widened vector)

@@ -1,0 +1,167 @@
+"""GPU parity for head dimensions other than 128 (compress / decompress take every multiple of 32 up to 256;
+upstream turboquant/compressors_v3.py:37-43 builds rotation and codebook for any head_dim).  Same bars as the
+128-wide tests: codes bit-exact outside a 1e-5 window around a decision boundary, fp16 norms within one ulp,
+reconstruction within 1e-3 relative L2 of the oracle's.
+"""
+import numpy as np
+import pytest
+import torch
+
+from test_gpu_parity import DEV, REL_L2, TORCH_DT, bits16, check_codes, check_norms, outlier_kv, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.fail("these tests need a HIP device; there is no CPU fallback to test")
+
+
+def _orthogonal(d, seed):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    q, r = torch.linalg.qr(torch.randn(d, d, generator=g))
+    return (q * torch.sign(torch.diagonal(r))).contiguous()
+
+
+def _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, label, max_frac=2e-4):
+    dn = {torch.float32: "f32", torch.float16: "f16", torch.bfloat16: "bf16"}[x.dtype]
+    D = x.shape[-1]
+    out = comp.compress(x.to(DEV))
+    assert out["idx_bytes"].shape[-1] == D // (8 // bits) and out["idx_pad"] == 0
+    ref, _ = check_codes(oracle, out["idx_bytes"].cpu().numpy(), x.float().numpy().reshape(-1, D), Pi, cent, bits, label, max_frac)
+    check_norms(oracle, bits16(out["vec_norms"]), ref["vec_norms"], label)
+    # de-quantise the ORACLE's packed form, so that a code on the other side of a boundary does not enter
+    packed = {"idx_bytes": torch.from_numpy(ref["idx_bytes"].reshape(out["idx_bytes"].shape)).to(DEV),
+              "vec_norms": torch.from_numpy(ref["vec_norms"].view(np.int16).reshape(out["vec_norms"].shape)).view(torch.float16).to(DEV),
+              "shape": tuple(x.shape), "idx_pad": 0}
+    want = oracle.NumpyOracle(Pi, cent, bits).decompress(ref["idx_bytes"], ref["vec_norms"])
+    rec = comp.decompress(packed)
+    assert rec.dtype == torch.float32 and rec.shape == x.shape
+    err, _ = rel_l2(rec.cpu().numpy(), want)
+    print(f"[recon] {label}: relative L2 {err:.2e}")
+    assert err <= REL_L2, label
+    # 16-bit outputs: the fp32 result's own error plus roundings that fall the other way (one ulp: 2^-11 resp. 2^-8)
+    for odt, tol in ((torch.float16, 1.5e-3), (torch.bfloat16, 4e-3)):
+        o = torch.empty(x.shape, dtype=odt, device=DEV)
+        comp.decompress_into(packed, o)
+        want_t = torch.from_numpy(want).to(odt).float().numpy()
+        err, _ = rel_l2(o.float().cpu().numpy(), want_t)
+        assert err <= tol, (label, odt, err)
+    return out
+
+
+@pytest.mark.parametrize("D,bits", [(64, 2), (64, 4), (256, 2), (256, 4)])
+def test_reference_codebooks_and_rotation(pkg, oracle, golden, D, bits):
+    """The head dimensions the reference's own fixtures cover: its d=64 / d=256 codebooks, its d=64 rotation
+    (seed 42); the d=256 rotation comes from this package's generator, which the CPU suite pins to the reference's."""
+    cent = golden["codebooks"][f"centroids_d{D}_b{bits}"]
+    comp = pkg.MSECompressor(D, bits, seed=42, device=DEV)
+    Pi = comp.Pi.cpu().numpy()
+    if D == 64:      # (QR on another host's LAPACK differs in the last bits: compare loosely, then use the reference's matrix)
+        np.testing.assert_allclose(Pi, golden["rotations"]["Pi_d64_s42"], rtol=0, atol=2e-6)
+        Pi = golden["rotations"]["Pi_d64_s42"]
+    np.testing.assert_allclose(comp.centroids.cpu().numpy(), cent, rtol=0, atol=2e-6)
+    comp = pkg.MSECompressor.from_tensors(torch.from_numpy(Pi), torch.from_numpy(cent), bits, device=DEV)
+    for dn in ("f32", "f16", "bf16"):
+        x = outlier_kv((2, 3, 173, D), seed=100 + D + bits, dtype=TORCH_DT[dn])
+        _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, f"d{D} b{bits} {dn}")
+
+
+@pytest.mark.parametrize("D,bits", [(32, 1), (32, 8), (96, 3), (160, 5), (192, 6), (224, 4), (256, 8), (64, 7)])
+def test_other_dimensions_and_widths(pkg, oracle, D, bits):
+    """Every multiple of 32 up to 256, every packing (8, 4, 2 codes per byte, one code per byte), random orthogonal
+    rotation, this package's Lloyd-Max codebook for the dimension."""
+    Pi_t = _orthogonal(D, seed=7 * D + bits)
+    cent_t = pkg.LloydMaxCodebook(D, bits).centroids
+    comp = pkg.MSECompressor.from_tensors(Pi_t, cent_t, bits, device=DEV)
+    Pi, cent = Pi_t.numpy(), cent_t.numpy()
+    for dn, shape in (("f32", (1, 2, 211, D)), ("bf16", (3, 1, 129, D)), ("f16", (1, 1, 31, D))):
+        x = outlier_kv(shape, seed=D + bits, dtype=TORCH_DT[dn])
+        _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, f"d{D} b{bits} {dn}", max_frac=4e-4)
+
+
+def test_edge_inputs(pkg, oracle):
+    """Empty input, a single vector, the all-zero vector, a one-hot vector, a norm that overflows fp16."""
+    D, bits = 64, 4
+    comp = pkg.MSECompressor(D, bits, seed=42, device=DEV)
+    empty = comp.compress(torch.empty((1, 2, 0, D), device=DEV))
+    assert empty["idx_bytes"].shape == (1, 2, 0, D // 2) and empty["vec_norms"].shape == (1, 2, 0)
+    assert comp.decompress(empty).shape == (1, 2, 0, D)
+    x = torch.zeros((1, 1, 4, D))
+    x[0, 0, 1, 5] = 3.0
+    x[0, 0, 2] = torch.randn(D) * 3e4      # norm about 2.4e5: infinite in fp16
+    x[0, 0, 3] = torch.randn(D) * 1e-3
+    out = comp.compress(x.to(DEV))
+    ref = oracle.COracle(comp.Pi.cpu().numpy(), comp.centroids.cpu().numpy(), bits, accum_double=True).compress(x.numpy().reshape(-1, D))
+    check_norms(oracle, bits16(out["vec_norms"]), ref["vec_norms"], "edge")
+    rec = comp.decompress(out).cpu().numpy().reshape(-1, D)
+    assert not rec[0].any()                                   # zero vector -> exact zeros
+    assert np.isinf(out["vec_norms"].float().cpu().numpy().reshape(-1)[2]) and not np.isfinite(rec[2]).any()
+    want = oracle.NumpyOracle(comp.Pi.cpu().numpy(), comp.centroids.cpu().numpy(), bits).decompress(
+        out["idx_bytes"].cpu().numpy().reshape(-1, D // 2), bits16(out["vec_norms"]).reshape(-1))
+    for i in (1, 3):
+        assert np.linalg.norm(rec[i] - want[i]) <= REL_L2 * np.linalg.norm(want[i]), i
+    one = comp.compress(x[:, :, 1:2].to(DEV))
+    assert torch.equal(one["idx_bytes"], out["idx_bytes"][:, :, 1:2])
+
+
+def test_strided_store_and_batched_jobs(pkg, oracle):
+    """Token-axis slices of a preallocated [B,H,capacity,..] store, and a job list of several tensors in one launch,
+    give the bytes of plain calls."""
+    native = pkg._native
+    D, bits = 256, 2
+    comp = pkg.MSECompressor(D, bits, seed=3, device=DEV)
+    B, H, cap = 2, 2, 300
+    x = outlier_kv((B, H, 140, D), seed=5, dtype=torch.bfloat16).to(DEV)
+    plain = comp.compress(x)
+    idx = torch.zeros((B, H, cap, D // 4), dtype=torch.uint8, device=DEV)
+    nrm = torch.zeros((B, H, cap), dtype=torch.float16, device=DEV)
+    comp.compress_into(x[:, :, :100], idx[:, :, 7:107], nrm[:, :, 7:107])
+    comp.compress_into(x[:, :, 100:], idx[:, :, 107:147], nrm[:, :, 107:147])
+    assert torch.equal(idx[:, :, 7:147], plain["idx_bytes"]) and torch.equal(nrm[:, :, 7:147], plain["vec_norms"])
+    assert not idx[:, :, :7].any() and not idx[:, :, 147:].any()
+    full = torch.zeros((B, H, 200, D), dtype=torch.bfloat16, device=DEV)
+    comp.decompress_packed(idx[:, :, 7:147], nrm[:, :, 7:147], full[:, :, 20:160])
+    assert torch.equal(full[:, :, 20:160], comp.decompress_into(plain, torch.empty_like(x)))
+    assert not full[:, :, :20].any() and not full[:, :, 160:].any()
+
+    jobs = []
+    for k, tokens in enumerate((64, 1, 257)):
+        t = outlier_kv((1, 2, tokens, D), seed=20 + k, dtype=torch.bfloat16).to(DEV)
+        jobs.append({"states": t, "idx_bytes": torch.empty((1, 2, tokens, D // 4), dtype=torch.uint8, device=DEV),
+                     "vec_norms": torch.empty((1, 2, tokens), dtype=torch.float16, device=DEV), "table": comp.table(),
+                     "bits": bits, "out": torch.empty_like(t)})
+    native.JobList(jobs, torch.device(DEV)).compress()
+    native.JobList([dict(j, states=j["out"]) for j in jobs], torch.device(DEV)).decompress()
+    for j in jobs:
+        single = comp.compress(j["states"])
+        assert torch.equal(j["idx_bytes"], single["idx_bytes"]) and torch.equal(j["vec_norms"], single["vec_norms"])
+        assert torch.equal(j["out"], comp.decompress_into(single, torch.empty_like(j["states"])))
+    with pytest.raises(native.TqError):
+        native.JobList([jobs[0], dict(jobs[0], states=torch.empty((1, 2, 64, 128), dtype=torch.bfloat16, device=DEV))], torch.device(DEV))
+
+
+def test_v3_orchestration_and_cache_at_head_dim_64(pkg, oracle):
+    """TurboQuantV3 and the streaming cache at head_dim 64 (compress_kv / decompress_kv / update); the attention
+    kernels read 128-wide stores only and say so."""
+    D = 64
+    tq = pkg.TurboQuantV3(D, key_bits=4, value_bits=2, residual_window=0, layer_idx=5, n_layers=12, protected_layers=2, device=DEV)
+    k = outlier_kv((1, 2, 200, D), seed=1, dtype=torch.float16).to(DEV)
+    v = outlier_kv((1, 2, 200, D), seed=2, dtype=torch.float16).to(DEV)
+    ck, cv = tq.compress_kv(k, v)
+    dk, dv = tq.decompress_kv(ck, cv)
+    assert dk.shape == k.shape and dv.shape == v.shape
+    cos = torch.nn.functional.cosine_similarity(dk.float().flatten(), k.float().flatten(), dim=0)
+    assert cos > 0.99
+    cache = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=16, n_layers=12)
+    fk, fv = cache.update(k[:, :, :150], v[:, :, :150], 5)
+    for t in range(150, 160):
+        fk, fv = cache.update(k[:, :, t:t + 1], v[:, :, t:t + 1], 5)
+    assert fk.shape == (1, 2, 160, D)
+    assert torch.equal(fk[:, :, -16:], k[:, :, 144:160]) and torch.equal(fv[:, :, -16:], v[:, :, 144:160])
+    want = tq.key_compressor.decompress_into(tq.key_compressor.compress(k[:, :, :144]), torch.empty_like(k[:, :, :144]))
+    assert torch.equal(fk[:, :, :144], want)
+    with pytest.raises(pkg._native.TqError):
+        cache.attend(torch.randn((1, 4, 1, D), device=DEV, dtype=torch.float16), 5)

@@ -291,7 +291,10 @@ def test_c_abi_argument_errors(pkg):
     assert lib.tq_bytes_per_vector(128, 6) == 128 and lib.tq_bytes_per_vector(128, 1) == 16
     assert lib.tq_bytes_per_vector(6, 2) == 2
     assert lib.tq_bytes_per_vector(128, 0) == E["BITS"] and lib.tq_bytes_per_vector(128, 9) == E["BITS"]
-    assert lib.tq_table_bytes(64, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(128, 9) == E["BITS"]
+    # compress / decompress take every multiple of 32 up to 256
+    assert lib.tq_table_bytes(80, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(288, 4) == E["HEAD_DIM"]
+    assert lib.tq_table_bytes(0, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(128, 9) == E["BITS"]
+    assert 0 < lib.tq_table_bytes(64, 4) < lib.tq_table_bytes(128, 4) < lib.tq_table_bytes(256, 4)
     cent = np.array([0.1, -0.1], np.float32)
     thr = np.zeros(1, np.float32)
     assert lib.tq_decision_thresholds(cent.ctypes.data, 2, thr.ctypes.data) == E["CODEBOOK"]
@@ -313,7 +316,8 @@ def test_c_abi_argument_errors(pkg):
         states, dtype, kw.get("rows", 1), kw.get("tokens", 4), kw.get("rs", 0), kw.get("ts", 128), table, hd, bits,
         idx, norms, kw.get("prs", 0), None)
     assert call(p, 1, 0, 128) == E["BITS"]
-    assert call(p, 1, 4, 64) == E["HEAD_DIM"]
+    assert call(p, 1, 4, 80) == E["HEAD_DIM"]
+    assert call(p, 1, 4, 64, ts=48) == E["SIZE"]
     assert call(p, 7, 4, 128) == E["DTYPE"]
     assert call(None, 1, 4, 128) == E["NULL"]
     assert call(p + 2, 1, 4, 128) == E["ALIGN"]
@@ -427,3 +431,43 @@ def test_v3cache_refuses_cpu_tensors_and_reports_state(pkg):
         cache.update(torch.zeros(1, 1, 8, 128), torch.zeros(1, 1, 8, 128), 0)
     with pytest.raises(ValueError, match="nothing is cached"):
         pkg.V3Cache(key_bits=4, value_bits=2).attend(torch.zeros(1, 4, 1, 128), 0)
+
+
+def test_tables_for_other_head_dimensions(pkg):
+    """Tables for head dimensions other than 128: section sizes follow d (d/32 row tiles x d/16 steps of 1 KiB per
+    operand term), the operands hold Pi in the compress tiling for both directions, and the quantiser grid may use
+    all of its LDS budget (no shifted copies), which is what makes the dense 8-bit codebook of d = 256 fit."""
+    native = pkg._native
+    import ctypes
+
+    class Header(ctypes.Structure):
+        _fields_ = [(n, ctypes.c_uint32) for n in ("magic", "version", "head_dim", "bits", "levels", "ipb", "bytes_per_vec", "grid_cells")] + \
+                   [("grid_scale", ctypes.c_float), ("grid_bias", ctypes.c_float)] + \
+                   [(n, ctypes.c_uint32) for n in ("total_bytes", "off_a_f16", "off_a_bf16", "off_grid", "off_at_f16", "off_lut")]
+
+    for D, bits in ((64, 4), (256, 8), (96, 3)):
+        g = torch.Generator().manual_seed(D)
+        Pi, _ = torch.linalg.qr(torch.randn(D, D, generator=g))
+        cent = pkg.LloydMaxCodebook(D, bits).centroids
+        blob = native.build_table(Pi, cent, bits)
+        hd = Header.from_buffer_copy(blob[:ctypes.sizeof(Header)].tobytes())
+        operand = (D // 32) * (D // 16) * 1024
+        assert (hd.head_dim, hd.bits, hd.total_bytes) == (D, bits, blob.size)
+        assert hd.off_a_bf16 - hd.off_a_f16 == 2 * operand and hd.off_at_f16 - hd.off_a_bf16 == 3 * operand
+        assert hd.bytes_per_vec == D // (8 // bits) and hd.grid_cells * 8 <= 18432
+        # element (tile t, step s, lane l, i) of the leading bf16 term: Pi[32t + 16h + 4a + b][16s + 8hk + i], MFMA row m = 8a + 4h + b
+        a = blob[hd.off_a_bf16:hd.off_a_bf16 + operand].view(np.uint16).reshape(D // 32, D // 16, 64, 8)
+        pi = Pi.numpy()
+        for (t, s, l, i) in ((0, 0, 0, 0), (D // 32 - 1, D // 16 - 1, 63, 7), (1, 2, 37, 3)):
+            m, hk = l % 32, l // 32
+            row = 32 * t + 16 * ((m // 4) % 2) + 4 * (m // 8) + m % 4
+            want = torch.tensor(pi[row, 16 * s + 8 * hk + i]).to(torch.bfloat16).view(torch.int16).item() & 0xffff
+            assert a[t, s, l, i] == want, (D, t, s, l, i)
+        # decompress operand: Pi^T in the same tiling (out = column of Pi), leading fp16 term
+        at = blob[hd.off_at_f16:hd.off_at_f16 + operand].view(np.float16).reshape(D // 32, D // 16, 64, 8)
+        t, s, l, i = 1, 1, 40, 5
+        m, hk = l % 32, l // 32
+        col = 32 * t + 16 * ((m // 4) % 2) + 4 * (m // 8) + m % 4
+        assert at[t, s, l, i] == np.float16(pi[16 * s + 8 * hk + i, col])
+        assert native.lib().tq_table_check(blob.ctypes.data, blob.size, D, bits) == 0
+        assert native.lib().tq_table_check(blob.ctypes.data, blob.size, 128, bits) != 0

@@ -20,8 +20,8 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(CSRC, "libtqamd.so")
-SOURCES = ("tq_host.cpp", "tq_compress.hip", "tq_decompress.hip", "tq_attend.hip", "tq_qjl.hip")
-HEADERS = ("tq_table.h", "tq_device.h", os.path.join("..", "..", "include", "tqamd.h"))
+SOURCES = ("tq_host.cpp", "tq_compress.hip", "tq_decompress.hip", "tq_anydim.hip", "tq_attend.hip", "tq_qjl.hip")
+HEADERS = ("tq_table.h", "tq_device.h", "tq_anydim.h", os.path.join("..", "..", "include", "tqamd.h"))
 GPU_ARCH = "gfx950"
 
 TQ_F32, TQ_F16, TQ_BF16 = 0, 1, 2
@@ -670,9 +670,12 @@ class JobList:
         self.device = torch.device(device)
         self.host = (TqJob * self.n)()
         self._keep = []
+        self.head_dim = int(jobs[0]["states"].shape[-1])
         for i, j in enumerate(jobs):
             t = j["states"]
             _require_gpu(t, "states")
+            if t.shape[-1] != self.head_dim:
+                raise TqError(f"the jobs of one list share a head dimension: {t.shape[-1]} after {self.head_dim}")
             prs = packed_row_stride(j["idx_bytes"], j["vec_norms"])
             lay = None if prs is None else (row_layout(t) if prs else vector_layout(t))
             if lay is None:
@@ -692,13 +695,13 @@ class JobList:
 
     def compress(self) -> None:
         with _on(self.device):
-            rc = lib().tq_compress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, HEAD_DIM,
+            rc = lib().tq_compress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, self.head_dim,
                                            _stream_handle(self.device))
         check(rc, "tq_compress_batched")
 
     def decompress(self) -> None:
         with _on(self.device):
-            rc = lib().tq_decompress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, HEAD_DIM,
+            rc = lib().tq_decompress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, self.head_dim,
                                              self.workspace.data_ptr(), _stream_handle(self.device))
         if rc:
             self.workspace.zero_()      # counters of a launch that did not complete are not trusted

@@ -25,6 +25,7 @@
 #include <mutex>
 #include <type_traits>
 
+#include "tq_anydim.h"
 #include "tq_device.h"
 
 namespace {
@@ -47,56 +48,6 @@ template <> struct InTraits<TQ_F32> { static constexpr int ELEM = 4, TERMS = 3, 
 
 constexpr int CWAVES = TQ_TILES;        // waves per block = MFMA row tiles
 constexpr int CTHREADS = CWAVES * TQ_WAVE;
-
-__device__ __forceinline__ tq_f16v mfma_f16(tq_u4 a, tq_u4 b, tq_f16v c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, a), __builtin_bit_cast(tq_half8, b), c, 0, 0, 0);
-}
-__device__ __forceinline__ tq_f16v mfma_bf16(tq_u4 a, tq_u4 b, tq_f16v c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(tq_bf8, a), __builtin_bit_cast(tq_bf8, b), c, 0, 0, 0);
-}
-
-// sum of squares of the eight 16-bit values in v, added to acc (fp32).
-// (Pairs are taken from the whole-vector cast: casting one 32-bit element of `v` to a 16-bit
-// pair made the compiler read element 0 four times.)
-template <int DTYPE>
-__device__ __forceinline__ float sumsq8(tq_u4 v, float acc) {
-    if constexpr (DTYPE == TQ_F16) {
-        const tq_half8 h8 = __builtin_bit_cast(tq_half8, v);
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const tq_half2 h = {h8[2 * d], h8[2 * d + 1]};
-            acc = __builtin_amdgcn_fdot2(h, h, acc, false);
-        }
-    } else {
-        const tq_bf8 b8 = __builtin_bit_cast(tq_bf8, v);
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const tq_bf2 b = {b8[2 * d], b8[2 * d + 1]};
-            acc = __builtin_amdgcn_fdot2_f32_bf16(b, b, acc, false);
-        }
-    }
-    return acc;
-}
-
-// Exact split of eight floats into three bf16 terms each (x = t0 + t1 + t2, every term a
-// truncation, every remainder exact in fp32).  Output: packed bf16 operands.
-__device__ __forceinline__ void split_f32x8(const float (&x)[8], tq_u4 &t0, tq_u4 &t1, tq_u4 &t2) {
-    uint32_t a[8], b[8], c[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t xa = __float_as_uint(x[i]) & 0xffff0000u;
-        const float r1 = x[i] - __uint_as_float(xa);
-        const uint32_t xb = __float_as_uint(r1) & 0xffff0000u;
-        const float r2 = r1 - __uint_as_float(xb);
-        a[i] = xa; b[i] = xb; c[i] = __float_as_uint(r2) & 0xffff0000u;
-    }
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        t0[d] = (a[2 * d] >> 16) | a[2 * d + 1];
-        t1[d] = (b[2 * d] >> 16) | b[2 * d + 1];
-        t2[d] = (c[2 * d] >> 16) | c[2 * d + 1];
-    }
-}
 
 // ---- packing geometry -------------------------------------------------------------------
 // A lane owns 16 consecutive codes = NB packed bytes, handled as NW words of WB bytes (a full
@@ -295,16 +246,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     struct Scale { float nrm, inv, inv_cell; };
     auto scale_from_ss = [&](float ss) {
         Scale sc;
-        // sqrt: reciprocal square root plus one Newton step is correctly rounded except for a
-        // vanishing fraction of inputs.  Sums below 1e-35 (norm < 1e-17: it vanishes both in
-        // norm + 1e-8 and in fp16) count as zero; infinite and NaN sums pass through.
-        {
-            const float r = __builtin_amdgcn_rsqf(ss);
-            const float g = ss * r, h = 0.5f * r;
-            sc.nrm = fmaf(fmaf(-g, g, ss), h, g);
-            sc.nrm = ss < 1e-35f ? 0.f : sc.nrm;
-            sc.nrm = ss < __builtin_inff() ? sc.nrm : ss;
-        }
+        sc.nrm = tq_norm_from_sumsq(ss);
         // 1 / (norm + 1e-8): the reciprocal only scales the coordinates, one ulp is irrelevant
         sc.inv = __builtin_amdgcn_rcpf(sc.nrm + 1e-8f);
         if (DTYPE == TQ_F16) sc.inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
@@ -708,7 +650,7 @@ int check_job(const void *states, int dtype, long long rows, long long tokens, l
               long long token_stride, const void *table, int head_dim, int bits, const void *idx_bytes,
               const void *vec_norms, long long packed_row_stride, long long *n_vec) {
     if (bits < 1 || bits > 8) return TQ_ERR_BITS;
-    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
+    if (head_dim != TQ_HEAD_DIM && !tq_anydim_supported(head_dim)) return TQ_ERR_HEAD_DIM;
     const int eb = elem_bytes(dtype);
     if (!eb) return TQ_ERR_DTYPE;
     if (rows < 0 || tokens < 0) return TQ_ERR_SIZE;
@@ -716,7 +658,7 @@ int check_job(const void *states, int dtype, long long rows, long long tokens, l
     *n_vec = rows * tokens;
     if (*n_vec == 0) return TQ_OK;
     if (!states || !table || !idx_bytes || !vec_norms) return TQ_ERR_NULL;
-    if (token_stride < TQ_HEAD_DIM && tokens > 1) return TQ_ERR_SIZE;
+    if (token_stride < head_dim && tokens > 1) return TQ_ERR_SIZE;
     if (rows > 1 && row_stride < 0) return TQ_ERR_SIZE;
     if (packed_row_stride != 0 && (packed_row_stride < tokens || packed_row_stride > (long long)0x7fffffff / rows)) return TQ_ERR_SIZE;
     if (((uintptr_t)states & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & 15u) || ((uintptr_t)vec_norms & 1u))
@@ -745,6 +687,8 @@ extern "C" int tq_compress(const void *states, int dtype, long long rows, long l
     job.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     job.row_stride = row_stride * elem_bytes(dtype);
     job.token_stride = token_stride * elem_bytes(dtype);
+    if (head_dim != TQ_HEAD_DIM)
+        return tq_anydim_compress(dtype, bits, head_dim, job, nullptr, 1, (uint32_t)n_vec, static_cast<hipStream_t>(stream));
     return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), static_cast<hipStream_t>(stream));
 }
 
@@ -766,6 +710,9 @@ extern "C" int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_d
     }
     if (max_vec == 0) return TQ_OK;
     TqDevJob none{};
+    if (head_dim != TQ_HEAD_DIM)
+        return tq_anydim_compress(jobs_host[0].dtype, jobs_host[0].bits, head_dim, none, jobs_dev, n_jobs, (uint32_t)max_vec,
+                                  static_cast<hipStream_t>(stream));
     return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec + 31) / 32),
                     static_cast<hipStream_t>(stream));
 }

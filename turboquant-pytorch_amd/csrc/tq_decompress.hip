@@ -24,6 +24,7 @@
 #include <mutex>
 #include <type_traits>
 
+#include "tq_anydim.h"
 #include "tq_device.h"
 
 // Ticket counters of tq_decompress_batched_noalloc: the workspace that tq_decompress_batched takes from its
@@ -410,7 +411,7 @@ int check_job(const void *out, int dtype, long long rows, long long tokens, long
               long long token_stride, const void *table, int head_dim, int bits, const void *idx_bytes,
               const void *vec_norms, long long packed_row_stride, long long *n_vec) {
     if (bits < 1 || bits > 8) return TQ_ERR_BITS;
-    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
+    if (head_dim != TQ_HEAD_DIM && !tq_anydim_supported(head_dim)) return TQ_ERR_HEAD_DIM;
     const int eb = elem_bytes(dtype);
     if (!eb) return TQ_ERR_DTYPE;
     if (rows < 0 || tokens < 0) return TQ_ERR_SIZE;
@@ -418,7 +419,7 @@ int check_job(const void *out, int dtype, long long rows, long long tokens, long
     *n_vec = rows * tokens;
     if (*n_vec == 0) return TQ_OK;
     if (!out || !table || !idx_bytes || !vec_norms) return TQ_ERR_NULL;
-    if (token_stride < TQ_HEAD_DIM && tokens > 1) return TQ_ERR_SIZE;
+    if (token_stride < head_dim && tokens > 1) return TQ_ERR_SIZE;
     if (rows > 1 && row_stride < 0) return TQ_ERR_SIZE;
     if (packed_row_stride != 0 && (packed_row_stride < tokens || packed_row_stride > (long long)0x7fffffff / rows)) return TQ_ERR_SIZE;
     if (((uintptr_t)out & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & 15u) || ((uintptr_t)vec_norms & 1u))
@@ -449,6 +450,8 @@ extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms
     job.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     job.row_stride = row_stride * elem_bytes(out_dtype);
     job.token_stride = token_stride * elem_bytes(out_dtype);
+    if (head_dim != TQ_HEAD_DIM)     // the run-time-dimension kernel assigns its tiles statically: no counters
+        return tq_anydim_decompress(out_dtype, bits, head_dim, job, nullptr, 1, (uint32_t)n_vec, static_cast<hipStream_t>(stream));
     return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), workspace, static_cast<hipStream_t>(stream));
 }
 
@@ -474,6 +477,9 @@ int decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jo
     }
     if (max_vec == 0) return TQ_OK;
     TqDevJob none{};
+    if (head_dim != TQ_HEAD_DIM)
+        return tq_anydim_decompress(jobs_host[0].dtype, jobs_host[0].bits, head_dim, none, jobs_dev, n_jobs, (uint32_t)max_vec,
+                                    static_cast<hipStream_t>(stream));
     return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec + 31) / 32),
                     workspace, static_cast<hipStream_t>(stream));
 }

@@ -125,6 +125,68 @@ __device__ __forceinline__ tq_f16v tq_zero16() {
     return z;
 }
 
+// ---- matrix-core and input helpers of the compress-side kernels -----------------------------------
+static __device__ __forceinline__ tq_f16v mfma_f16(tq_u4 a, tq_u4 b, tq_f16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, a), __builtin_bit_cast(tq_half8, b), c, 0, 0, 0);
+}
+static __device__ __forceinline__ tq_f16v mfma_bf16(tq_u4 a, tq_u4 b, tq_f16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(tq_bf8, a), __builtin_bit_cast(tq_bf8, b), c, 0, 0, 0);
+}
+
+// sum of squares of the eight 16-bit values in v, added to acc (fp32).
+// (Pairs are taken from the whole-vector cast: casting one 32-bit element of `v` to a 16-bit
+// pair made the compiler read element 0 four times.)
+template <int DTYPE>
+static __device__ __forceinline__ float sumsq8(tq_u4 v, float acc) {
+    if constexpr (DTYPE == TQ_F16) {
+        const tq_half8 h8 = __builtin_bit_cast(tq_half8, v);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const tq_half2 h = {h8[2 * d], h8[2 * d + 1]};
+            acc = __builtin_amdgcn_fdot2(h, h, acc, false);
+        }
+    } else {
+        const tq_bf8 b8 = __builtin_bit_cast(tq_bf8, v);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const tq_bf2 b = {b8[2 * d], b8[2 * d + 1]};
+            acc = __builtin_amdgcn_fdot2_f32_bf16(b, b, acc, false);
+        }
+    }
+    return acc;
+}
+
+// Exact split of eight floats into three bf16 terms each (x = t0 + t1 + t2, every term a
+// truncation, every remainder exact in fp32).  Output: packed bf16 operands.
+static __device__ __forceinline__ void split_f32x8(const float (&x)[8], tq_u4 &t0, tq_u4 &t1, tq_u4 &t2) {
+    uint32_t a[8], b[8], c[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t xa = __float_as_uint(x[i]) & 0xffff0000u;
+        const float r1 = x[i] - __uint_as_float(xa);
+        const uint32_t xb = __float_as_uint(r1) & 0xffff0000u;
+        const float r2 = r1 - __uint_as_float(xb);
+        a[i] = xa; b[i] = xb; c[i] = __float_as_uint(r2) & 0xffff0000u;
+    }
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        t0[d] = (a[2 * d] >> 16) | a[2 * d + 1];
+        t1[d] = (b[2 * d] >> 16) | b[2 * d + 1];
+        t2[d] = (c[2 * d] >> 16) | c[2 * d + 1];
+    }
+}
+
+// Norm of a vector from the fp32 sum of its squares.  Reciprocal square root plus one Newton step is correctly
+// rounded except for a vanishing fraction of inputs.  Sums below 1e-35 (norm < 1e-17: it vanishes both in
+// norm + 1e-8 and in fp16) count as zero; infinite and NaN sums pass through.
+static __device__ __forceinline__ float tq_norm_from_sumsq(float ss) {
+    const float r = __builtin_amdgcn_rsqf(ss);
+    const float g = ss * r, h = 0.5f * r;
+    float nrm = fmaf(fmaf(-g, g, ss), h, g);
+    nrm = ss < 1e-35f ? 0.f : nrm;
+    return ss < __builtin_inff() ? nrm : ss;
+}
+
 // Decode the eight codes of MFMA step s held by this lane (codes 64*hk + 8*s .. + 7 of its vector)
 // into a packed fp16x8 operand, through the byte -> centroids table `lut` in LDS.
 // raw[] holds the lane's 64/IPB packed bytes, little-endian dwords.

@@ -97,13 +97,17 @@ struct Layout {
     uint32_t off_a_f16, off_a_bf16, off_grid, off_at_f16, off_lut, off_centroids, off_thresholds, total;
     uint32_t lut_entry_bytes;
 };
-Layout layout_for(int bits) {
+// head dimensions the kernels take: 128 (the tuned kernels) and the other multiples of 32 up to 256
+bool supported_head_dim(int d) { return d >= TQ_ANYDIM_MIN && d <= TQ_ANYDIM_MAX && d % 32 == 0; }
+
+Layout layout_for(int head_dim, int bits) {
     const uint32_t levels = 1u << bits, ipb = 8u / (uint32_t)bits;
+    const uint32_t operand = (uint32_t)TQ_OPERAND_BYTES_FOR(head_dim);
     Layout L{};
     uint32_t off = sizeof(TqTableHeader);
-    L.off_a_f16 = off;      off += 2 * TQ_OPERAND_BYTES;
-    L.off_a_bf16 = off;     off += 3 * TQ_OPERAND_BYTES;
-    L.off_at_f16 = off;     off += 2 * TQ_OPERAND_BYTES;
+    L.off_a_f16 = off;      off += 2 * operand;
+    L.off_a_bf16 = off;     off += 3 * operand;
+    L.off_at_f16 = off;     off += 2 * operand;
     L.off_grid = off;       off += round_up(TQ_GRID_LDS_BYTES, 256);
     L.lut_entry_bytes = 2 * ipb;
     L.off_lut = off;        off += round_up(256 * L.lut_entry_bytes, 256);
@@ -124,7 +128,7 @@ const char *tq_status_string(int status) {
         case TQ_OK: return "ok";
         case TQ_ERR_NULL: return "null pointer argument";
         case TQ_ERR_BITS: return "bits must be in 1..8";
-        case TQ_ERR_HEAD_DIM: return "unsupported head_dim (the gfx950 kernels handle 128)";
+        case TQ_ERR_HEAD_DIM: return "unsupported head_dim (compress / decompress: multiples of 32 up to 256; the other kernels: 128)";
         case TQ_ERR_DTYPE: return "unknown element type";
         case TQ_ERR_SIZE: return "invalid size or stride";
         case TQ_ERR_CODEBOOK: return "centroids must be finite and strictly ascending";
@@ -164,19 +168,20 @@ int tq_decision_thresholds(const float *centroids, int levels, float *thresholds
 
 long long tq_table_bytes(int head_dim, int bits) {
     if (bits < 1 || bits > 8) return TQ_ERR_BITS;
-    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
-    return layout_for(bits).total;
+    if (!supported_head_dim(head_dim)) return TQ_ERR_HEAD_DIM;
+    return layout_for(head_dim, bits).total;
 }
 
 int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bits,
                    void *table_host, size_t table_bytes) {
     if (!Pi || !centroids || !table_host) return TQ_ERR_NULL;
     if (bits < 1 || bits > 8) return TQ_ERR_BITS;
-    if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
-    const Layout L = layout_for(bits);
+    if (!supported_head_dim(head_dim)) return TQ_ERR_HEAD_DIM;
+    const Layout L = layout_for(head_dim, bits);
     if (table_bytes < L.total) return TQ_ERR_SIZE;
     const int levels = 1 << bits;
-    const int D = TQ_HEAD_DIM;
+    const int D = head_dim;
+    const bool tuned = D == TQ_HEAD_DIM;   // the 128-wide kernels have their own decompress tiling and keep shifted grid copies
     if (!valid_codebook(centroids, levels)) return TQ_ERR_CODEBOOK;
     for (int i = 0; i < D * D; ++i)
         if (!std::isfinite(Pi[i])) return TQ_ERR_SIZE;
@@ -205,7 +210,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     for (int lg = 3; lg <= 12 && !ok; ++lg) {
         scale = (float)(1 << lg);
         cells = 2u * (uint32_t)std::ceil(range * scale);
-        if (cells > (uint32_t)TQ_GRID_MAX_CELLS(bits)) break;
+        if (cells > (uint32_t)(tuned ? TQ_GRID_MAX_CELLS(bits) : TQ_GRID_LDS_BYTES / 8)) break;
         bias = (float)(cells / 2) + TQ_GRID_MAGIC;
         grid.assign(cells, TqGridCell{INFINITY, 0});
         auto edge = [&](uint32_t k) { return ((double)k - (double)(cells / 2) - 0.0625) / (double)scale; };
@@ -225,20 +230,21 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     std::memcpy(blob + L.off_grid, grid.data(), (size_t)cells * sizeof(TqGridCell));
 
     // ---- rotation operands ----
-    auto operand_index = [](int t, int s, int l, int i) { return (((size_t)t * TQ_STEPS + s) * 64 + l) * 8 + i; };
+    const int tiles = D / 32, steps = D / 16;
+    auto operand_index = [steps](int t, int s, int l, int i) { return (((size_t)t * steps + s) * 64 + l) * 8 + i; };
     uint16_t *a_f16 = reinterpret_cast<uint16_t *>(blob + L.off_a_f16);
     uint16_t *a_bf16 = reinterpret_cast<uint16_t *>(blob + L.off_a_bf16);
     uint16_t *at_f16 = reinterpret_cast<uint16_t *>(blob + L.off_at_f16);
-    const size_t term = TQ_OPERAND_BYTES / 2;  // halves per operand set
+    const size_t term = (size_t)TQ_OPERAND_BYTES_FOR(D) / 2;  // halves per operand set
     const double pi_scale = (double)(1 << TQ_F16_PI_SHIFT);
-    for (int t = 0; t < TQ_TILES; ++t)
-        for (int s = 0; s < TQ_STEPS; ++s)
+    for (int t = 0; t < tiles; ++t)
+        for (int s = 0; s < steps; ++s)
             for (int l = 0; l < 64; ++l) {
                 const int m = l % 32, hk = l / 32;
                 // MFMA row m = 8a + 4h + b  <->  accumulator register r = 4a + b of lane-half h
                 const int a = m / 8, h = (m / 4) % 2, b = m % 4;
                 const int out_c = 32 * t + 16 * h + 4 * a + b;                        // compress (see tq_table.h)
-                const int out_d = 64 * h + 16 * t + 4 * a + b;                        // decompress
+                const int out_d = tuned ? 64 * h + 16 * t + 4 * a + b : out_c;        // decompress
                 for (int i = 0; i < 8; ++i) {
                     const size_t o = operand_index(t, s, l, i);
                     {   // compress: rotated[out] = sum_k x[k] * Pi[out][k],  k = 16s + 8hk + i
@@ -258,7 +264,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
                         a_bf16[2 * term + o] = to_bf16(r2);
                     }
                     {   // decompress: x[out] = sum_j y[j] * Pi[j][out],  j = 64hk + 8s + i
-                        const int j = 64 * hk + 8 * s + i;
+                        const int j = tuned ? 64 * hk + 8 * s + i : 16 * s + 8 * hk + i;
                         const float p = Pi[j * D + out_d];
                         const uint16_t hi = to_f16(p);
                         at_f16[o] = hi;

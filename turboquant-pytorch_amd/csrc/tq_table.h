@@ -29,6 +29,14 @@
 #define TQ_STEPS 8  /* 128 inputs  / 16 deep  */
 #define TQ_OPERAND_BYTES (TQ_TILES * TQ_STEPS * 64 * 16) /* one 128x128 16-bit operand set: 32 KiB */
 
+// Other head dimensions (multiples of 32 from TQ_ANYDIM_MIN to TQ_ANYDIM_MAX) go through one pair of kernels that
+// takes the dimension at run time.  Their tables hold d/32 row tiles x d/16 steps per operand set, compress AND
+// decompress operands in the compress tiling above (out = 32t + 16h + r, in = 16s + 8hk + i), and a quantiser grid
+// of up to TQ_GRID_LDS_BYTES / 8 cells whatever the width (those kernels keep a single, unshifted copy).
+#define TQ_ANYDIM_MIN 32
+#define TQ_ANYDIM_MAX 256
+#define TQ_OPERAND_BYTES_FOR(d) (((d) / 32) * ((d) / 16) * 64 * 16)
+
 // The fp16 split of Pi is stored multiplied by 2^TQ_F16_PI_SHIFT so that the low term stays
 // in the fp16 normal range; the kernels fold 2^-shift into the per-vector scale.
 #define TQ_F16_PI_SHIFT 10

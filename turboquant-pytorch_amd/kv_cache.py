@@ -119,7 +119,8 @@ class _LayerStore:
         into the next packed slot and the new token takes the next window slot.  False (nothing done) when the
         step is not of that kind or the tensors are not laid out for it; the general path then runs."""
         rw = self.window_tokens
-        if (rw == 0 or self.n_recent != rw or self.w0 + rw + 1 > self.win_cap or self.n_compressed + 1 > self.capacity
+        if (rw == 0 or self.D != _native.HEAD_DIM      # (the one-call step exists for the 128-wide kernels only)
+                or self.n_recent != rw or self.w0 + rw + 1 > self.win_cap or self.n_compressed + 1 > self.capacity
                 or keys.dtype != self.dtype or values.dtype != self.dtype or keys.device != self.device
                 or values.device != self.device or torch.compiler.is_compiling()):
             return False
