@@ -139,7 +139,10 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     // (fp32 inputs sum their squares while they walk the steps, every wave over the whole vector: same order in all waves)
     const uint32_t step0 = ELEM == 2 ? 2u * wave : 0u;
     tq_u4 areg[T::TERMS][TQ_STEPS];
-    {
+    // Rotation operands into registers and the quantiser grid into LDS (one copy per code position, base pre-shifted).
+    // Every cell is fetched once and written to all its copies; the fetches of a thread are issued together.
+    // Called once per block: behind the first tile loads on the pipelined path, so that their latencies overlap.
+    auto load_tables = [&]() {
         const uint8_t *src = job.table + (DTYPE == TQ_F16 ? hd->off_a_f16 : hd->off_a_bf16);
 #pragma unroll
         for (int term = 0; term < T::TERMS; ++term)
@@ -147,17 +150,27 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             for (int s = 0; s < TQ_STEPS; ++s)
                 areg[term][s] = tq_gload16(src + (size_t)term * TQ_OPERAND_BYTES +
                                            (((size_t)wave * TQ_STEPS + ((s + step0) & 7u)) * 64 + lane) * 16);
-    }
-    {   // one grid copy per code position, base pre-shifted
+        constexpr int CELL_TRIPS = (TQ_GRID_MAX_CELLS(BITS) + CTHREADS - 1) / CTHREADS;
         const uint32_t cells = hd->grid_cells;
-        const uint8_t *src = job.table + hd->off_grid;
-        for (uint32_t i = tid; i < cells * P::COPIES; i += CTHREADS) {
-            const uint32_t c = i / cells, q = i - c * cells;
-            tq_u2 e = tq_gload8(src + 8u * q);
-            e[1] <<= copy_shift_rt<BITS>(c);
-            *reinterpret_cast<tq_u2 *>(lds_grid + c * P::COPY_STRIDE + 8u * q) = e;
+        const uint8_t *gsrc = job.table + hd->off_grid;
+        tq_u2 cell[CELL_TRIPS];
+#pragma unroll
+        for (int k = 0; k < CELL_TRIPS; ++k) {
+            const uint32_t q = tid + k * CTHREADS;
+            cell[k] = tq_gload8(gsrc + 8u * (q < cells ? q : 0u));
         }
-    }
+#pragma unroll
+        for (int k = 0; k < CELL_TRIPS; ++k) {
+            const uint32_t q = tid + k * CTHREADS;
+            if (q < cells) {
+#pragma unroll
+                for (int c = 0; c < P::COPIES; ++c) {
+                    const tq_u2 e = {cell[k][0], cell[k][1] << copy_shift_rt<BITS>(c)};
+                    *reinterpret_cast<tq_u2 *>(lds_grid + c * P::COPY_STRIDE + 8u * q) = e;
+                }
+            }
+        }
+    };
     const float grid_scale = hd->grid_scale, grid_bias = hd->grid_bias;
 
     const uint32_t ld_vec = lane / PIECES, ld_piece = lane % PIECES;  // role in the coalesced loads
@@ -344,7 +357,9 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     float nrm;
     // the pipelined path addresses a tile's vectors with 32-bit offsets from a scalar base
     const bool dma_ok = one_row && job.token_stride < (1ll << 26);
-    if (tile < n_full && ELEM == 2 && dma_ok) {
+    const bool pipelined = tile < n_full && ELEM == 2 && dma_ok;
+    if (!pipelined) load_tables();
+    if (pipelined) {
         if constexpr (ELEM == 2) {
             // Single-row jobs with 16-bit elements (the KV-cache case): a software pipeline over this block's full
             // tiles t_0 .. t_{m-1}.  Tiles travel from memory straight into a ring of RING LDS slots
@@ -509,6 +524,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
 
 #pragma unroll
             for (int p = 0; p < P - 1; ++p) issue((uint32_t)p);
+            load_tables();      // (the waits for these loads also cover the older tile loads: harmless, once per block)
             tq_f16v acc_a, acc_b;
             uint32_t done = 0;     // iterations finished
             iteration(std::false_type{}, std::integral_constant<uint32_t, 0>{}, false, 0u, acc_a, acc_a);
