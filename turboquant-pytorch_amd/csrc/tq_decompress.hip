@@ -13,7 +13,8 @@
 // instruction writes 1 KiB of consecutive memory.
 //
 // Which tiles a block works on.  A block draws "tickets": one ticket = WAVES consecutive tiles,
-// one per wave.  With a workspace the tickets of a job come from a counter in device memory
+// one per wave.  A block's first ticket is fixed (block b: tiles b * WAVES ...), so its loads start before the tables
+// are staged; with a workspace the later tickets of a job come from a counter in device memory
 // (atomicAdd), so the blocks walk through the job in the order in which they become free and the
 // addresses being written at any moment stay within a few MiB of each other; on this part that
 // write pattern reaches 10-15 % more bandwidth than a fixed assignment (block b takes tickets
@@ -80,27 +81,40 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     uint8_t *lds_lut = lds + TQ_OPERAND_BYTES;
     uint8_t *stage = lds_lut + LUT_LDS_BYTES + wave * STAGE;
 
-    tq_copy_to_lds(lds_a, job.table + hd->off_at_f16, TQ_OPERAND_BYTES, tid, T::WAVES * TQ_WAVE);
-    tq_copy_to_lds(lds_lut, job.table + hd->off_lut, 256u * 2u * IPB, tid, T::WAVES * TQ_WAVE);
-
-    // tickets: counter[0] = next tile to hand out, counter[1] = blocks of this job that are done
+    // tickets: counter[0] = tiles handed out beyond every block's first ticket, counter[1] = blocks of this job that are done.
+    // The first ticket of a block is fixed (block b: tiles b * WAVES ...), so its loads can start before anything else.
     __shared__ uint32_t tk[3];         // ticket k of the block sits in slot k % 3
     uint32_t *counter = workspace ? workspace + blockIdx.y * (TQ_WORKSPACE_BYTES_PER_JOB / 4) : nullptr;
-    uint32_t fixed_next = blockIdx.x * T::WAVES;
+    const uint32_t first = blockIdx.x * T::WAVES;
+    const uint32_t drawn_origin = gridDim.x * T::WAVES;
+    uint32_t fixed_next = first + drawn_origin;
     auto draw = [&]() -> uint32_t {     // thread 0 only
-        if (counter) return atomicAdd(counter, (uint32_t)T::WAVES);
+        if (counter) {
+            const uint32_t t = drawn_origin + atomicAdd(counter, (uint32_t)T::WAVES);
+            return t < n_tiles ? t : n_tiles;
+        }
         const uint32_t t = fixed_next < n_tiles ? fixed_next : n_tiles;   // saturates: no wrap-around on huge grids
-        fixed_next = t + gridDim.x * T::WAVES;
+        fixed_next = t + drawn_origin;
         return t;
     };
-    if (tid == 0) {
-        const uint32_t t0 = draw(), t1 = draw();
-        tk[0] = t0;
-        tk[1] = t1;
-    }
-    __syncthreads();
+    // Everything a block needs besides its first tile: Pi^T and the byte -> centroids table into LDS (all fetches
+    // of a thread issued together), the second ticket, one barrier.  Called behind the first tile's loads.
+    auto stage_tables = [&]() {
+        constexpr int NT = T::WAVES * TQ_WAVE;
+        constexpr int A_TRIPS = TQ_OPERAND_BYTES / 16 / NT;
+        static_assert(A_TRIPS * NT * 16 == TQ_OPERAND_BYTES, "whole trips");
+        const uint8_t *a_src = job.table + hd->off_at_f16;
+        tq_u4 v[A_TRIPS];
+#pragma unroll
+        for (int k = 0; k < A_TRIPS; ++k) v[k] = tq_gload16(a_src + 16u * (tid + k * NT));
+        if (tid == 0) tk[1] = draw();
+#pragma unroll
+        for (int k = 0; k < A_TRIPS; ++k) reinterpret_cast<tq_u4 *>(lds_a)[tid + k * NT] = v[k];
+        tq_copy_to_lds(lds_lut, job.table + hd->off_lut, 256u * 2u * IPB, tid, NT);
+        __syncthreads();
+    };
 
-    uint32_t base = tk[0];             // first tile of the block's current ticket (the same in every wave)
+    uint32_t base = first;             // first tile of the block's current ticket (the same in every wave)
     uint32_t tile = base + wave;
     const uint32_t n = lane & 31u, hk = lane >> 5;
     const uint32_t st_vec = lane / PIECES, st_piece = lane % PIECES;
@@ -250,8 +264,9 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     auto run = [&](auto fast_tag) {
         uint32_t cur[NW];
         float nrm = 0.f;
+        if (tile < n_full) issue_loads(std::true_type{}, fast_tag, tile);
+        stage_tables();
         if (tile < n_full) {
-            issue_loads(std::true_type{}, fast_tag, tile);
 #pragma unroll
             for (int i = 0; i < NW; ++i) cur[i] = raw[i];
             nrm = half_bits_to_float(norm_bits);
