@@ -40,6 +40,10 @@ namespace {
 #ifndef TQ_PIN_SCHEDULE
 #define TQ_PIN_SCHEDULE 1
 #endif
+// log2 of the iterations a block keeps one issue priority before it moves to the next (0: priorities stay untouched)
+#ifndef TQ_PRIO_SHIFT
+#define TQ_PRIO_SHIFT 3
+#endif
 template <int DTYPE> struct InTraits;
 template <> struct InTraits<TQ_F16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = TQ_C16_WAVES; };
 template <> struct InTraits<TQ_BF16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = TQ_C16_WAVES; };
@@ -531,9 +535,24 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             ++done;
             // unrolled by U = lcm(2 accumulator sets, P slots); iteration j runs variant j % U
             constexpr uint32_t U = (P % 2 == 0) ? P : 2 * P;
+            // The blocks that share a compute unit do not advance at the same pace: the instruction arbiter prefers the
+            // oldest wave, so the block dispatched first finishes its tiles well before the one dispatched last, and the
+            // unit then runs under-occupied until that one is done.  Every block therefore walks through the issue
+            // priorities 0 .. RES-1, a few iterations each, starting from its place in the dispatch order: over time each
+            // of the co-resident blocks is preferred equally often, and they finish together.
+            constexpr uint32_t RES = T::MIN_WAVES;
+            const uint32_t age = ((blockIdx.y * gridDim.x + blockIdx.x) * RES) / (gridDim.x * gridDim.y);
             auto step = [&](auto k_tag) -> bool {    // true = all tiles rotated
                 constexpr uint32_t K = decltype(k_tag)::value;
                 if (done == m) return true;
+                if constexpr (K == 0 && TQ_PRIO_SHIFT > 0) {
+                    if ((done & ((1u << TQ_PRIO_SHIFT) - 1u)) == 0u) {
+                        const uint32_t prio = (age + (done >> TQ_PRIO_SHIFT)) % RES;
+                        if (prio == 0u) __builtin_amdgcn_s_setprio(0);
+                        else if (prio == 1u) __builtin_amdgcn_s_setprio(1);
+                        else __builtin_amdgcn_s_setprio(2);
+                    }
+                }
                 if constexpr (K & 1u) iteration(std::true_type{}, std::integral_constant<uint32_t, K % P>{}, done >= (uint32_t)P, 1u, acc_b, acc_a);
                 else iteration(std::true_type{}, std::integral_constant<uint32_t, K % P>{}, done >= (uint32_t)P, 0u, acc_a, acc_b);
                 ++done;
