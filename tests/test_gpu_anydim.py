@@ -25,7 +25,7 @@ def _orthogonal(d, seed):
     return (q * torch.sign(torch.diagonal(r))).contiguous()
 
 
-def _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, label, max_frac=2e-4):
+def _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, label, max_frac=None):
     dn = {torch.float32: "f32", torch.float16: "f16", torch.bfloat16: "bf16"}[x.dtype]
     D = x.shape[-1]
     out = comp.compress(x.to(DEV))
@@ -79,7 +79,7 @@ def test_other_dimensions_and_widths(pkg, oracle, D, bits):
     Pi, cent = Pi_t.numpy(), cent_t.numpy()
     for dn, shape in (("f32", (1, 2, 211, D)), ("bf16", (3, 1, 129, D)), ("f16", (1, 1, 31, D))):
         x = outlier_kv(shape, seed=D + bits, dtype=TORCH_DT[dn])
-        _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, f"d{D} b{bits} {dn}", max_frac=4e-4)
+        _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, f"d{D} b{bits} {dn}", max_frac=2.5e-4 if bits > 4 else None)
 
 
 def test_edge_inputs(pkg, oracle):

@@ -49,8 +49,17 @@ def outlier_kv(shape, seed, dtype):
     return (x * ch * tok).to(dtype)
 
 
-def check_codes(oracle, got_bytes, x_f32, Pi, cent, bits, label, max_frac=2e-4):
+def allowed_code_fraction(bits):
+    """Share of coordinates that may carry the neighbouring code (all of them inside the boundary window, which is
+    checked separately).  Measured on the MI355X, worst case over the suite: bf16 inputs (two bf16 rotation terms,
+    2^-17) 15 ppm at 4 bits and below, 70 ppm at 8 bits on 33 million coordinates (101 ppm on one sample of 99 072);
+    fp16 and fp32 inputs 0-1 ppm.  The bounds leave a factor of about two."""
+    return 3e-5 if bits <= 4 else 1.5e-4
+
+
+def check_codes(oracle, got_bytes, x_f32, Pi, cent, bits, label, max_frac=None):
     """Compare packed bytes with the oracle (double-accumulating C restatement).  Returns the report."""
+    max_frac = allowed_code_fraction(bits) if max_frac is None else max_frac
     orc = oracle.COracle(Pi, cent, bits, accum_double=True)
     ref = orc.compress(x_f32)
     got = got_bytes.reshape(-1, got_bytes.shape[-1])
@@ -591,7 +600,7 @@ def test_config4_shape_llama_32k(pkg, oracle):
             # bf16 inputs meet the rotation as two bf16 terms (2^-17): a few hundred coordinates per million sit
             # within 1e-6 of a boundary at 8 bits, where boundaries are densest; all inside the 1e-5 window
             ref, _ = check_codes(oracle, c["compressed"]["idx_bytes"].cpu().numpy(), x.float().numpy().reshape(-1, 128), Pi, cent,
-                                 comp.bits, f"config 4 layer {layer} {name}", max_frac=6e-4 if comp.bits == 8 else 2e-4)
+                                 comp.bits, f"config 4 layer {layer} {name}")
             check_norms(oracle, bits16(c["compressed"]["vec_norms"]), ref["vec_norms"], f"config 4 layer {layer} {name}")
             want = oracle.COracle(Pi, cent, comp.bits, True).decompress(ref["idx_bytes"], ref["vec_norms"])
             err, _ = rel_l2(rec.float().cpu().numpy().reshape(-1, 128), want)

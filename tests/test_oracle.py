@@ -314,3 +314,24 @@ def test_v2_qjl_oracle_against_reference_vectors(oracle):
     assert seen == 12
     s = np.array([[1, -1, -1, -1, -1, -1, -1, 1] + [1] * 8])
     assert oracle.pack_signs(s).tolist() == [[0x81, 0xFF]]
+
+
+def test_c_oracle_under_sanitizers(tmp_path):
+    """tq_oracle.c built with AddressSanitizer and UndefinedBehaviorSanitizer (host code only) and driven over ragged
+    sizes, every bit width, both accumulation modes and every fp16 bit pattern: no out-of-bounds access, no overflowed
+    shift, no misaligned read in the checker itself."""
+    import os
+    import shutil
+    import subprocess
+    ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc on this machine")
+    src = os.path.join(ROOT, "oracle", "tq_oracle_sanitize.c")
+    exe = str(tmp_path / "tq_oracle_sanitize")
+    build = subprocess.run([gcc, "-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined",
+                            "-fno-sanitize-recover=all", "-static-libasan", "-o", exe, src, "-lm"],
+                           capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0 and run.stdout.strip() == "ok", run.stdout + run.stderr
