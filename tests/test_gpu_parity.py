@@ -674,3 +674,22 @@ def test_operators_trace_under_a_compiler(pkg):
     compiled = torch.compile(round_trip, backend="aot_eager", fullgraph=True)(x)
     for a, b in zip(eager, compiled):
         assert torch.equal(a, b)
+
+
+def test_compressor_on_the_cpu_follows_the_tensors(pkg):
+    """A compressor built with the reference's default device ("cpu") works on HIP tensors: tables and rotation copies
+    are uploaded per device; results equal those of a compressor built on the device; CPU tensors are refused."""
+    host = pkg.MSECompressor(128, 4, seed=9)
+    dev = pkg.MSECompressor(128, 4, seed=9, device=DEV)
+    x = outlier_kv((1, 2, 77, 128), seed=3, dtype=torch.float16).to(DEV)
+    a, b = host.compress(x), dev.compress(x)
+    assert torch.equal(a["idx_bytes"], b["idx_bytes"]) and torch.equal(a["vec_norms"], b["vec_norms"])
+    assert torch.equal(host.decompress(a), dev.decompress(b))
+    q = torch.randn((1, 4, 1, 128), device=DEV)
+    assert torch.equal(host.packed_scores(a["idx_bytes"], a["vec_norms"], q), dev.packed_scores(b["idx_bytes"], b["vec_norms"], q))
+    tq_host = pkg.TurboQuantV3(128, residual_window=8)
+    ck, cv = tq_host.compress_kv(x, x)
+    k, v = tq_host.decompress_kv(ck, cv)
+    assert k.shape == x.shape and torch.equal(k[:, :, -8:], x[:, :, -8:])
+    with pytest.raises(Exception):
+        host.compress(x.cpu())

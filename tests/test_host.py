@@ -471,3 +471,17 @@ def test_tables_for_other_head_dimensions(pkg):
         assert at[t, s, l, i] == np.float16(pi[16 * s + 8 * hk + i, col])
         assert native.lib().tq_table_check(blob.ctypes.data, blob.size, D, bits) == 0
         assert native.lib().tq_table_check(blob.ctypes.data, blob.size, 128, bits) != 0
+
+
+def test_device_default_is_the_references(pkg):
+    """compressors_v3.py:37,151 and compressors.py default to device="cpu": so do these classes; Pi and centroids then
+    live on the CPU, and asking for a codec table there (there is no CPU codec) raises."""
+    import inspect
+    for cls in (pkg.MSECompressor, pkg.TurboQuantV3, pkg.TurboQuantCompressorV2, pkg.TurboQuantCompressorMSE):
+        assert inspect.signature(cls.__init__).parameters["device"].default == "cpu", cls
+    comp = pkg.MSECompressor(128, 4, seed=1)
+    assert comp.Pi.device.type == "cpu" and comp.centroids.device.type == "cpu"
+    with pytest.raises(pkg._native.TqError, match="HIP devices only"):
+        comp.table()
+    tq = pkg.TurboQuantV3(128)
+    assert tq.key_compressor.Pi.device.type == "cpu"

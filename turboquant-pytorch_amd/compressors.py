@@ -29,7 +29,7 @@ def _qjl_matrix(head_dim: int, seed: int) -> torch.Tensor:
 class TurboQuantCompressorV2:
     """Keys for asymmetric attention: interface of compressors.py:25-158."""
 
-    def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cuda"):
+    def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cpu"):
         self.head_dim = head_dim
         self.bits = bits
         self.mse_bits = max(bits - 1, 1)
@@ -39,7 +39,7 @@ class TurboQuantCompressorV2:
         self._setup(pi_host, _qjl_matrix(head_dim, seed), cent_host)
 
     @classmethod
-    def from_tensors(cls, Pi: torch.Tensor, S: torch.Tensor, centroids: torch.Tensor, bits: int, device: str = "cuda"):
+    def from_tensors(cls, Pi: torch.Tensor, S: torch.Tensor, centroids: torch.Tensor, bits: int, device: str = "cpu"):
         """A compressor over explicit matrices and codebook (parity tests pass the reference's own through here)."""
         self = cls.__new__(cls)
         self.head_dim = Pi.shape[0]
@@ -70,15 +70,27 @@ class TurboQuantCompressorV2:
         _native.check(L.tq_qjl_table_build(pi.ctypes.data, s.ctypes.data, c.ctypes.data, self.head_dim, self.mse_bits,
                                            blob.ctypes.data, blob.size), "tq_qjl_table_build")
         self._qjl_host = blob
-        self._qjl_table = None
+        self._qjl_tables = {}
+        self._s_on = {}
 
-    def _table(self) -> torch.Tensor:
-        if self._qjl_table is None:
-            dev = torch.device(self.device)
+    def _table(self, device) -> torch.Tensor:
+        """The QJL table on `device` (the compressor itself may sit on the CPU, the reference's default)."""
+        dev = torch.device(device)
+        t = self._qjl_tables.get(dev)
+        if t is None:
             if dev.type != "cuda":
-                raise _native.TqError(f"TurboQuantCompressorV2(device={self.device!r}): the codec runs on HIP devices only")
-            self._qjl_table = torch.from_numpy(self._qjl_host).to(dev)
-        return self._qjl_table
+                raise _native.TqError(f"TurboQuantCompressorV2: the codec runs on HIP devices only (asked for a table on {dev})")
+            t = self._qjl_tables[dev] = torch.from_numpy(self._qjl_host).to(dev)
+        return t
+
+    def _s(self, device) -> torch.Tensor:
+        dev = torch.device(device)
+        if dev == self.S.device:
+            return self.S
+        t = self._s_on.get(dev)
+        if t is None:
+            t = self._s_on[dev] = self.S.to(dev)
+        return t
 
     @torch.no_grad()
     def compress(self, states: torch.Tensor) -> dict:
@@ -95,7 +107,7 @@ class TurboQuantCompressorV2:
         if n_vec:
             with _native._on(states.device):
                 rc = _native.lib().tq_qjl_signs(states.data_ptr(), _native.dtype_code(states.dtype), n_vec, D,
-                                                first["idx_bytes"].data_ptr(), self._table().data_ptr(), D, self.mse_bits,
+                                                first["idx_bytes"].data_ptr(), self._table(states.device).data_ptr(), D, self.mse_bits,
                                                 sign_bytes.data_ptr(), residual_norm.data_ptr(),
                                                 _native._stream_handle(states.device))
             _native.check(rc, "tq_qjl_signs")
@@ -126,7 +138,7 @@ class TurboQuantCompressorV2:
         if "idx_bytes" not in compressed:
             k_mse = compressed["k_mse"].float()
             term1 = torch.matmul(queries.float(), k_mse.transpose(-2, -1))
-            ip = torch.matmul(torch.matmul(queries.float(), self.S.T), compressed["qjl_signs"].float().transpose(-2, -1))
+            ip = torch.matmul(torch.matmul(queries.float(), self._s(queries.device).T), compressed["qjl_signs"].float().transpose(-2, -1))
             return term1 + corr * ip * compressed["residual_norm"].float().unsqueeze(-2)
         B, H, S_k, D = compressed["shape"]
         S_q = queries.shape[2]
@@ -134,7 +146,7 @@ class TurboQuantCompressorV2:
         if out.numel() == 0:
             return out
         q = queries.float()
-        q_sign = torch.matmul(q, self.S.T) * corr
+        q_sign = torch.matmul(q, self._s(q.device).T) * corr
         step = 32                                   # query tokens per key row and launch
         for lo in range(0, S_q, step):
             hi = min(lo + step, S_q)
@@ -151,7 +163,7 @@ class TurboQuantCompressorMSE:
     ("indices" one code per byte [N, D], "vec_norms" fp16 [N], "shape") next to the packed bytes the kernels wrote;
     `decompress` reads the packed bytes when they are there and packs the indices otherwise."""
 
-    def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cuda"):
+    def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cpu"):
         self.head_dim = head_dim
         self.bits = bits
         self.device = device

@@ -45,10 +45,10 @@ class MSECompressor:
     Interface of compressors_v3.py:28-120.
     """
 
-    def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cuda"):
+    def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cpu"):
         self.head_dim = head_dim
         self.bits = bits
-        self.device = device
+        self.device = device      # where Pi and centroids live (the reference's default: "cpu"); the kernels follow the tensors
 
         pi_host = _cached_rotation(head_dim, seed)
         cent_host = _cached_centroids(head_dim, bits)
@@ -57,10 +57,11 @@ class MSECompressor:
         # Everything the kernels read, baked once: split rotation tiles, quantiser grid, decode tables.
         # (above 8 bits the reference constructs fine and fails in compress(); keep that order)
         self._table_host = _native.build_table(pi_host, cent_host, bits) if 1 <= bits <= 8 else None
-        self._table = None
+        self._tables = {}
+        self._pi_on = {}
 
     @classmethod
-    def from_tensors(cls, Pi: torch.Tensor, centroids: torch.Tensor, bits: int, device: str = "cuda"):
+    def from_tensors(cls, Pi: torch.Tensor, centroids: torch.Tensor, bits: int, device: str = "cpu"):
         """Build a compressor from an explicit rotation and codebook (parity tests pass the
         reference's own matrices through here)."""
         self = cls.__new__(cls)
@@ -70,24 +71,41 @@ class MSECompressor:
         self.Pi = Pi.to(device=device, dtype=torch.float32).contiguous()
         self.centroids = centroids.to(device=device, dtype=torch.float32)
         self._table_host = _native.build_table(Pi, centroids, bits)
-        self._table = None
+        self._tables = {}
+        self._pi_on = {}
         return self
 
-    def pi_transposed(self) -> torch.Tensor:
-        """Pi^T as its own contiguous tensor (made on first use): the decode-step kernels read it row by row."""
-        t = getattr(self, "_pi_t", None)
+    def pi(self, device=None) -> torch.Tensor:
+        """Pi on `device` (default: the compressor's own): the compressor may sit on the CPU, as the reference's does
+        by default, while the tensors it is given are on a HIP device; copies are made once per device."""
+        dev = torch.device(self.device if device is None else device)
+        if dev == self.Pi.device:
+            return self.Pi
+        t = self._pi_on.get(dev)
         if t is None:
-            t = self._pi_t = self.Pi.t().contiguous()
+            t = self._pi_on[dev] = self.Pi.to(dev).contiguous()
         return t
 
-    def table(self) -> torch.Tensor:
-        """Device copy of the codec table (uploaded on first use)."""
-        if self._table is None:
-            dev = torch.device(self.device)
+    def pi_transposed(self, device=None) -> torch.Tensor:
+        """Pi^T as its own contiguous tensor (made on first use): the decode-step kernels read it row by row."""
+        dev = torch.device(self.device if device is None else device)
+        t = self._pi_on.get(("t", dev))
+        if t is None:
+            t = self._pi_on[("t", dev)] = self.pi(dev).t().contiguous()
+        return t
+
+    def table(self, device=None) -> torch.Tensor:
+        """Copy of the codec table on `device` (default: the compressor's own), uploaded on first use."""
+        dev = torch.device(self.device if device is None else device)
+        if dev.type == "cuda" and dev.index is None:
+            dev = torch.device("cuda", torch.cuda.current_device())
+        t = self._tables.get(dev)
+        if t is None:
             if dev.type != "cuda":
-                raise _native.TqError(f"MSECompressor(device={self.device!r}): the codec runs on HIP devices only")
-            self._table = _native.upload_table(self._table_host, self.head_dim, self.bits, dev)
-        return self._table
+                raise _native.TqError(f"MSECompressor: the codec runs on HIP devices only (asked for a table on {dev}); "
+                                      "pass tensors that live on the GPU")
+            t = self._tables[dev] = _native.upload_table(self._table_host, self.head_dim, self.bits, dev)
+        return t
 
     @torch.no_grad()
     def compress(self, states: torch.Tensor) -> dict:
@@ -95,7 +113,7 @@ class MSECompressor:
         B, H, S, D = states.shape
         indices_per_byte = 8 // self.bits
         idx_pad = (indices_per_byte - D % indices_per_byte) % indices_per_byte
-        idx_bytes, vec_norms = _native.call("compress", states, self.table(), self.bits)
+        idx_bytes, vec_norms = _native.call("compress", states, self.table(states.device), self.bits)
         return {
             "idx_bytes": idx_bytes,
             "vec_norms": vec_norms,
@@ -116,7 +134,7 @@ class MSECompressor:
         if idx_bytes.dtype != torch.uint8 or vec_norms.dtype != torch.float16:
             raise ValueError("packed buffers must be uint8 codes and float16 norms")
         if S * B * H:
-            _native.call("compress_into", states, self.table(), self.bits, idx_bytes, vec_norms)
+            _native.call("compress_into", states, self.table(states.device), self.bits, idx_bytes, vec_norms)
 
     @torch.no_grad()
     def decompress_packed(self, idx_bytes: torch.Tensor, vec_norms: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -126,7 +144,7 @@ class MSECompressor:
             raise ValueError(f"packed buffers {tuple(idx_bytes.shape)} / {tuple(vec_norms.shape)} do not match "
                              f"output {tuple(out.shape)}")
         if S * B * H:
-            _native.call("decompress_into", idx_bytes, vec_norms, self.table(), self.bits, out)
+            _native.call("decompress_into", idx_bytes, vec_norms, self.table(out.device), self.bits, out)
         return out
 
     @torch.no_grad()
@@ -141,11 +159,11 @@ class MSECompressor:
         Hq = q.shape[1]
         if Hq % H:
             raise ValueError(f"{Hq} query heads do not divide over {H} kv heads")
-        q_rot = torch.matmul(q.to(torch.float32), self.Pi.T) * scale        # (Pi q): rotate once per step
+        q_rot = torch.matmul(q.to(torch.float32), self.pi(q.device).T) * scale        # (Pi q): rotate once per step
         if out is None:
             out = torch.empty((B, Hq, S), dtype=torch.float32, device=idx_bytes.device)
         if B * Hq * S:
-            _native.call("scores_into", idx_bytes, vec_norms, self.table(), self.bits, q_rot, out)
+            _native.call("scores_into", idx_bytes, vec_norms, self.table(idx_bytes.device), self.bits, q_rot, out)
         return out
 
     @torch.no_grad()
@@ -156,8 +174,8 @@ class MSECompressor:
         B, H, S, _ = idx_bytes.shape
         if S == 0:
             return torch.zeros((B, weights.shape[1], self.head_dim), dtype=torch.float32, device=idx_bytes.device)
-        out_rot = _native.call("weighted_values", idx_bytes, vec_norms, self.table(), self.bits, weights, self.head_dim)
-        return torch.matmul(out_rot, self.Pi)
+        out_rot = _native.call("weighted_values", idx_bytes, vec_norms, self.table(idx_bytes.device), self.bits, weights, self.head_dim)
+        return torch.matmul(out_rot, self.pi(out_rot.device))
 
     @torch.no_grad()
     def decompress(self, compressed: dict) -> torch.Tensor:
@@ -166,7 +184,7 @@ class MSECompressor:
         width = math.ceil(D / (8 // self.bits))
         idx_bytes = compressed["idx_bytes"].reshape(B, H, S, width)
         vec_norms = compressed["vec_norms"].reshape(B, H, S)
-        return _native.call("decompress", idx_bytes, vec_norms, self.table(), self.bits, D, torch.float32)
+        return _native.call("decompress", idx_bytes, vec_norms, self.table(idx_bytes.device), self.bits, D, torch.float32)
 
     @torch.no_grad()
     def decompress_into(self, compressed: dict, out: torch.Tensor) -> torch.Tensor:
@@ -176,7 +194,7 @@ class MSECompressor:
             raise ValueError(f"output shape {tuple(out.shape)} does not match compressed shape {(B, H, S, D)}")
         width = math.ceil(D / (8 // self.bits))
         _native.call("decompress_into", compressed["idx_bytes"].reshape(B, H, S, width),
-                                        compressed["vec_norms"].reshape(B, H, S), self.table(), self.bits, out)
+                                        compressed["vec_norms"].reshape(B, H, S), self.table(out.device), self.bits, out)
         return out
 
     def memory_bytes(self, B: int, H: int, S: int) -> dict:
@@ -210,7 +228,7 @@ class TurboQuantV3:
         protected_layers: int = 4,
         protected_bits: int = 8,
         seed: int = 42,
-        device: str = "cuda",
+        device: str = "cpu",
     ):
         self.head_dim = head_dim
         self.residual_window = residual_window
