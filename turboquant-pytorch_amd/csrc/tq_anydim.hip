@@ -4,7 +4,8 @@
 // matrix cores, fp32 accumulation, norm applied after the rotation, threshold-grid code search, MSB-first packing,
 // fp16 centroids on the way back), in a plain form: no register-resident rotation, no software pipeline.
 //
-// A block works on groups of NT x 32 consecutive vectors.  The group is staged in LDS as 16-bit MFMA operands
+// A block (four waves) works on groups of nt x 32 consecutive vectors (nt = 4, or fewer where that lets a second block
+// share the compute unit's LDS).  The group is staged in LDS as 16-bit MFMA operands
 // (compress: the input itself, fp32 inputs as three exact bf16 terms; decompress: the centroids of the codes as
 // fp16); wave w then produces the row tiles w, w + waves, ... of the rotation (32 output coordinates each) for
 // all NT column tiles, reading its A operands from the table in memory (they stay in L2: one 16-byte load per
@@ -31,14 +32,34 @@ __host__ __device__ constexpr uint32_t align16(uint32_t v) { return (v + 15u) & 
 
 // LDS of the compress kernel: quantiser grid | per-piece sums of squares | per-vector sums | staged operand terms
 template <int DTYPE>
-__host__ __device__ constexpr uint32_t compress_lds_bytes(uint32_t d) {
+__host__ __device__ constexpr uint32_t compress_lds_bytes(uint32_t d, uint32_t nt) {
     using T = AnyIn<DTYPE>;
-    const uint32_t gv = T::NT * 32, pieces = d * T::ELEM / 16;
+    const uint32_t gv = nt * 32, pieces = d * T::ELEM / 16;
     return TQ_GRID_LDS_BYTES + align16(gv * pieces * 4) + gv * 4 + T::XTERMS * gv * (d + ROW_PAD) * 2;
 }
 // LDS of the decompress kernel: byte -> centroids table | per-vector norms | staged centroids
-__host__ __device__ constexpr uint32_t decompress_lds_bytes(uint32_t d) {
-    return 4096 + DEC_NT * 32 * 4 + DEC_NT * 32 * (d + ROW_PAD) * 2;
+__host__ __device__ constexpr uint32_t decompress_lds_bytes(uint32_t d, uint32_t nt) {
+    return 4096 + nt * 32 * 4 + nt * 32 * (d + ROW_PAD) * 2;
+}
+
+// A wave's share of a group's NT column tiles x d/32 row tiles.  With four or more row tiles every wave walks row tiles
+// wave, wave + 4, ... over all column tiles (one operand load feeds NT matrix instructions); with fewer, the waves
+// left over take a part of the column tiles each, so that all four work.
+struct WaveShare {
+    uint32_t rb0, rb_step;   // first row tile, stride
+    uint32_t ct0, ct_n;      // column tiles [ct0, ct0 + ct_n); ct_n == 0: nothing to do
+};
+__device__ __forceinline__ WaveShare wave_share(uint32_t wave, uint32_t nwaves, uint32_t tiles, uint32_t nt) {
+    WaveShare w;
+    const uint32_t rb_waves = tiles < nwaves ? tiles : nwaves;
+    uint32_t split = nwaves / rb_waves;          // waves per row tile: 4, 2, 1 (3 row tiles: 1, one wave rests)
+    split = split < nt ? split : nt;
+    const uint32_t part = wave / rb_waves;
+    w.rb0 = wave % rb_waves;
+    w.rb_step = rb_waves;
+    w.ct_n = part < split ? nt / split : 0u;
+    w.ct0 = part * (nt / split);
+    return w;
 }
 
 template <int BITS>
@@ -49,11 +70,12 @@ struct PackAny {
 };
 
 template <int DTYPE, int BITS>
-__global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_compress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t d) {
+__global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t d, uint32_t nt) {
     using T = AnyIn<DTYPE>;
     using P = PackAny<BITS>;
-    constexpr int ELEM = T::ELEM, NT = T::NT, GV = NT * 32;
+    constexpr int ELEM = T::ELEM, NT = T::NT;      // NT: the most column tiles a group may have; nt <= NT: those it has
     constexpr int NB = P::NB, NW = P::NW, IPB = P::IPB;
+    const uint32_t GV = nt * 32u;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -129,7 +151,8 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_compress_kernel(
         }
         __syncthreads();
 
-        for (uint32_t rb = wave; rb < tiles; rb += nwaves) {
+        const WaveShare share = wave_share(wave, nwaves, tiles, nt);
+        for (uint32_t rb = share.rb0; rb < tiles && share.ct_n; rb += share.rb_step) {
             tq_f16v acc[NT];
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct) acc[ct] = tq_zero16();
@@ -143,8 +166,9 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_compress_kernel(
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
 #pragma unroll
-                    for (int ct = 0; ct < NT; ++ct) {
-                        const uint16_t *row = xs + (ct * 32u + n) * row_halves + 16u * (s + u) + 8u * hk;
+                    for (int ct = 0; ct < NT; ++ct) {     // acc[ct] belongs to column tile share.ct0 + ct
+                        if ((uint32_t)ct >= share.ct_n) break;
+                        const uint16_t *row = xs + ((share.ct0 + ct) * 32u + n) * row_halves + 16u * (s + u) + 8u * hk;
 #pragma unroll
                         for (int xt = 0; xt < T::XTERMS; ++xt) {
                             const tq_u4 b = *reinterpret_cast<const tq_u4 *>(row + xt * term_halves);
@@ -163,7 +187,8 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_compress_kernel(
             // ---- code search and packing: lane (n, hk) holds coordinates 32 rb + 16 hk + r of vector ct * 32 + n
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct) {
-                const float nrm = tq_norm_from_sumsq(sumsq[ct * 32 + n]);
+                if ((uint32_t)ct >= share.ct_n) break;
+                const float nrm = tq_norm_from_sumsq(sumsq[(share.ct0 + ct) * 32u + n]);
                 float inv = __builtin_amdgcn_rcpf(nrm + 1e-8f);
                 if (DTYPE == TQ_F16) inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
                 const float inv_cell = inv * grid_scale;
@@ -180,7 +205,7 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_compress_kernel(
                     const int byte = r / IPB, k = r % IPB;                            // most significant code of a byte first
                     words[byte / 4] |= code << (8 * (byte % 4) + BITS * (IPB - 1 - k));
                 }
-                const uint32_t v = g * GV + ct * 32u + n;
+                const uint32_t v = g * GV + (share.ct0 + ct) * 32u + n;
                 if (v < job.n_vec) {
                     const uint32_t slot = tq_packed_slot(job, v);
                     uint8_t *dst = job.idx_bytes + (size_t)slot * g_bytes + (2u * rb + hk) * NB;
@@ -206,9 +231,10 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_compress_kernel(
 }
 
 template <int DTYPE, int IPB>
-__global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_decompress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t d) {
+__global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t d, uint32_t nt) {
     constexpr int ELEM = DTYPE == TQ_F32 ? 4 : 2;
-    constexpr int NT = DEC_NT, GV = NT * 32;
+    constexpr int NT = DEC_NT;
+    const uint32_t GV = nt * 32u;
     constexpr int ENTRY = 2 * IPB;                 // bytes of a table entry: the fp16 centroids of one packed byte
 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -260,7 +286,8 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_decompress_kerne
         }
         __syncthreads();
 
-        for (uint32_t rb = wave; rb < tiles; rb += nwaves) {
+        const WaveShare share = wave_share(wave, nwaves, tiles, nt);
+        for (uint32_t rb = share.rb0; rb < tiles && share.ct_n; rb += share.rb_step) {
             tq_f16v acc[NT];
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct) acc[ct] = tq_zero16();
@@ -272,7 +299,8 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_decompress_kerne
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
                     for (int ct = 0; ct < NT; ++ct) {
-                        const tq_u4 b = *reinterpret_cast<const tq_u4 *>(ys + (ct * 32u + n) * row_halves + 16u * (s + u) + 8u * hk);
+                        if ((uint32_t)ct >= share.ct_n) break;
+                        const tq_u4 b = *reinterpret_cast<const tq_u4 *>(ys + ((share.ct0 + ct) * 32u + n) * row_halves + 16u * (s + u) + 8u * hk);
                         acc[ct] = mfma_f16(a_cur[u], b, acc[ct]);
                     }
                 a_cur[0] = a_nxt[0];
@@ -281,9 +309,10 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE) void tq_anydim_decompress_kerne
             // ---- scale, cast, store: lane (n, hk) holds elements 32 rb + 16 hk + r of vector ct * 32 + n
 #pragma unroll
             for (int ct = 0; ct < NT; ++ct) {
-                const uint32_t v = g * GV + ct * 32u + n;
+                if ((uint32_t)ct >= share.ct_n) break;
+                const uint32_t v = g * GV + (share.ct0 + ct) * 32u + n;
                 if (v >= job.n_vec) continue;
-                const float nrm = norms[ct * 32 + n];
+                const float nrm = norms[(share.ct0 + ct) * 32u + n];
                 uint8_t *dst = out_base + tq_vec_offset(job, v) + (32u * rb + 16u * hk) * ELEM;
                 if constexpr (ELEM == 2) {
 #pragma unroll
@@ -337,11 +366,16 @@ int device_cus(int &dev, int &cus) {
     return 0;
 }
 
-// Launches `kernel` over (blocks per job) x n_jobs blocks of d / 32 waves (at most MAX_WAVES) with `lds` bytes of
+// Launches `kernel` over (blocks per job) x n_jobs blocks of MAX_WAVES waves with `lds` bytes of
 // dynamic LDS; `raised[dev]` remembers the largest LDS size the kernel has been allowed on each device.
-template <typename K>
-int launch(K kernel, uint32_t (&raised)[MAX_DEVICES], uint32_t lds, uint32_t group_vectors, const TqDevJob &job,
+template <typename K, typename L>
+int launch(K kernel, uint32_t (&raised)[MAX_DEVICES], L lds_for, uint32_t nt_max, const TqDevJob &job,
            const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, hipStream_t stream) {
+    // column tiles per group: as many as leave room for two blocks on a compute unit (the phases of a block do not
+    // overlap one another; a second block fills the gaps), but at least half of the most
+    uint32_t nt = nt_max;
+    while (nt > 1u && nt > nt_max / 2u && lds_for(d, nt) > 80u * 1024u) nt /= 2u;
+    const uint32_t lds = lds_for(d, nt), group_vectors = nt * 32u;
     int dev = 0, cus = 0;
     const int rc = device_cus(dev, cus);
     if (rc) return rc;
@@ -354,17 +388,17 @@ int launch(K kernel, uint32_t (&raised)[MAX_DEVICES], uint32_t lds, uint32_t gro
         }
     }
     const uint32_t groups = (max_vec + group_vectors - 1u) / group_vectors;
-    const uint32_t waves = d / 32u < (uint32_t)MAX_WAVES ? d / 32u : (uint32_t)MAX_WAVES;
-    const int resident = lds <= 40u * 1024u ? 3 : lds <= 64u * 1024u ? 2 : 1;     // blocks a compute unit's 160 KiB of LDS hold
+    const uint32_t waves = MAX_WAVES;
+    const int resident = lds <= 53u * 1024u ? 3 : lds <= 80u * 1024u ? 2 : 1;     // blocks per compute unit (160 KiB of LDS, 168 registers)
     const uint32_t bx = tq_blocks_per_job(groups, cus * resident, n_jobs);
-    hipLaunchKernelGGL(kernel, dim3(bx, (unsigned)n_jobs, 1), dim3(waves * TQ_WAVE, 1, 1), lds, stream, job, jobs_dev, d);
+    hipLaunchKernelGGL(kernel, dim3(bx, (unsigned)n_jobs, 1), dim3(waves * TQ_WAVE, 1, 1), lds, stream, job, jobs_dev, d, nt);
     return (int)hipGetLastError();
 }
 
 template <int DTYPE, int BITS>
 int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, hipStream_t s) {
     static uint32_t raised[MAX_DEVICES] = {};
-    return launch(&tq_anydim_compress_kernel<DTYPE, BITS>, raised, compress_lds_bytes<DTYPE>(d), AnyIn<DTYPE>::NT * 32, job, jobs_dev,
+    return launch(&tq_anydim_compress_kernel<DTYPE, BITS>, raised, compress_lds_bytes<DTYPE>, AnyIn<DTYPE>::NT, job, jobs_dev,
                   n_jobs, max_vec, d, s);
 }
 template <int DTYPE>
@@ -383,7 +417,7 @@ int compress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_j
 template <int DTYPE, int IPB>
 int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, hipStream_t s) {
     static uint32_t raised[MAX_DEVICES] = {};
-    return launch(&tq_anydim_decompress_kernel<DTYPE, IPB>, raised, decompress_lds_bytes(d), DEC_NT * 32, job, jobs_dev, n_jobs, max_vec, d, s);
+    return launch(&tq_anydim_decompress_kernel<DTYPE, IPB>, raised, decompress_lds_bytes, DEC_NT, job, jobs_dev, n_jobs, max_vec, d, s);
 }
 template <int DTYPE>
 int decompress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, hipStream_t s) {
