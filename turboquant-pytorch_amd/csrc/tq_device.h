@@ -279,8 +279,9 @@ __device__ __forceinline__ tq_u4 decode_rep(const uint32_t (&raw)[NW], int s, co
 }
 
 // Blocks per job for a (blocks_per_job x n_jobs) grid of equal-cost blocks on `cus` compute units
-// that hold one block each: enough blocks to fill the device a few times over, with the total as
-// close to a whole number of device-wide rounds as possible (a partial last round idles CUs).
+// that hold one block each.  Every block pays a set-up (rotation operands, tables), so the fewest
+// device-wide rounds win as long as the last round is nearly full (at most 3 % of the slots idle);
+// failing that, the round count with the fullest last round.
 static inline uint32_t tq_blocks_per_job(uint32_t want, int cus, int n_jobs) {
     if (n_jobs <= 1) return want < (uint32_t)cus ? (want ? want : 1u) : (uint32_t)cus;
     uint32_t best = 1;
@@ -291,9 +292,9 @@ static inline uint32_t tq_blocks_per_job(uint32_t want, int cus, int n_jobs) {
         if (per_job > want) per_job = want ? want : 1u;
         const long long total = (long long)per_job * n_jobs;
         const long long padded = (total + cus - 1) / cus * cus;
-        const double waste = (double)(padded - total) / (double)total;
+        const double waste = (double)(padded - total) / (double)padded;
         if (waste < best_waste - 1e-9) { best_waste = waste; best = per_job; }
-        if (per_job >= want) break;
+        if (waste <= 0.03 || per_job >= want) break;
     }
     return best;
 }
