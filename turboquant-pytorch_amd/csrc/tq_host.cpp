@@ -308,7 +308,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
 long long tq_qjl_table_bytes(int head_dim, int mse_bits) {
     if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
     if (mse_bits < 1 || mse_bits > 7) return TQ_ERR_BITS;
-    return (long long)sizeof(TqQjlHeader) + 5ll * TQ_OPERAND_BYTES + 1024;
+    return (long long)sizeof(TqQjlHeader) + 4ll * TQ_OPERAND_BYTES + 1024;
 }
 
 int tq_qjl_table_build(const float *Pi, const float *S, const float *centroids, int head_dim, int mse_bits,
@@ -321,6 +321,22 @@ int tq_qjl_table_build(const float *Pi, const float *S, const float *centroids, 
     if (!valid_codebook(centroids, levels)) return TQ_ERR_CODEBOOK;
     for (int i = 0; i < D * D; ++i)
         if (!std::isfinite(Pi[i]) || !std::isfinite(S[i])) return TQ_ERR_SIZE;
+    // power of two that puts the largest magnitude of v[0..n) into [2^13, 2^14) (all zeros: 1)
+    auto shift_for = [](const float *v, size_t n) {
+        float m = 0.f;
+        for (size_t i = 0; i < n; ++i) m = std::fmax(m, std::fabs(v[i]));
+        if (!(m > 0.f)) return 0;
+        int e = 0;
+        (void)std::frexp(m, &e);           // m = f * 2^e, f in [0.5, 1)
+        const int sh = 14 - e;
+        return sh < -100 ? -100 : sh > 100 ? 100 : sh;
+    };
+    const int sh_pit = shift_for(Pi, (size_t)D * D), sh_s = shift_for(S, (size_t)D * D), sh_c = shift_for(centroids, (size_t)levels);
+    auto split = [](float v, int sh, uint16_t &hi, uint16_t &lo) {
+        const double x = std::ldexp((double)v, sh);
+        hi = to_f16((float)x);
+        lo = to_f16((float)(x - (double)from_f16(hi)));
+    };
     uint8_t *blob = static_cast<uint8_t *>(table_host);
     std::memset(blob, 0, (size_t)need);
     TqQjlHeader hd{};
@@ -330,9 +346,10 @@ int tq_qjl_table_build(const float *Pi, const float *S, const float *centroids, 
     hd.mse_bits = (uint32_t)mse_bits;
     hd.levels = (uint32_t)levels;
     hd.off_pit = sizeof(TqQjlHeader);
-    hd.off_s = hd.off_pit + 3 * TQ_OPERAND_BYTES;
+    hd.off_s = hd.off_pit + 2 * TQ_OPERAND_BYTES;
     hd.off_centroids = hd.off_s + 2 * TQ_OPERAND_BYTES;
     hd.total_bytes = (uint32_t)need;
+    hd.k_scale = std::ldexp(1.0f, -(sh_pit + sh_c));
     uint16_t *pit = reinterpret_cast<uint16_t *>(blob + hd.off_pit);
     uint16_t *sm = reinterpret_cast<uint16_t *>(blob + hd.off_s);
     const size_t term = TQ_OPERAND_BYTES / 2;
@@ -345,21 +362,16 @@ int tq_qjl_table_build(const float *Pi, const float *S, const float *centroids, 
                 for (int i = 0; i < 8; ++i) {
                     const size_t o = (((size_t)t * TQ_STEPS + s) * 64 + l) * 8 + i;
                     const int k = 16 * s + 8 * hk + i;
-                    float v = Pi[k * D + out];                 // Pi^T[out][k]
-                    for (int q = 0; q < 3; ++q) {
-                        const uint16_t h16 = to_bf16(v);
-                        pit[q * term + o] = h16;
-                        v -= from_bf16(h16);
-                    }
-                    v = S[out * D + k];
-                    for (int q = 0; q < 2; ++q) {
-                        const uint16_t h16 = to_bf16(v);
-                        sm[q * term + o] = h16;
-                        v -= from_bf16(h16);
-                    }
+                    split(Pi[k * D + out], sh_pit, pit[o], pit[term + o]);      // Pi^T[out][k]
+                    split(S[out * D + k], sh_s, sm[o], sm[term + o]);
                 }
             }
-    std::memcpy(blob + hd.off_centroids, centroids, (size_t)levels * 4);
+    uint32_t *pairs = reinterpret_cast<uint32_t *>(blob + hd.off_centroids);
+    for (int i = 0; i < levels; ++i) {
+        uint16_t hi, lo;
+        split(centroids[i], sh_c, hi, lo);
+        pairs[i] = (uint32_t)hi | ((uint32_t)lo << 16);
+    }
     std::memcpy(blob, &hd, sizeof(hd));
     return TQ_OK;
 }

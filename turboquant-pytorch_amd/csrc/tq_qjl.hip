@@ -7,10 +7,13 @@
 //     signs    = (residual @ S^T >= 0)                    (:116-117), packed 8 per byte, coordinate 8b+k in bit 7-k
 //
 // Work decomposition (gfx950, wave64): a block is four waves that share tiles of 32 vectors; wave w keeps the rows
-// [32w, 32w+32) of Pi^T (three bf16 terms) and of S (two bf16 terms) resident in registers as MFMA A operands.  The
-// B operands are exact three-term bf16 splits of float32 data (the centroid of every code, then the residual),
-// staged in LDS in the XOR-swizzled tile layout of the compress kernel; all products whose weight is at least
-// 2^-24 of the leading one are taken, accumulation is fp32, so both rotations agree with a float32 GEMM to ~1e-6.
+// [32w, 32w+32) of Pi^T and of S resident in registers as MFMA A operands, each as two fp16 terms (hi + lo: 22 bits)
+// of the matrix times a power of two.  The B operands are two-term fp16 splits as well (the centroid of every code,
+// from a table of ready-made pairs; then the residual, scaled per vector by a power of two taken from its norm's
+// exponent), staged in LDS in the XOR-swizzled tile layout of the compress kernel.  The three products hi*hi, hi*lo,
+// lo*hi are taken (the fourth weighs 2^-22), accumulation is fp32: both rotations agree with a float32 GEMM to a few
+// 1e-7 of the vector's scale, the noise level of that GEMM's own rounding.  (The residual is a difference of nearly
+// equal vectors, up to 70 times smaller than they are at 7 bits: this is the precision its signs need.)
 #include <mutex>
 
 #include "tq_device.h"
@@ -30,27 +33,13 @@ struct QjlArgs {
     uint32_t mse_bits;
 };
 
-__device__ __forceinline__ tq_f16v qmfma(tq_u4 a, tq_u4 b, tq_f16v c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(tq_bf8, a), __builtin_bit_cast(tq_bf8, b), c, 0, 0, 0);
-}
-
-// Exact split of eight floats into three bf16 terms each (every term a truncation, every remainder exact in fp32).
-__device__ __forceinline__ void qsplit8(const float (&x)[8], tq_u4 &t0, tq_u4 &t1, tq_u4 &t2) {
-    uint32_t a[8], b[8], c[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t xa = __float_as_uint(x[i]) & 0xffff0000u;
-        const float r1 = x[i] - __uint_as_float(xa);
-        const uint32_t xb = __float_as_uint(r1) & 0xffff0000u;
-        const float r2 = r1 - __uint_as_float(xb);
-        a[i] = xa; b[i] = xb; c[i] = __float_as_uint(r2) & 0xffff0000u;
-    }
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        t0[d] = (a[2 * d] >> 16) | a[2 * d + 1];
-        t1[d] = (b[2 * d] >> 16) | b[2 * d + 1];
-        t2[d] = (c[2 * d] >> 16) | c[2 * d + 1];
-    }
+// Two floats -> their fp16 terms (hi: round toward zero, lo: the remainder, exact in fp32 before its own rounding).
+struct TermPair { uint32_t hi, lo; };
+__device__ __forceinline__ TermPair split_pair(float x0, float x1) {
+    typedef __fp16 pk_half2 __attribute__((ext_vector_type(2)));
+    const pk_half2 h = __builtin_amdgcn_cvt_pkrtz(x0, x1);
+    const pk_half2 l = __builtin_amdgcn_cvt_pkrtz(x0 - (float)h[0], x1 - (float)h[1]);
+    return {__builtin_bit_cast(uint32_t, h), __builtin_bit_cast(uint32_t, l)};
 }
 
 // BITS: packing class of the codes (1, 2, 3, 4, or 8 = one code per byte for 5..7 bits)
@@ -60,10 +49,10 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_residual_kernel(QjlArgs a)
     constexpr int IPB = 8 / BITS;
     constexpr int NB = 16 / IPB;           // packed bytes of 16 codes
     constexpr int G = 8 * NB;              // packed bytes per vector
-    constexpr int TILE = 32 * TQ_HEAD_DIM * 2;   // one bf16 term of a 32-vector tile: 8 KiB
+    constexpr int TILE = 32 * TQ_HEAD_DIM * 2;   // one fp16 term of a 32-vector tile: 8 KiB
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds_terms[3][TILE];   // centroid terms, then residual terms
-    __shared__ float lds_cent[256];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_terms[2][TILE];   // centroid terms, then residual terms
+    __shared__ uint32_t lds_cent[256];     // code -> fp16 terms of its centroid (hi | lo << 16)
     __shared__ float lds_n2[4][32];        // shares of ||x||^2
     __shared__ float lds_r2[4][32];        // shares of ||residual||^2
 
@@ -73,20 +62,21 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_residual_kernel(QjlArgs a)
     const TqQjlHeader *hd = reinterpret_cast<const TqQjlHeader *>(a.table);
 
     // ---- this wave's rows of Pi^T and S, resident for the whole kernel
-    tq_u4 a_pit[3][TQ_STEPS], a_s[2][TQ_STEPS];
+    tq_u4 a_pit[2][TQ_STEPS], a_s[2][TQ_STEPS];
     {
         const uint8_t *pit = a.table + hd->off_pit, *sm = a.table + hd->off_s;
 #pragma unroll
         for (int s = 0; s < TQ_STEPS; ++s) {
             const size_t o = (((size_t)wave * TQ_STEPS + s) * 64 + lane) * 16;
 #pragma unroll
-            for (int q = 0; q < 3; ++q) a_pit[q][s] = tq_gload16(pit + (size_t)q * TQ_OPERAND_BYTES + o);
+            for (int q = 0; q < 2; ++q) a_pit[q][s] = tq_gload16(pit + (size_t)q * TQ_OPERAND_BYTES + o);
 #pragma unroll
             for (int q = 0; q < 2; ++q) a_s[q][s] = tq_gload16(sm + (size_t)q * TQ_OPERAND_BYTES + o);
         }
     }
     for (uint32_t i = tid; i < 256u; i += QTHREADS)
-        lds_cent[i] = i < hd->levels ? *reinterpret_cast<const TQ_GLOBAL float *>((const TQ_GLOBAL uint8_t *)(a.table + hd->off_centroids) + 4u * i) : 0.f;
+        lds_cent[i] = i < hd->levels ? *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)(a.table + hd->off_centroids) + 4u * i) : 0u;
+    const float k_scale = hd->k_scale;
     __syncthreads();
 
     const uint32_t n_tiles = (a.n_vec + 31u) / 32u;
@@ -95,20 +85,41 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_residual_kernel(QjlArgs a)
     // the lane's 16 coordinates [32w + 16hk, +16) of vector n are pieces 4w + 2hk and 4w + 2hk + 1 of its row
     const uint32_t my_piece = 4u * wave + 2u * hk;
 
+    // What a thread reads of a tile: the packed bytes of 16 codes of vector dv (decode role) and the 16 input
+    // coordinates [32w + 16hk, +16) of vector n (matrix role).  Fetched one tile ahead of the work on them.
+    constexpr int XQ = 16 * ELEM / 16;     // 16-byte pieces of the lane's coordinates
+    struct Fetched { uint32_t raw[4]; tq_u4 xq[XQ]; };
+    auto fetch = [&](uint32_t tl) {
+        Fetched f;
+        uint32_t v = tl * 32u + dv;
+        v = v < a.n_vec ? v : a.n_vec - 1u;              // tail: the last vector again, never stored
+        const uint8_t *src = a.idx_bytes + (size_t)v * G + seg * NB;
+        f.raw[0] = f.raw[1] = f.raw[2] = f.raw[3] = 0u;
+        if constexpr (NB == 2) f.raw[0] = tq_gload2(reinterpret_cast<const uint16_t *>(src));
+        else if constexpr (NB == 4) f.raw[0] = *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)src);
+        else if constexpr (NB == 8) { const tq_u2 t = tq_gload8(src); f.raw[0] = t[0]; f.raw[1] = t[1]; }
+        else { const tq_u4 t = tq_gload16(src); f.raw[0] = t[0]; f.raw[1] = t[1]; f.raw[2] = t[2]; f.raw[3] = t[3]; }
+        uint32_t vx = tl * 32u + n;
+        vx = vx < a.n_vec ? vx : a.n_vec - 1u;
+        const uint8_t *xs = a.states + (long long)vx * a.token_stride + (32u * wave + 16u * hk) * ELEM;
+#pragma unroll
+        for (int q = 0; q < XQ; ++q) f.xq[q] = tq_gload16(xs + 16 * q);
+        return f;
+    };
+    Fetched ahead = fetch(blockIdx.x < n_tiles ? blockIdx.x : 0u);
+
     for (uint32_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-        // ---- (1) codes -> centroids -> three bf16 terms in LDS (vector dv, codes [16 seg, 16 seg + 16))
+        const Fetched cur = ahead;
         {
-            uint32_t v = tile * 32u + dv;
-            v = v < a.n_vec ? v : a.n_vec - 1u;              // tail: the last vector again, never stored
-            const uint8_t *src = a.idx_bytes + (size_t)v * G + seg * NB;
-            uint32_t raw[4] = {0u, 0u, 0u, 0u};
-            if constexpr (NB == 2) raw[0] = tq_gload2(reinterpret_cast<const uint16_t *>(src));
-            else if constexpr (NB == 4) raw[0] = *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)src);
-            else if constexpr (NB == 8) { const tq_u2 t = tq_gload8(src); raw[0] = t[0]; raw[1] = t[1]; }
-            else { const tq_u4 t = tq_gload16(src); raw[0] = t[0]; raw[1] = t[1]; raw[2] = t[2]; raw[3] = t[3]; }
+            const uint32_t next = tile + gridDim.x;
+            ahead = fetch(next < n_tiles ? next : tile);     // past the end: the same tile again, never used
+        }
+        // ---- (1) codes -> the fp16 terms of their centroids in LDS (vector dv, codes [16 seg, 16 seg + 16))
+        {
+            const uint32_t (&raw)[4] = cur.raw;
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-                float c[8];
+                uint32_t c[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int k = 8 * half + i;                       // code number inside the segment
@@ -117,31 +128,31 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_residual_kernel(QjlArgs a)
                     const uint32_t code = (bv >> (BITS * (IPB - 1 - pos))) & code_mask;
                     c[i] = lds_cent[code];
                 }
-                tq_u4 t0, t1, t2;
-                qsplit8(c, t0, t1, t2);
+                tq_u4 t0, t1;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {     // two codes per word: their hi terms, their lo terms
+                    t0[d] = __builtin_amdgcn_perm(c[2 * d + 1], c[2 * d], 0x05040100u);
+                    t1[d] = __builtin_amdgcn_perm(c[2 * d + 1], c[2 * d], 0x07060302u);
+                }
                 const uint32_t off = dv * 256u + (((2u * seg + half) ^ (dv & 15u)) << 4);
                 *reinterpret_cast<tq_u4 *>(lds_terms[0] + off) = t0;
                 *reinterpret_cast<tq_u4 *>(lds_terms[1] + off) = t1;
-                *reinterpret_cast<tq_u4 *>(lds_terms[2] + off) = t2;
             }
         }
         // ---- the lane's 16 input coordinates, and its share of ||x||^2
         float x[16];
         {
-            uint32_t v = tile * 32u + n;
-            v = v < a.n_vec ? v : a.n_vec - 1u;
-            const uint8_t *src = a.states + (long long)v * a.token_stride + (32u * wave + 16u * hk) * ELEM;
             if constexpr (ELEM == 4) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const tq_u4 t = tq_gload16(src + 16 * q);
+                    const tq_u4 t = cur.xq[q];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) x[4 * q + i] = __uint_as_float(t[i]);
                 }
             } else {
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
-                    const tq_u4 t = tq_gload16(src + 16 * q);
+                    const tq_u4 t = cur.xq[q];
                     if constexpr (DTYPE == TQ_BF16) {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
@@ -171,19 +182,23 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_residual_kernel(QjlArgs a)
         for (int s = 0; s < TQ_STEPS; ++s) {
             const uint32_t off = n * 256u + (((2u * s + hk) ^ (n & 15u)) << 4);
 #pragma unroll
-            for (int i = 0; i < 3; ++i) {
+            for (int i = 0; i < 2; ++i) {
                 const tq_u4 bop = *reinterpret_cast<const tq_u4 *>(lds_terms[i] + off);
 #pragma unroll
-                for (int j = 0; i + j < 3; ++j) acc = qmfma(a_pit[j][s], bop, acc);
+                for (int j = 0; i + j < 2; ++j) acc = mfma_f16(a_pit[j][s], bop, acc);
             }
         }
         const float nrm = sqrtf((lds_n2[0][n] + lds_n2[1][n]) + (lds_n2[2][n] + lds_n2[3][n]));
-        // ---- (3) residual, its norm, its three bf16 terms
+        // power of two that brings the residual (|r_i| <= 2 ||x||) into the fp16 range: 2^(10 - E), ||x|| = f * 2^E, f in [0.5, 1)
+        uint32_t r_exp = 263u - ((__float_as_uint(nrm) >> 23) & 0xffu);
+        r_exp = r_exp > 254u ? 254u : r_exp;
+        const float r_scale = __uint_as_float(r_exp << 23);
+        // ---- (3) residual, its norm, its two fp16 terms
         float r[16];
         float r2 = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float km = acc[i] * nrm;
+            const float km = (acc[i] * k_scale) * nrm;
             r[i] = x[i] - km;
             r2 = fmaf(r[i], r[i], r2);
         }
@@ -192,15 +207,16 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_residual_kernel(QjlArgs a)
         __syncthreads();                   // everybody has read the centroid terms
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-            float c[8];
+            tq_u4 t0, t1;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) c[i] = r[8 * half + i];
-            tq_u4 t0, t1, t2;
-            qsplit8(c, t0, t1, t2);
+            for (int d = 0; d < 4; ++d) {
+                const TermPair t = split_pair(r[8 * half + 2 * d] * r_scale, r[8 * half + 2 * d + 1] * r_scale);
+                t0[d] = t.hi;
+                t1[d] = t.lo;
+            }
             const uint32_t off = n * 256u + (((my_piece + half) ^ (n & 15u)) << 4);
             *reinterpret_cast<tq_u4 *>(lds_terms[0] + off) = t0;
             *reinterpret_cast<tq_u4 *>(lds_terms[1] + off) = t1;
-            *reinterpret_cast<tq_u4 *>(lds_terms[2] + off) = t2;
         }
         __syncthreads();
 
@@ -210,10 +226,10 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_residual_kernel(QjlArgs a)
         for (int s = 0; s < TQ_STEPS; ++s) {
             const uint32_t off = n * 256u + (((2u * s + hk) ^ (n & 15u)) << 4);
 #pragma unroll
-            for (int i = 0; i < 3; ++i) {
+            for (int i = 0; i < 2; ++i) {
                 const tq_u4 bop = *reinterpret_cast<const tq_u4 *>(lds_terms[i] + off);
 #pragma unroll
-                for (int j = 0; j < 2 && i + j < 3; ++j) prj = qmfma(a_s[j][s], bop, prj);
+                for (int j = 0; i + j < 2; ++j) prj = mfma_f16(a_s[j][s], bop, prj);
             }
         }
         uint32_t word = 0;                 // byte 0: coordinates 0..7 of the lane, most significant bit first; byte 1: 8..15

@@ -90,21 +90,26 @@ struct TqTableHeader {
 static_assert(sizeof(TqTableHeader) == 256, "header is one 256-byte block");
 
 // --- table of the V2 key path (MSE codes + 1-bit QJL signs of the residual) ---------------------------------------
-// Operand tiles in the compress tiling above (tile = wave, out = 32w + 16h + r, input = 16s + 8hk + i), as bf16 terms:
-//   Pi^T : k_unit[out] = sum_j centroid(code_j) * Pi[j][out]      three terms (hi, mid, lo: exact to 2^-24)
-//   S    : projected[out] = sum_k residual[k] * S[out][k]         two terms (2^-17)
+// Operand tiles in the compress tiling above (tile = wave, out = 32w + 16h + r, input = 16s + 8hk + i), as fp16 terms
+// (hi, lo: 22 bits, 2^-22 of the largest entry) of the matrices times a power of two that puts their largest entry
+// into [2^13, 2^14), so that the low terms stay in the fp16 normal range:
+//   Pi^T : k_unit[out] = sum_j centroid(code_j) * Pi[j][out]
+//   S    : projected[out] = sum_k residual[k] * S[out][k]      (only its sign is used: any positive scale does)
+// The centroids come as pairs of fp16 terms of centroid * 2^cent_shift, one 32-bit word per code (hi | lo << 16);
+// k_scale = 2^-(pit_shift + cent_shift) takes the product back.
 #define TQ_QJL_MAGIC 0x54514a4cu /* "TQJL" */
-#define TQ_QJL_VERSION 1u
+#define TQ_QJL_VERSION 2u
 struct TqQjlHeader {
     uint32_t magic;
     uint32_t version;
     uint32_t head_dim;
     uint32_t mse_bits;
     uint32_t levels;
-    uint32_t off_pit;        // 3 x TQ_OPERAND_BYTES
+    uint32_t off_pit;        // 2 x TQ_OPERAND_BYTES
     uint32_t off_s;          // 2 x TQ_OPERAND_BYTES
-    uint32_t off_centroids;  // float[256], the first `levels` used
+    uint32_t off_centroids;  // uint32[256], the first `levels` used
     uint32_t total_bytes;
-    uint32_t reserved[55];
+    float k_scale;
+    uint32_t reserved[54];
 };
 static_assert(sizeof(TqQjlHeader) == 256, "header is one 256-byte block");
