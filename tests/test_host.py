@@ -485,3 +485,28 @@ def test_device_default_is_the_references(pkg):
         comp.table()
     tq = pkg.TurboQuantV3(128)
     assert tq.key_compressor.Pi.device.type == "cpu"
+
+
+def test_host_side_of_the_abi_under_sanitizers(tmp_path):
+    """csrc/tq_host.cpp (table builders, thresholds, host quantiser) compiled with AddressSanitizer and
+    UndefinedBehaviorSanitizer and driven by tests/native/host_sanitize.cpp over head dimensions 32 ... 256 and every
+    width, with table buffers of exactly the size tq_table_bytes reports; the driver also checks the host quantiser
+    against the nearest-centroid definition."""
+    import shutil
+    import subprocess
+    gxx = shutil.which("g++")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    if gxx is None or not os.path.exists(os.path.join(rocm, "lib", "libamdhip64.so")):
+        pytest.skip("needs g++ and the HIP runtime library to link tq_status_string")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = str(tmp_path / "host_sanitize")
+    cmd = [gxx, "-O1", "-g", "-std=c++17", "-fno-omit-frame-pointer", "-fsanitize=address,undefined",
+           "-fno-sanitize-recover=all", "-static-libasan", "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(rocm, "include"),
+           os.path.join(root, "tests", "native", "host_sanitize.cpp"),
+           os.path.join(root, "turboquant-pytorch_amd", "csrc", "tq_host.cpp"), "-o", exe,
+           "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    build = subprocess.run(cmd, capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr[-2000:]
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")      # (the HIP runtime keeps its own allocations until exit)
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=300, env=env)
+    assert run.returncode == 0 and run.stdout.strip() == "ok", run.stdout + run.stderr[-3000:]
