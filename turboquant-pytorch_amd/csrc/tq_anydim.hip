@@ -112,11 +112,15 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kern
     for (uint32_t g = blockIdx.x; g < n_groups; g += gridDim.x) {
         __syncthreads();      // nobody still reads the previous group (first trip: the grid copy is published below)
         // ---- stage the group: 16-byte pieces, coalesced; vectors past the end re-read the last one (never stored)
-        for (uint32_t i = tid; i < GV * pieces; i += nthreads) {
+        // (four fetches of a thread are in flight together)
+        auto fetch = [&](uint32_t i) {
             const uint32_t v = i / pieces, p = i - v * pieces;
             uint32_t gv = g * GV + v;
             gv = gv < job.n_vec ? gv : job.n_vec - 1u;
-            const tq_u4 q = tq_gload16(job.states + tq_vec_offset(job, gv) + p * 16u);
+            return tq_gload16(job.states + tq_vec_offset(job, gv) + p * 16u);
+        };
+        auto place = [&](uint32_t i, const tq_u4 q) {
+            const uint32_t v = i / pieces, p = i - v * pieces;
             if constexpr (ELEM == 2) {
                 *reinterpret_cast<tq_u4 *>(xs + v * row_halves + p * 8u) = q;
                 part[i] = sumsq8<DTYPE>(q, 0.f);
@@ -141,6 +145,20 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kern
                 *reinterpret_cast<tq_u2 *>(dst + term_halves) = w1;
                 *reinterpret_cast<tq_u2 *>(dst + 2u * term_halves) = w2;
                 part[i] = ss;
+            }
+        };
+        const uint32_t total = GV * pieces;
+        for (uint32_t i0 = tid; i0 < total; i0 += 4u * nthreads) {
+            tq_u4 q[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t i = i0 + u * nthreads;
+                q[u] = fetch(i < total ? i : i0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t i = i0 + u * nthreads;
+                if (i < total) place(i, q[u]);
             }
         }
         __syncthreads();
@@ -263,12 +281,15 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_ke
     for (uint32_t g = blockIdx.x; g < n_groups; g += gridDim.x) {
         __syncthreads();
         // ---- stage: every packed byte becomes its IPB centroids (one table entry), in code order
-        for (uint32_t i = tid; i < GV * g_words; i += nthreads) {
+        auto fetch = [&](uint32_t i) {
             const uint32_t v = i / g_words, w = i - v * g_words;
             uint32_t gv = g * GV + v;
             gv = gv < job.n_vec ? gv : job.n_vec - 1u;
             const uint32_t slot = tq_packed_slot(job, gv);
-            const uint32_t raw = *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)job.idx_bytes + (size_t)slot * g_bytes + 4u * w);
+            return *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)job.idx_bytes + (size_t)slot * g_bytes + 4u * w);
+        };
+        auto place = [&](uint32_t i, uint32_t raw) {
+            const uint32_t v = i / g_words, w = i - v * g_words;
             uint8_t *dst = reinterpret_cast<uint8_t *>(ys + v * row_halves) + 4u * w * ENTRY;
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
@@ -277,6 +298,20 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_ke
                 else if constexpr (ENTRY == 4) *reinterpret_cast<uint32_t *>(dst + b * ENTRY) = *reinterpret_cast<const uint32_t *>(e);
                 else if constexpr (ENTRY == 8) *reinterpret_cast<tq_u2 *>(dst + b * ENTRY) = *reinterpret_cast<const tq_u2 *>(e);
                 else *reinterpret_cast<tq_u4 *>(dst + b * ENTRY) = *reinterpret_cast<const tq_u4 *>(e);
+            }
+        };
+        const uint32_t total = GV * g_words;
+        for (uint32_t i0 = tid; i0 < total; i0 += 4u * nthreads) {     // four fetches of a thread in flight together
+            uint32_t raw[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t i = i0 + u * nthreads;
+                raw[u] = fetch(i < total ? i : i0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t i = i0 + u * nthreads;
+                if (i < total) place(i, raw[u]);
             }
         }
         for (uint32_t v = tid; v < GV; v += nthreads) {
