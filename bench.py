@@ -91,6 +91,33 @@ def cpu_model() -> str:
     return platform.processor() or platform.machine()
 
 
+def stream_rates(torch, dev, gib=1.0, reps=7):
+    """What this part's memory system delivers to plain streaming kernels (torch operators only, untimed leg of the
+    bench): copy (1 GiB read + 1 GiB written), read-only (a sum over 1 GiB) and write-only (a fill of 1 GiB), in GB/s of
+    bytes moved, median of `reps` runs after two warm-up runs.  The buffers are four times the last-level cache."""
+    n = int(gib * (1 << 30)) // 4
+    a = torch.zeros(n, dtype=torch.float32, device=dev)
+    b = torch.empty_like(a)
+
+    def rate(fn, nbytes):
+        times = []
+        for k in range(reps + 2):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            if k >= 2:
+                times.append(e0.elapsed_time(e1))
+        times.sort()
+        return nbytes / times[len(times) // 2] / 1e6
+
+    out = {"copy": rate(lambda: b.copy_(a), 8 * n), "read": rate(lambda: a.sum(), 4 * n), "write": rate(lambda: b.fill_(1.0), 4 * n),
+           "buffer_GiB": gib, "how": "torch copy_ / sum / fill_ on float32, HIP events, median of %d" % reps}
+    del a, b
+    return out
+
+
 def _timed_sample(run, make_input, share, budget_s, probe_n=2048, cap=4_000_000):
     """Times run(x) on a sample sized so that it takes about share * budget_s seconds; returns (vectors/s, n)."""
     x = make_input(probe_n)
@@ -301,6 +328,10 @@ def main():
     ap.add_argument("--workload", default="llama3-8b-32k", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
+    ap.add_argument("--skeleton", action="store_true",
+                    help="time the memory-skeleton build of the two codec kernels (csrc/libtqamd_skeleton.so from "
+                         "_native.build_skeleton(): loads, LDS traffic and stores only; the output is garbage)")
+    ap.add_argument("--no-stream-rates", action="store_true", help="skip the plain-stream leg (copy / read / write rates of the part)")
     ap.add_argument("--launch-order", default="",
                     help="sequence of the step's launches, e.g. c2,c4,c8,d8,d4,d2 (default: compress by width, then decompress by width)")
     args = ap.parse_args()
@@ -311,6 +342,11 @@ def main():
     import torch
     pkg = importlib.import_module("turboquant-pytorch_amd")
     native = pkg._native
+    if args.skeleton:
+        if not os.path.exists(native.SKELETON_LIB_PATH):
+            sys.exit(f"bench.py --skeleton: {native.SKELETON_LIB_PATH} is missing; build it first (on the CPU): "
+                     "python -c 'import importlib; importlib.import_module(\"turboquant-pytorch_amd._native\").build_skeleton()'")
+        native.LIB_PATH = native.SKELETON_LIB_PATH          # before the first call loads the library
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a HIP device")
     dev = torch.device("cuda:0")
@@ -425,7 +461,7 @@ def main():
     # ---- sanity: what was timed is a real round trip ----------------------------------------------
     j = groups[order[0]][0]
     rel = float((j["out"].float() - j["states"].float()).norm() / j["states"].float().norm())
-    if not (0.0 < rel < 0.6):
+    if not (0.0 < rel < 0.6) and not args.skeleton:
         sys.exit(f"bench.py: round trip looks wrong (relative error {rel})")
 
     # ---- accounting ------------------------------------------------------------------------------------
@@ -483,6 +519,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w["dtype"], "data": "synthetic",
         "untimed_steps_after_warmup": 3 + conditioning_steps + table_steps,
+        "warmup_total": args.warmup + 3 + conditioning_steps + table_steps,      # every untimed step before the timed region
         "config": {"workload": args.workload, "layers": L, "batch": B, "kv_heads": H, "tokens": S, "head_dim": 128,
                    "key_bits": w["key_bits"], "value_bits": w["value_bits"], "protected_layers": w["protected"],
                    "residual_window": 0, "width_groups": {str(b): len(groups[b]) for b in order},
@@ -497,7 +534,14 @@ def main():
         "kernels": kernels,
         "round_trip_rel_error": rel,
     }
-    if not args.no_cpu_baseline:
+    if args.skeleton:
+        result["skeleton"] = ("memory-skeleton build: no matrix instructions, no code search, no decode; the output is "
+                              "garbage and `value` is not a measurement of the codec")
+    if not args.no_stream_rates:
+        # the part's plain-stream rates beside the codec's: what a copy, a read and a write kernel reach on this box
+        result["roofline"]["stream_GBps"] = stream_rates(torch, dev)
+        result["roofline"]["step_frac_of_copy_rate"] = result["step_GBps"] / result["roofline"]["stream_GBps"]["copy"]
+    if not args.no_cpu_baseline and not args.skeleton:
         result["cpu_baseline"] = cpu_baseline(pkg, widths, args.cpu_seconds)
     print(json.dumps(result))
 

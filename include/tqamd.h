@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define TQ_ABI_VERSION 4
+#define TQ_ABI_VERSION 5
 
 /* element types of K/V tensors */
 enum { TQ_F32 = 0, TQ_F16 = 1, TQ_BF16 = 2 };
@@ -120,12 +120,19 @@ int tq_table_quantize_host(const void *table_host, const float *r, long long n, 
  *               [rows, capacity]: pass pointers already advanced to the first free token and
  *               packed_row_stride = capacity (the chunk list of generation_test_v2.py:109-126
  *               kept as one buffer).
+ *   workspace   device memory of tq_workspace_bytes(1) bytes, 64-byte aligned, or NULL: the counters from which
+ *               the blocks of a large single-row job of 16-bit elements draw runs of tiles in the order in which
+ *               they become free (compute units that run slower take fewer, and all blocks end together; the
+ *               results are the same bytes).  Same contract as the workspace of tq_decompress below: zero before
+ *               its first use, left zero by every launch that completes, never shared by launches that can
+ *               overlap in time.  NULL selects the fixed assignment of tiles to blocks.
  *   stream      hipStream_t (NULL = the default stream)
  */
 int tq_compress(const void *states, int dtype, long long rows, long long tokens,
                 long long row_stride, long long token_stride,
                 const void *table_dev, int head_dim, int bits,
-                uint8_t *idx_bytes, uint16_t *vec_norms, long long packed_row_stride, void *stream);
+                uint8_t *idx_bytes, uint16_t *vec_norms, long long packed_row_stride,
+                void *workspace, void *stream);
 
 /*
  * decompress: packed codes + fp16 norms -> vectors of `out_dtype`.
@@ -163,8 +170,9 @@ int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms, long long
  * `jobs_host` is read for validation and launch sizing; `jobs_dev` is a device copy of the
  * same n_jobs records that the kernel reads -- the caller uploads it once and may reuse it
  * for every call with the same buffers (nothing is allocated here).
- * tq_decompress_batched takes a workspace of tq_workspace_bytes(n_jobs) bytes under the contract
- * stated at tq_decompress (job i uses bytes [i * TQ_WORKSPACE_BYTES_PER_JOB, ...)), or NULL.
+ * Both take a workspace of tq_workspace_bytes(n_jobs) bytes under the contract stated at
+ * tq_decompress (job i uses bytes [i * TQ_WORKSPACE_BYTES_PER_JOB, ...)), or NULL; a compress and a
+ * decompress launch that cannot overlap in time may share one.
  */
 typedef struct tq_job {
     const void *states;        /* compress: input vectors;   decompress: output vectors   */
@@ -180,7 +188,7 @@ typedef struct tq_job {
 } tq_job;
 
 int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
-                        int head_dim, void *stream);
+                        int head_dim, void *workspace, void *stream);
 int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
                           int head_dim, void *workspace, void *stream);
 

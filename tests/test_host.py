@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol(pkg):
     for name in declared:
         assert hasattr(lib, name), name
     assert sorted(pkg._native.EXPORTS) == declared
-    assert lib.tq_abi_version() == 4
+    assert lib.tq_abi_version() == 5
     assert lib.tq_status_string(0) == b"ok"
     assert b"bits" in lib.tq_status_string(-2)
 
@@ -259,16 +259,30 @@ def test_table_and_width_must_agree(pkg):
     broken[0] ^= 0xFF
     assert lib.tq_table_check(broken.ctypes.data, broken.size, 128, 4) == -7
     assert lib.tq_table_check(None, 0, 128, 4) == -1
-    # the launch-side check: a tensor registered as a 4-bit table cannot be launched as a 2-bit one
+    # the launch-side check: a tensor tagged as a 4-bit table cannot be launched as a 2-bit one
     fake = torch.zeros(16, dtype=torch.uint8)
-    native._table_widths[fake.data_ptr()] = (128, 4)
-    try:
-        native.check_table(fake, 128, 4)
-        with pytest.raises(native.TqError, match="4 bits used with head_dim 128, 2 bits"):
-            native.check_table(fake, 128, 2)
-        native.check_table(torch.zeros(16, dtype=torch.uint8), 128, 2)             # unknown tables pass
-    finally:
-        del native._table_widths[fake.data_ptr()]
+    setattr(fake, native._TABLE_TAG, (128, 4))
+    native.check_table(fake, 128, 4)
+    with pytest.raises(native.TqError, match="4 bits used with head_dim 128, 2 bits"):
+        native.check_table(fake, 128, 2)
+    native.check_table(torch.zeros(16, dtype=torch.uint8), 128, 2)             # unknown tables pass
+
+
+def test_table_tag_does_not_outlive_its_tensor(pkg):
+    """The width a table was uploaded for is a property of the tensor object, not of its address: when a table is
+    freed and a caller's own, untagged upload lands on the same storage, no stale width is found for it."""
+    native = pkg._native
+    storage = torch.zeros(64, dtype=torch.uint8)
+    tagged = storage[:16]
+    setattr(tagged, native._TABLE_TAG, (128, 4))
+    address = tagged.data_ptr()
+    with pytest.raises(native.TqError):
+        native.check_table(tagged, 128, 2)
+    del tagged
+    reused = storage[:16]                       # same address, another tensor object: a caller's own table
+    assert reused.data_ptr() == address
+    native.check_table(reused, 128, 2)          # passes: nothing is known about it
+    native.check_table(reused, 64, 8)
 
 
 def test_workspace_is_dropped_after_a_failed_call(pkg):
@@ -314,7 +328,7 @@ def test_c_abi_argument_errors(pkg):
     args = dict(rows=1, tokens=4, rs=0, ts=128)
     call = lambda states, dtype, bits, hd, idx=p, norms=p, table=p, **kw: lib.tq_compress(
         states, dtype, kw.get("rows", 1), kw.get("tokens", 4), kw.get("rs", 0), kw.get("ts", 128), table, hd, bits,
-        idx, norms, kw.get("prs", 0), None)
+        idx, norms, kw.get("prs", 0), kw.get("ws", None), None)
     assert call(p, 1, 0, 128) == E["BITS"]
     assert call(p, 1, 4, 80) == E["HEAD_DIM"]
     assert call(p, 1, 4, 64, ts=48) == E["SIZE"]
@@ -339,8 +353,10 @@ def test_c_abi_argument_errors(pkg):
     assert lib.tq_decompress_batched(None, None, 0, 128, None, None) == 0
     assert lib.tq_decompress_batched(None, None, 3, 128, None, None) == E["NULL"]
     assert lib.tq_decompress_batched(p, p, 3, 128, p64 + 32, None) == E["ALIGN"]
-    assert lib.tq_compress_batched(None, None, 0, 128, None) == 0
-    assert lib.tq_compress_batched(None, None, 3, 128, None) == E["NULL"]
+    assert call(p, 1, 4, 128, ws=p64 + 16) == E["ALIGN"]              # workspace: 64-byte aligned
+    assert lib.tq_compress_batched(None, None, 0, 128, None, None) == 0
+    assert lib.tq_compress_batched(None, None, 3, 128, None, None) == E["NULL"]
+    assert lib.tq_compress_batched(p, p, 3, 128, p64 + 32, None) == E["ALIGN"]
     # the decode-step ends: (queries, q_dtype, rows, group, scale, pi_k_t, k_win, v_win, win_dtype, n_win, win_stride, q_rot, part_w)
     prep = lambda q=p, g=4, pit=p, kw=p, vw=p, wd=2, nw=8, ws=1024, qr=p, pw=p, rows=1, qd=2: lib.tq_attend_prepare(
         q, qd, rows, g, 0.5, pit, kw, vw, wd, nw, ws, qr, pw, None)

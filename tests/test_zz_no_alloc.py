@@ -77,17 +77,19 @@ def _run_case(pkg, lib, oracle, bits, counts, seed):
     ha, da = upload(jobs_a)
     hb, db = upload(jobs_b)
     nj = len(counts)
-    rc = lib.tq_compress_batched(hc, _p(dc), nj, D, stream)
+    rc = lib.tq_compress_batched(hc, _p(dc), nj, D, None, stream)
     assert rc == 0, lib.tq_status_string(rc)
     ws = torch.zeros(lib.tq_workspace_bytes(nj), dtype=torch.uint8, device=DEV)
     rc = lib.tq_decompress_batched(ha, _p(da), nj, D, _p(ws), stream)
     assert rc == 0, lib.tq_status_string(rc)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # "allocates nothing" is a statement about the driver, not about torch's caching allocator (which a hipMalloc
+    # inside the library would never touch): the device's free memory is read before and after the call
+    free_before = torch.cuda.mem_get_info()[0]
     rc = lib.tq_decompress_batched_noalloc(hb, _p(db), nj, D, stream)
     assert rc == 0, lib.tq_status_string(rc)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     for a, b in zip(outs_a, outs_b):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     # and the bytes are the right ones: the first job against the oracle's decode of the same packed bytes
@@ -109,6 +111,43 @@ def test_noalloc_equals_workspace_form_twice_second_smaller(tq, oracle):
     _run_case(pkg, lib, oracle, 2, [131072 + 5, 131072], seed=2)
     # third: tiny jobs (fixed assignment of tiles inside the kernel), ragged sizes, an empty job in the list
     _run_case(pkg, lib, oracle, 8, [33, 0, 1000], seed=3)
+
+
+def test_noalloc_call_can_be_captured_into_a_graph(tq):
+    """Stream capture fails on any allocation or synchronising call: a call recorded into a HIP graph, after an eager
+    call has looked up the library's counters, replays to the bytes of the workspace form, three times over with the
+    program's own work and synchronisations in between."""
+    pkg, lib = tq
+    bits, n = 4, 131072 + 40
+    G = lib.tq_bytes_per_vector(D, bits)
+    table, pi, cent = _table(pkg, lib, bits, seed=77)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(n, D, generator=g).to(torch.bfloat16).to(DEV)
+    idx = torch.empty(n, G, dtype=torch.uint8, device=DEV)
+    nrm = torch.empty(n, dtype=torch.float16, device=DEV)
+    ref = torch.empty(n, D, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty(n, D, dtype=torch.bfloat16, device=DEV)
+    mk = lambda t: (Job * 1)(Job(t.data_ptr(), idx.data_ptr(), nrm.data_ptr(), table.data_ptr(), 1, n, 0, D, bits, 2, 0))
+    up = lambda h: torch.from_numpy(np.frombuffer(bytes(h), dtype=np.uint8).copy()).to(DEV)
+    hc, hr, ho = mk(x), mk(ref), mk(out)
+    dc, dr, do = up(hc), up(hr), up(ho)
+    cur = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert lib.tq_compress_batched(hc, _p(dc), 1, D, None, cur()) == 0
+    ws = torch.zeros(lib.tq_workspace_bytes(1), dtype=torch.uint8, device=DEV)
+    assert lib.tq_decompress_batched(hr, _p(dr), 1, D, _p(ws), cur()) == 0
+    assert lib.tq_decompress_batched_noalloc(ho, _p(do), 1, D, cur()) == 0       # eager: looks the counters up
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):           # captures on a side stream, which is the current one inside the block
+        rc = lib.tq_decompress_batched_noalloc(ho, _p(do), 1, D, cur())
+    assert rc == 0, lib.tq_status_string(rc)
+    for _ in range(3):
+        out.fill_(3.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
 
 
 def test_noalloc_rejects_what_it_cannot_hold(tq):

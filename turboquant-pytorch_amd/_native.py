@@ -36,33 +36,83 @@ class TqError(RuntimeError):
 # ------------------------------------------------------------------------------------
 # build
 # ------------------------------------------------------------------------------------
-def hipcc_command(out_path: str = LIB_PATH) -> List[str]:
-    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    return [
-        hipcc, "-shared", "-fPIC", "-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}",
-        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-        "-Wno-unused-command-line-argument",
-        "-Wno-inline-asm",      # the direct-to-LDS loads name m0 as clobbered, which clang reports as a reserved register
-        *[os.path.join(CSRC, s) for s in SOURCES],
-        "-o", out_path,
-    ]
+OBJ_DIR = os.path.join(CSRC, "build")
+# The "memory skeleton" build of the two codec kernels: same loads, LDS traffic, barriers and stores, with the matrix
+# instructions and the code search (compress) or the decode, matrix instructions and operand reads (decompress) left
+# out.  Its output is garbage; it exists to time what the memory pattern alone costs (bench.py --skeleton).
+SKELETON_LIB_PATH = os.path.join(CSRC, "libtqamd_skeleton.so")
+SKELETON_SOURCES = ("tq_compress.hip", "tq_decompress.hip")
+SKELETON_DEFINES = ("-DTQ_SKELETON=1",)
+
+
+def hipcc_flags() -> List[str]:
+    return ["-fPIC", "-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}",
+            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+            "-Wno-unused-command-line-argument",
+            # The ticket draws are single-lane atomics whose result is needed a tile's work later.  The atomic optimizer
+            # would turn each into a wave-wide scan with a read-first-lane of the result, i.e. a wait for every memory
+            # operation of the wave right behind the atomic.
+            "-mllvm", "-amdgpu-atomic-optimizer-strategy=None",
+            "-Wno-inline-asm"]      # the direct-to-LDS loads name m0 as clobbered, which clang reports as a reserved register
+
+
+def _hipcc() -> str:
+    return shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+
+def _run(cmd: List[str]) -> str:
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    return res.stderr
+
+
+def _compile_objects(tag: str, defines: Sequence[str], only: Optional[Sequence[str]], force: bool, verbose: bool) -> Dict[str, str]:
+    """One object per source under csrc/build, compiled side by side; `only`: the sources that take `defines`
+    (their objects carry `tag` in the name), the others are the plain objects.  Up-to-date objects are kept unless `force`."""
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    newest_header = max(os.path.getmtime(os.path.join(CSRC, h)) for h in HEADERS)
+    jobs, objs = [], {}
+    for src in SOURCES:
+        special = bool(defines) and (only is None or src in only)
+        obj = os.path.join(OBJ_DIR, src + ("." + tag if special else "") + ".o")
+        objs[src] = obj
+        path = os.path.join(CSRC, src)
+        if not force and os.path.exists(obj) and os.path.getmtime(obj) >= max(os.path.getmtime(path), newest_header):
+            continue
+        jobs.append([_hipcc(), *hipcc_flags(), *(defines if special else ()), "-c", path, "-o", obj])
+    if jobs:
+        with ThreadPoolExecutor(max_workers=min(len(jobs), max(1, (os.cpu_count() or 2) - 1))) as pool:
+            for err in pool.map(_run, jobs):
+                if verbose and err:
+                    print(err)
+    return objs
+
+
+def _link(objs: Dict[str, str], out_path: str) -> None:
+    tmp = out_path + ".tmp"
+    _run([_hipcc(), "-shared", "-fPIC", f"--offload-arch={GPU_ARCH}", *objs.values(), "-o", tmp])
+    os.replace(tmp, out_path)
 
 
 def build(force: bool = True, verbose: bool = False) -> str:
-    """Compile the HIP/C++ sources into csrc/libtqamd.so (cross-compiles without a GPU)."""
+    """Compile the HIP/C++ sources into csrc/libtqamd.so (cross-compiles without a GPU): one object per source,
+    compiled in parallel, then linked."""
     if not force and os.path.exists(LIB_PATH):
         newest = max(os.path.getmtime(os.path.join(CSRC, f)) for f in SOURCES + HEADERS)
         if os.path.getmtime(LIB_PATH) >= newest:
             return LIB_PATH
-    tmp = LIB_PATH + ".tmp"
-    cmd = hipcc_command(tmp)
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
-    if verbose and res.stderr:
-        print(res.stderr)
-    os.replace(tmp, LIB_PATH)
+    _link(_compile_objects("", (), None, force, verbose), LIB_PATH)
     return LIB_PATH
+
+
+def build_skeleton(force: bool = True, verbose: bool = False) -> str:
+    """csrc/libtqamd_skeleton.so: the library with the memory-skeleton form of the compress and decompress kernels
+    (a measurement aid, never loaded by the package itself)."""
+    _compile_objects("", (), None, False, verbose)                       # the plain objects, if a build has not left them
+    _link(_compile_objects("skeleton", SKELETON_DEFINES, SKELETON_SOURCES, force, verbose), SKELETON_LIB_PATH)
+    return SKELETON_LIB_PATH
 
 
 # ------------------------------------------------------------------------------------
@@ -118,11 +168,11 @@ def lib() -> ctypes.CDLL:
     L.tq_table_build.argtypes = [vp, vp, ci, ci, vp, ctypes.c_size_t]
     L.tq_table_check.argtypes = [vp, ctypes.c_size_t, ci, ci]
     L.tq_table_quantize_host.argtypes = [vp, vp, ll, vp]
-    L.tq_compress.argtypes = [vp, ci, ll, ll, ll, ll, vp, ci, ci, vp, vp, ll, vp]
+    L.tq_compress.argtypes = [vp, ci, ll, ll, ll, ll, vp, ci, ci, vp, vp, ll, vp, vp]
     L.tq_decompress.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, ll, ll, vp, vp]
     L.tq_workspace_bytes.restype = ll
     L.tq_workspace_bytes.argtypes = [ci]
-    L.tq_compress_batched.argtypes = [vp, vp, ci, ci, vp]
+    L.tq_compress_batched.argtypes = [vp, vp, ci, ci, vp, vp]
     L.tq_scores.argtypes = [vp, vp, ll, ll, ll, vp, ci, ci, vp, ci, vp, ll, vp]
     L.tq_weighted_values_splits.argtypes = [ll, ll]
     L.tq_attend_splits.argtypes = [ll, ll]
@@ -181,22 +231,24 @@ def build_table(Pi: torch.Tensor, centroids: torch.Tensor, bits: int) -> np.ndar
 
 # The launch entry points take a table in device memory and a bit width that selects the kernel; nothing on the
 # device side can tell them apart when they disagree (the codes would be garbage, silently).  Every table this
-# module uploads is therefore remembered with the width it was built for, and every launch checks its pair.
-_table_widths: Dict[int, Tuple[int, int]] = {}     # device address of an uploaded table -> (head_dim, bits)
+# module uploads therefore carries the width it was built for as an attribute of the tensor object, and every launch
+# checks its pair.  (The tag lives and dies with the tensor: a map keyed by device address would keep entries of
+# freed tables, and a later upload that the allocator places at the same address would meet a stale one.)
+_TABLE_TAG = "_tq_table_width"
 
 
 def upload_table(blob: np.ndarray, head_dim: int, bits: int, device: torch.device) -> torch.Tensor:
     """Device copy of a blob from build_table, after tq_table_check(blob, head_dim, bits)."""
     check(lib().tq_table_check(blob.ctypes.data, blob.size, head_dim, bits), "tq_table_check")
     t = torch.from_numpy(blob).to(device)
-    _table_widths[t.data_ptr()] = (head_dim, bits)
+    setattr(t, _TABLE_TAG, (head_dim, bits))
     return t
 
 
 def check_table(table: torch.Tensor, head_dim: int, bits: int) -> None:
     """Raises if `table` was uploaded for another (head_dim, bits).  Tables this module never saw (a caller's own
     upload) pass: their owner has to make the check, with tq_table_check on the host copy."""
-    known = _table_widths.get(table.data_ptr())
+    known = getattr(table, _TABLE_TAG, None)
     if known is not None and known != (head_dim, 8 if bits > 8 else bits):
         raise TqError(f"codec table built for head_dim {known[0]}, {known[1]} bits used with head_dim {head_dim}, {bits} bits")
 
@@ -324,7 +376,7 @@ _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
 def _workspace(device: torch.device, stream: int) -> int:
-    """Address of the ticket counters tq_decompress draws its tiles from, or 0 (fixed assignment of tiles).
+    """Address of the ticket counters tq_compress / tq_decompress draw their tiles from, or 0 (fixed assignment of tiles).
     One zero-filled buffer per (device, stream): launches on one stream run one after the other and each
     leaves the counters at zero, launches on different streams never share.  While a graph is being
     captured the answer is 0: the graph may be replayed on any stream, next to eager launches on this one."""
@@ -378,9 +430,14 @@ def compress_into(states: torch.Tensor, table: torch.Tensor, bits: int,
     rows, tokens, row_stride, token_stride = lay
     check_table(table, states.shape[-1], bits)
     with _on(states.device):
+        stream = _stream_handle(states.device)
+        # counters only where the kernel can use them (a large single-row job): a one-token append needs no look-up
+        ws = _workspace(states.device, stream) if rows == 1 and tokens >= 65536 else 0
         rc = lib().tq_compress(states.data_ptr(), dtype_code(states.dtype), rows, tokens, row_stride, token_stride,
                                table.data_ptr(), states.shape[-1], bits,
-                               idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, _stream_handle(states.device))
+                               idx_bytes.data_ptr(), vec_norms.data_ptr(), prs, ws, stream)
+    if rc and ws:
+        _drop_workspace(states.device, stream)
     check(rc, "tq_compress")
 
 
@@ -689,14 +746,16 @@ class JobList:
             self._keep.append((t, j["idx_bytes"], j["vec_norms"], j["table"]))
         raw = np.frombuffer(bytes(self.host), dtype=np.uint8).copy()
         self.dev = torch.from_numpy(raw).to(self.device)
-        # ticket counters of the decompress launch, one record per job; zero now, and every launch leaves them zero.
-        # Launches of one list write the same outputs, so they never overlap and can share the counters.
+        # ticket counters of the launches, one record per job; zero now, and every launch leaves them zero.
+        # Launches of one list read or write the same buffers, so they never overlap and can share the counters.
         self.workspace = torch.zeros(int(lib().tq_workspace_bytes(self.n)), dtype=torch.uint8, device=self.device)
 
     def compress(self) -> None:
         with _on(self.device):
             rc = lib().tq_compress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, self.head_dim,
-                                           _stream_handle(self.device))
+                                           self.workspace.data_ptr(), _stream_handle(self.device))
+        if rc:
+            self.workspace.zero_()      # counters of a launch that did not complete are not trusted
         check(rc, "tq_compress_batched")
 
     def decompress(self) -> None:

@@ -26,10 +26,20 @@ def _qjl_matrix(head_dim: int, seed: int) -> torch.Tensor:
     return torch.randn(head_dim, head_dim, generator=gen)
 
 
+def _check_v2_bits(bits: int) -> None:
+    """The kernels of the key path take MSE codes of 1 ... 7 bits (bits - 1 of them: the packings of the V3 codec,
+    decoded through a 128-entry-per-half table), so `bits` is 1 ... 8.  The reference also constructs with bits = 9
+    (256 levels in a uint8 index, compressors.py:38-47); here that is a clear error at construction."""
+    if not 1 <= int(bits) <= 8:
+        raise ValueError(f"TurboQuantCompressorV2: bits must be 1 ... 8 on this implementation (got {bits}); "
+                         "the reference's bits = 9 (8-bit MSE codes plus the sign bit) is not supported")
+
+
 class TurboQuantCompressorV2:
     """Keys for asymmetric attention: interface of compressors.py:25-158."""
 
     def __init__(self, head_dim: int, bits: int, seed: int, device: str = "cpu"):
+        _check_v2_bits(bits)
         self.head_dim = head_dim
         self.bits = bits
         self.mse_bits = max(bits - 1, 1)
@@ -41,6 +51,7 @@ class TurboQuantCompressorV2:
     @classmethod
     def from_tensors(cls, Pi: torch.Tensor, S: torch.Tensor, centroids: torch.Tensor, bits: int, device: str = "cpu"):
         """A compressor over explicit matrices and codebook (parity tests pass the reference's own through here)."""
+        _check_v2_bits(bits)
         self = cls.__new__(cls)
         self.head_dim = Pi.shape[0]
         self.bits = bits
@@ -98,8 +109,10 @@ class TurboQuantCompressorV2:
         "residual_norm" f16 [B,H,S], "shape"}.  Two launches: MSE codes and norms, then residual signs and norms."""
         B, H, S, D = states.shape
         _native._require_gpu(states, "states")
-        if not states.is_contiguous() or states.data_ptr() % 16:
+        if not states.is_contiguous():
             states = states.contiguous()
+        if states.data_ptr() % 16:       # a contiguous view into the middle of a buffer: contiguous() would hand it back as it is
+            states = states.clone(memory_format=torch.contiguous_format)
         first = self._mse.compress(states)
         sign_bytes = torch.empty((B, H, S, D // 8), dtype=torch.uint8, device=states.device)
         residual_norm = torch.empty((B, H, S), dtype=torch.float16, device=states.device)

@@ -8,7 +8,8 @@ reached through the C ABI in include/tqamd.h.  There is no CPU path: tensors mus
 HIP device.
 
 Differences a caller can observe, all deliberate:
-  * `device` defaults to "cuda" (the reference defaults to "cpu").
+  * `device` (default "cpu", as in the reference) says where `Pi` and `centroids` live; the kernels
+    run on the device of the tensors they are given, with their tables uploaded there on first use.
   * Codebooks and rotations are cached per (head_dim, bits) / (head_dim, seed); the reference
     re-solves them for every instance.  Values are identical.
   * `TurboQuantV3.decompress_kv` writes the de-quantised tokens straight into the

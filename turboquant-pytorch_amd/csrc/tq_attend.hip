@@ -1376,10 +1376,10 @@ extern "C" int tq_append_token(const void *k_new, const void *v_new, int dtype, 
         const uint8_t *kw = static_cast<const uint8_t *>(k_win) + evict * TQ_HEAD_DIM * eb;
         const uint8_t *vw = static_cast<const uint8_t *>(v_win) + evict * TQ_HEAD_DIM * eb;
         int rc = tq_compress(kw, dtype, rows, 1, win_stride, TQ_HEAD_DIM, table_k, head_dim, bits_k,
-                             k_idx + packed_slot * gk, k_norms + packed_slot, packed_row_stride, stream);
+                             k_idx + packed_slot * gk, k_norms + packed_slot, packed_row_stride, nullptr, stream);
         if (rc) return rc;
         rc = tq_compress(vw, dtype, rows, 1, win_stride, TQ_HEAD_DIM, table_v, head_dim, bits_v,
-                         v_idx + packed_slot * gv, v_norms + packed_slot, packed_row_stride, stream);
+                         v_idx + packed_slot * gv, v_norms + packed_slot, packed_row_stride, nullptr, stream);
         if (rc) return rc;
     }
     const uint32_t pieces = (uint32_t)(TQ_HEAD_DIM * eb / 16);

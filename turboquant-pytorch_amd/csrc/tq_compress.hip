@@ -44,6 +44,12 @@ namespace {
 #ifndef TQ_PRIO_SHIFT
 #define TQ_PRIO_SHIFT 3
 #endif
+// Measurement build (never the shipped library): the pipelined path keeps its loads, LDS traffic, barriers, norm
+// arithmetic and stores, and leaves out the matrix instructions and the code search.  What it writes is garbage; its
+// time is what the kernel's memory pattern costs on its own.
+#ifndef TQ_SKELETON
+#define TQ_SKELETON 0
+#endif
 template <int DTYPE> struct InTraits;
 template <> struct InTraits<TQ_F16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = TQ_C16_WAVES; };
 template <> struct InTraits<TQ_BF16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = TQ_C16_WAVES; };
@@ -107,7 +113,8 @@ __device__ __forceinline__ bool run_tail(F &step) {
 }
 
 template <int DTYPE, int BITS>
-__global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compress_kernel(TqDevJob job0, const tq_job *jobs) {
+__global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t *workspace,
+                                                                                          uint32_t tshift) {
     using T = InTraits<DTYPE>;
     using P = Pack<BITS>;
     constexpr int ELEM = T::ELEM;
@@ -131,8 +138,33 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     const uint32_t lane = tid & 63u;
     const uint32_t wave = tid >> 6;
     const uint32_t n_tiles = (job.n_vec + 31u) / 32u;
-    uint32_t tile = blockIdx.x;
-    if (tile >= n_tiles) return;  // whole block idle (uniform)
+    if (n_tiles == 0u) return;    // an empty job of a batch: its table may be NULL, and its counters stay untouched (zero)
+    const uint32_t n_full = job.n_vec / 32u;
+    const bool one_row = job.tokens >= job.n_vec;
+    // Which tiles a block works on.  Single-row jobs of 16-bit elements (the pipelined path below) hand their tiles out
+    // as tickets of 2^tshift consecutive tiles: block b starts with ticket b; its later tickets are b + grid, b + 2 grid, ...
+    // (fixed assignment) or, with a workspace, come from a counter in device memory in the order in which the blocks
+    // ask, so that compute units that run slower than others (the dies of this part do not all run at one pace) take
+    // fewer tiles and all blocks of a job end together.  counter[0] = tiles handed out beyond every block's first ticket,
+    // counter[1] = blocks of the job that are done; the last block to finish sets both back to zero, so a workspace
+    // that was zero before a launch is zero after it (the contract of the decompress kernel's counters).
+    // Every other job walks single tiles blockIdx.x, blockIdx.x + grid, ...
+    const bool ticket_job = ELEM == 2 && one_row && job.token_stride < (1ll << 26);
+    // (a ticket has to outlast the pipeline's depth: the first drawn ticket is published one iteration after the start)
+    uint32_t *counter = workspace && (1u << tshift) > (uint32_t)TQ_RING ? workspace + blockIdx.y * (TQ_WORKSPACE_BYTES_PER_JOB / 4) : nullptr;
+    auto report_done = [&]() {      // once per block of a non-empty job, after its last draw has been answered
+        if (counter && tid == 0) {
+            if (atomicAdd(counter + 1, 1u) == gridDim.x - 1u) {
+                atomicExch(counter, 0u);
+                atomicExch(counter + 1, 0u);
+            }
+        }
+    };
+    uint32_t tile = ticket_job ? blockIdx.x << tshift : blockIdx.x;
+    if (tile >= n_tiles) {        // whole block idle (uniform)
+        report_done();
+        return;
+    }
     const uint32_t tile_stride = gridDim.x;
 
     const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
@@ -179,7 +211,6 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
 
     const uint32_t ld_vec = lane / PIECES, ld_piece = lane % PIECES;  // role in the coalesced loads
     const uint32_t n = lane & 31u, hk = lane >> 5;                    // role in the MFMA: column, half
-    const bool one_row = job.tokens >= job.n_vec;
 
     // LDS offset of this lane's piece of load j (computed where it is used: these paths are not the hot one)
     auto st_off = [&](int j) {
@@ -355,13 +386,11 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     };
     const uint32_t lane_slot = (2u * wave + hk) * NB;   // this lane's bytes inside a vector's G = 8 * NB
 
-    const uint32_t n_full = job.n_vec / 32u;
     uint32_t buf = 0;
     uint32_t words[NW];
     float nrm;
-    // the pipelined path addresses a tile's vectors with 32-bit offsets from a scalar base
-    const bool dma_ok = one_row && job.token_stride < (1ll << 26);
-    const bool pipelined = tile < n_full && ELEM == 2 && dma_ok;
+    // (the pipelined path addresses a tile's vectors with 32-bit offsets from a scalar base: the stride limit of ticket_job)
+    const bool pipelined = ticket_job && tile < n_full;
     if (!pipelined) load_tables();
     if (pipelined) {
         if constexpr (ELEM == 2) {
@@ -382,8 +411,6 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             // 2 stores per iteration.
             constexpr int P = RING;
             static_assert(NLOAD == 2 && P >= 2 && P <= 6, "the wait counts below assume two loads per wave and tile");
-            const uint32_t m = (n_full - tile + tile_stride - 1u) / tile_stride;   // this block's full tiles
-            const long long in_step = (long long)tile_stride * 32 * job.token_stride;
             // lane i of load j fills bytes [16 i, 16 i + 16) of KiB (wave * NLOAD + j) of the slot: vector
             // vl = (wave * NLOAD + j) * 4 + i / 16, position i % 16, which has to hold piece (i % 16) ^ (vl & 15)
             uint32_t src_off[NLOAD];
@@ -394,11 +421,53 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             }
             const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
                 (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)&lds_stage[0][0] + wave * (NLOAD * 1024u));
-            const uint8_t *src = job.states + (long long)tile * 32 * job.token_stride;   // the same in every lane
-            uint32_t ahead = m - 1u;      // tiles beyond the one `src` points at
-            // past the block's last tile the pointer stays where it is: a harmless re-read, never used
-            auto issue = [&](uint32_t slot) {
-                const uint64_t a = (uint64_t)(uintptr_t)src;
+
+            // ---- the block's sequence of tiles.  q[i] = the tile of iteration j - 1 + i while iteration j runs: q[0] is
+            // searched and stored, q[1] rotated, q[P] loaded.  All of it lives in scalar registers.  A value >= n_full
+            // marks the end (the sequence of a block only grows); loads past the end re-read the job's last full tile.
+            __shared__ uint32_t tk[4];          // ticket k of the block sits in slot k % 4 (counter mode only)
+            const uint32_t per_ticket = 1u << tshift;
+            const uint32_t drawn_origin = gridDim.x << tshift;
+            uint32_t q[P + 1];
+            uint32_t left = per_ticket - 1u;    // tiles of the head's ticket beyond the head
+            uint32_t kt = 0;                    // tickets the head has entered beyond the first
+            uint32_t drawn = 0;                 // thread 0: what the atomic of this iteration's draw returned, not yet looked at
+            bool have_drawn = false;
+            auto draw = [&]() {                 // counter mode; the value is taken by thread 0 alone
+                // (the returned value stays untouched until publish(): arithmetic on it here would put a wait for all of
+                // the wave's memory operations right behind the atomic)
+                if (tid == 0) drawn = atomicAdd(counter, per_ticket);
+                have_drawn = true;
+            };
+            auto publish = [&]() {              // at the end of an iteration: the draw's latency hides behind the tile's work
+                if (have_drawn) {
+                    if (tid == 0) tk[(kt + 1u) & 3u] = drawn_origin + drawn;
+                    have_drawn = false;
+                }
+            };
+            auto advance = [&](uint32_t head) -> uint32_t {    // the tile after `head` in this block's sequence
+                if (left) {
+                    --left;
+                    return head + 1u;
+                }
+                left = per_ticket - 1u;
+                ++kt;
+                if (counter) {
+                    // ticket kt was drawn when the head entered ticket kt - 1, at least four iterations (one barrier) ago
+                    const uint32_t base = (uint32_t)__builtin_amdgcn_readfirstlane(tk[kt & 3u]);
+                    draw();
+                    return base;
+                }
+                return (blockIdx.x + kt * gridDim.x) << tshift;
+            };
+            q[0] = 0xffffffffu;
+            q[1] = tile;
+#pragma unroll
+            for (int i = 2; i <= P; ++i) q[i] = advance(q[i - 1]);     // (counter mode: tickets hold more than P tiles, no draw here)
+            if (counter) draw();                // ticket 1: in LDS at the end of the first iteration, read per_ticket - P iterations later
+            auto issue = [&](uint32_t slot, uint32_t tl) {
+                tl = tl < n_full ? tl : n_full - 1u;
+                const uint64_t a = (uint64_t)(uintptr_t)job.states + (uint64_t)tl * (uint64_t)(32 * job.token_stride);
                 // (the builtin returns int: widen through uint32_t, or the low half is sign-extended into the high one)
                 const uint32_t a_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
                 const uint32_t a_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)a);
@@ -409,8 +478,6 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
                     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                                  :: "s"(dst), "v"(src_off[j]), "s"(base) : "memory", "m0");
                 }
-                src += ahead ? in_step : 0;
-                ahead -= ahead ? 1u : 0u;
             };
             // operand addresses inside a slot, in this wave's step order
             uint32_t op_off[TQ_STEPS];
@@ -421,11 +488,11 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             }
             const uint32_t bperm_other_half = (lane ^ 32u) << 2;
 
-            // output addresses: a base that is the same in every lane, advanced per tile, plus a per-lane constant
-            uint8_t *cd = job.idx_bytes + (size_t)tile * 32u * (8 * NB);
-            uint16_t *nd = job.vec_norms + (size_t)tile * 32u;
+            // output addresses: a base per tile that is the same in every lane, plus a per-lane constant
             const uint32_t cd_lane = n * (8 * NB) + lane_slot, nd_lane = n;
-            const size_t cd_step = (size_t)tile_stride * 32u * (8 * NB), nd_step = (size_t)tile_stride * 32u;
+            auto store_tile = [&](uint32_t tl, const uint32_t (&w)[NW], float nrm_of_tile) {
+                store(job.idx_bytes + (size_t)tl * (32u * (8 * NB)) + cd_lane, job.vec_norms + (size_t)tl * 32u + nd_lane, w, nrm_of_tile);
+            };
 
             auto scale_from_shares = [&](uint32_t par) {
                 const float4 q = *reinterpret_cast<const float4 *>(&lds_part[par][n][0]);
@@ -438,11 +505,16 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
                 // younger than the loads of t_j: the loads of P-2 tiles and, once the pipeline is full, the stores of P-1
                 if (warm) wait_vmcnt<2 * (P - 2) + 2 * (P - 1)>(); else wait_vmcnt<2 * (P - 2)>();
                 __syncthreads();
-                issue((SLOT + P - 1u) % P);
+                issue((SLOT + P - 1u) % P, q[P]);
+                const uint32_t head_next = advance(q[P]);
                 const uint8_t *stage = lds_stage[SLOT];
                 auto operand = [&](int i) { return *reinterpret_cast<const tq_u4 *>(stage + op_off[i]); };
                 auto mfma = [&](int term, int i, tq_u4 bop) {
+#if TQ_SKELETON
+                    if (term == 0) acc_new[i] = __uint_as_float(bop[0] ^ bop[1] ^ bop[2] ^ bop[3]);     // the operand read stays alive
+#else
                     acc_new = (DTYPE == TQ_F16) ? mfma_f16(areg[term][i], bop, acc_new) : mfma_bf16(areg[term][i], bop, acc_new);
+#endif
                 };
                 acc_new = tq_zero16();
                 Search z;
@@ -459,24 +531,24 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
                     tq_u4 bop_next = bop;
                     tq_u2 n0 = c0, n1 = c1;
                     if (i + 1 < TQ_STEPS) bop_next = operand(i + 1);
-                    if constexpr (SEARCH) {
+                    if constexpr (SEARCH && !TQ_SKELETON) {
                         if (i >= 1) { n0 = search_lookup(2 * i - 2, acc_old, sc_old); n1 = search_lookup(2 * i - 1, acc_old, sc_old); }
                     }
                     mfma(0, i, bop);
                     if (i < 2) share = sumsq8<DTYPE>(bop, share);
                     if constexpr (SEARCH) {
                         if (i == 0) sc_old = scale_from_shares(par ^ 1u);
-                        if (i >= 2) search_apply(z, 2 * i - 4, acc_old, sc_old, c0);
+                        if (i >= 2 && !TQ_SKELETON) search_apply(z, 2 * i - 4, acc_old, sc_old, c0);
                     }
                     mfma(1, i, bop);
-                    if constexpr (SEARCH) {
+                    if constexpr (SEARCH && !TQ_SKELETON) {
                         if (i >= 2) search_apply(z, 2 * i - 3, acc_old, sc_old, c1);
                     }
                     if (i == 1) {
                         share += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((int)bperm_other_half, __builtin_bit_cast(int, share)));
                         lds_part[par][n][wave] = share;
                     }
-#if TQ_PIN_SCHEDULE
+#if TQ_PIN_SCHEDULE && !TQ_SKELETON
                     if constexpr (SEARCH) {
                         // pin the order: address arithmetic, the step's LDS reads, then each MFMA followed by the
                         // VALU work that fills its shadow
@@ -505,15 +577,22 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
                     bop = bop_next; c0 = n0; c1 = n1;
                 }
                 if constexpr (SEARCH) {
+#if TQ_SKELETON
+#pragma unroll
+                    for (int w = 0; w < NW; ++w) words[w] = __float_as_uint(acc_old[w] * sc_old.inv);
+#else
                     search_apply(z, 12, acc_old, sc_old, c0);
                     search_apply(z, 13, acc_old, sc_old, c1);
                     search_coord(z, 14, acc_old, sc_old);
                     search_coord(z, 15, acc_old, sc_old);
                     search_end(z, words);
-                    store(cd + cd_lane, nd + nd_lane, words, sc_old.nrm);
-                    cd += cd_step;
-                    nd += nd_step;
+#endif
+                    store_tile(q[0], words, sc_old.nrm);
                 }
+                publish();
+#pragma unroll
+                for (int i = 0; i < P; ++i) q[i] = q[i + 1];
+                q[P] = head_next;
             };
             auto drain = [&](uint32_t par, const tq_f16v &acc_old) {    // par: parity of the iteration that would come next
                 __syncthreads();    // the last tile's shares of the sum of squares are complete
@@ -523,11 +602,11 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
 #pragma unroll
                 for (int q = 0; q < 16; ++q) search_coord(z, q, acc_old, sc_old);
                 search_end(z, words);
-                store(cd + cd_lane, nd + nd_lane, words, sc_old.nrm);
+                store_tile(q[0], words, sc_old.nrm);
             };
 
 #pragma unroll
-            for (int p = 0; p < P - 1; ++p) issue((uint32_t)p);
+            for (int p = 0; p < P - 1; ++p) issue((uint32_t)p, q[1 + p]);
             load_tables();      // (the waits for these loads also cover the older tile loads: harmless, once per block)
             tq_f16v acc_a, acc_b;
             uint32_t done = 0;     // iterations finished
@@ -544,7 +623,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             const uint32_t age = ((blockIdx.y * gridDim.x + blockIdx.x) * RES) / (gridDim.x * gridDim.y);
             auto step = [&](auto k_tag) -> bool {    // true = all tiles rotated
                 constexpr uint32_t K = decltype(k_tag)::value;
-                if (done == m) return true;
+                if (q[1] >= n_full) return true;
                 if constexpr (K == 0 && TQ_PRIO_SHIFT > 0) {
                     if ((done & ((1u << TQ_PRIO_SHIFT) - 1u)) == 0u) {
                         const uint32_t prio = (age + (done >> TQ_PRIO_SHIFT)) % RES;
@@ -564,10 +643,10 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             if (done & 1u) drain(1u, acc_a); else drain(0u, acc_b);
             wait_vmcnt<0>();       // re-reads past the last tile may still be on their way into the ring
             __syncthreads();
-            tile += m * tile_stride;
+            tile = q[1];           // where the sequence left the full tiles: n_full itself in the one block whose turn the partial tile is
             buf = 0u;
         }
-    } else if (tile < n_full) {
+    } else if (!ticket_job && tile < n_full) {
         // General case (several rows with their own stride, fp32 elements).  Iteration k: start the
         // loads of tile k+1, barrier (publishes buffer k, and everyone has finished reading buffer
         // k-1), compute and store tile k, then park tile k+1 into the other buffer.  Loads, stores
@@ -598,6 +677,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             store(job.idx_bytes + (size_t)slot * (8 * NB) + lane_slot, job.vec_norms + slot, words, nrm);
         }
     }
+    report_done();
 }
 
 // ---- host side --------------------------------------------------------------------------
@@ -631,8 +711,12 @@ int query_device(DeviceInfo &info) {
     return 0;
 }
 
+#ifndef TQ_COMPRESS_TICKET_SHIFT
+#define TQ_COMPRESS_TICKET_SHIFT 3
+#endif
+
 template <int DTYPE, int BITS>
-int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t stream) {
+int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *workspace, hipStream_t stream) {
     DeviceInfo info;
     int rc = query_device(info);
     if (rc) return rc;
@@ -650,30 +734,43 @@ int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uin
         }
         resident = resident_on[info.dev];
     }
-    const uint32_t bx = tq_blocks_per_job(max_tiles, info.cus * resident, n_jobs);
+    // Tickets from a counter pay off once every block has several to draw; below that (and without a workspace) the
+    // blocks walk single tiles b, b + grid, ..., which splits a small job most evenly.
+    uint32_t bx = tq_blocks_per_job(max_tiles, info.cus * resident, n_jobs);
+    uint32_t tshift = 0;
+    uint32_t *counters = nullptr;
+    if (workspace && InTraits<DTYPE>::ELEM == 2 && TQ_COMPRESS_TICKET_SHIFT > 0) {
+        const uint32_t tickets = (max_tiles + (1u << TQ_COMPRESS_TICKET_SHIFT) - 1u) >> TQ_COMPRESS_TICKET_SHIFT;
+        const uint32_t bt = tq_blocks_per_job(tickets, info.cus * resident, n_jobs);
+        if (tickets >= 4u * bt) {
+            bx = bt;
+            tshift = TQ_COMPRESS_TICKET_SHIFT;
+            counters = static_cast<uint32_t *>(workspace);
+        }
+    }
     dim3 grid(bx, (unsigned)n_jobs, 1), block(CTHREADS, 1, 1);
-    hipLaunchKernelGGL((tq_compress_kernel<DTYPE, BITS>), grid, block, 0, stream, job, jobs_dev);
+    hipLaunchKernelGGL((tq_compress_kernel<DTYPE, BITS>), grid, block, 0, stream, job, jobs_dev, counters, tshift);
     return (int)hipGetLastError();
 }
 
 template <int DTYPE>
-int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t s) {
+int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, hipStream_t s) {
     switch (bits) {
-        case 1: return launch_compress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, s);
-        case 2: return launch_compress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, s);
-        case 3: return launch_compress<DTYPE, 3>(job, jobs_dev, n_jobs, max_tiles, s);
-        case 4: return launch_compress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, s);
+        case 1: return launch_compress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case 2: return launch_compress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case 3: return launch_compress<DTYPE, 3>(job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case 4: return launch_compress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, ws, s);
         case 5: case 6: case 7: case 8:  // one code per byte: identical packing
-            return launch_compress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, s);
+            return launch_compress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, ws, s);
         default: return TQ_ERR_BITS;
     }
 }
 
-int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, hipStream_t s) {
+int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, hipStream_t s) {
     switch (dtype) {
-        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, s);
-        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, s);
-        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, s);
+        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
         default: return TQ_ERR_DTYPE;
     }
 }
@@ -707,11 +804,13 @@ int check_job(const void *states, int dtype, long long rows, long long tokens, l
 extern "C" int tq_compress(const void *states, int dtype, long long rows, long long tokens,
                            long long row_stride, long long token_stride, const void *table_dev,
                            int head_dim, int bits, uint8_t *idx_bytes, uint16_t *vec_norms,
-                           long long packed_row_stride, void *stream) {
+                           long long packed_row_stride, void *workspace, void *stream) {
     long long n_vec = 0;
     const int rc = check_job(states, dtype, rows, tokens, row_stride, token_stride, table_dev, head_dim, bits,
                              idx_bytes, vec_norms, packed_row_stride, &n_vec);
-    if (rc || n_vec == 0) return rc;
+    if (rc) return rc;
+    if ((uintptr_t)workspace & 63u) return TQ_ERR_ALIGN;
+    if (n_vec == 0) return TQ_OK;
     TqDevJob job;
     job.states = static_cast<const uint8_t *>(states);
     job.idx_bytes = idx_bytes;
@@ -724,14 +823,15 @@ extern "C" int tq_compress(const void *states, int dtype, long long rows, long l
     job.token_stride = token_stride * elem_bytes(dtype);
     if (head_dim != TQ_HEAD_DIM)
         return tq_anydim_compress(dtype, bits, head_dim, job, nullptr, 1, (uint32_t)n_vec, static_cast<hipStream_t>(stream));
-    return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), static_cast<hipStream_t>(stream));
+    return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), workspace, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
-                                   int head_dim, void *stream) {
+                                   int head_dim, void *workspace, void *stream) {
     if (n_jobs == 0) return TQ_OK;
     if (!jobs_host || !jobs_dev) return TQ_ERR_NULL;
     if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
+    if ((uintptr_t)workspace & 63u) return TQ_ERR_ALIGN;
     long long max_vec = 0;
     for (int i = 0; i < n_jobs; ++i) {
         const tq_job &j = jobs_host[i];
@@ -749,5 +849,5 @@ extern "C" int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_d
         return tq_anydim_compress(jobs_host[0].dtype, jobs_host[0].bits, head_dim, none, jobs_dev, n_jobs, (uint32_t)max_vec,
                                   static_cast<hipStream_t>(stream));
     return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec + 31) / 32),
-                    static_cast<hipStream_t>(stream));
+                    workspace, static_cast<hipStream_t>(stream));
 }

@@ -34,6 +34,13 @@
 // hipGetSymbolAddress; launches receive the per-device address kept by static_counters().
 static __device__ __align__(256) uint32_t scratch[TQ_NOALLOC_MAX_JOBS * (TQ_WORKSPACE_BYTES_PER_JOB / 4)];
 
+// Measurement build (never the shipped library): full tiles keep their loads, the scale / cast / transposition through
+// LDS and their stores, and leave out the decode, the matrix instructions and their operand reads.  What it writes is
+// garbage; its time is what the kernel's memory pattern costs on its own.
+#ifndef TQ_SKELETON
+#define TQ_SKELETON 0
+#endif
+
 namespace {
 
 template <int DTYPE> struct OutTraits;
@@ -88,7 +95,11 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
     const uint32_t first = blockIdx.x * T::WAVES;
     const uint32_t drawn_origin = gridDim.x * T::WAVES;
     uint32_t fixed_next = first + drawn_origin;
-    auto draw = [&]() -> uint32_t {     // thread 0 only
+    // thread 0 only.  The ticket is computed from the atomic's result on the spot, which makes the drawing wave wait for
+    // its own outstanding loads and stores once per ticket.  Measured against a form that leaves the result untouched
+    // until it is published a tile later (no wait at the draw): the launches of the Llama-3-8B 32K workload take
+    // 318 / 382 / 300 us this way and 339 / 388 / 305 us that way (2-, 4-, 8-bit), so the wait stays.
+    auto draw = [&]() -> uint32_t {
         if (counter) {
             const uint32_t t = drawn_origin + atomicAdd(counter, (uint32_t)T::WAVES);
             return t < n_tiles ? t : n_tiles;
@@ -185,6 +196,12 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
         tq_f16v acc[TQ_TILES];
 #pragma unroll
         for (int t = 0; t < TQ_TILES; ++t) acc[t] = tq_zero16();
+#if TQ_SKELETON
+#pragma unroll
+        for (int t = 0; t < TQ_TILES; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][r] = __uint_as_float(cur[(4 * t + r) % NW] + (uint32_t)r);
+#else
 #pragma unroll
         for (int s = 0; s < TQ_STEPS; ++s) {
             const tq_u4 b = decode_step<IPB, NW>(cur, s, lds_lut);
@@ -196,6 +213,7 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
                                                                 __builtin_bit_cast(tq_half8, b), acc[t], 0, 0, 0);
             }
         }
+#endif
 
         // ---- scale, cast, transpose through LDS.  Lane (n, hk) holds elements 64*hk + 16*t + r.
         if constexpr (ELEM == 2) {
@@ -476,9 +494,9 @@ extern "C" long long tq_workspace_bytes(int n_jobs) {
 }
 
 namespace {
-int decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs, int head_dim, void *workspace,
-                       void *stream) {
-    long long max_vec = 0;
+// Argument checks of a batch; max_vec = vectors of its largest job (0: nothing to launch).
+int check_batch(const tq_job *jobs_host, int n_jobs, int head_dim, long long *max_vec) {
+    *max_vec = 0;
     for (int i = 0; i < n_jobs; ++i) {
         const tq_job &j = jobs_host[i];
         if (8 / (j.bits < 1 || j.bits > 8 ? 1 : j.bits) != 8 / (jobs_host[0].bits < 1 || jobs_host[0].bits > 8 ? 1 : jobs_host[0].bits))
@@ -488,9 +506,13 @@ int decompress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jo
         const int rc = check_job(j.states, j.dtype, j.rows, j.tokens, j.row_stride, j.token_stride, j.table_dev,
                                  head_dim, j.bits, j.idx_bytes, j.vec_norms, j.packed_row_stride, &n_vec);
         if (rc) return rc;
-        if (n_vec > max_vec) max_vec = n_vec;
+        if (n_vec > *max_vec) *max_vec = n_vec;
     }
-    if (max_vec == 0) return TQ_OK;
+    return TQ_OK;
+}
+
+int launch_batch(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs, int head_dim, long long max_vec,
+                 void *workspace, void *stream) {
     TqDevJob none{};
     if (head_dim != TQ_HEAD_DIM)
         return tq_anydim_decompress(jobs_host[0].dtype, jobs_host[0].bits, head_dim, none, jobs_dev, n_jobs, (uint32_t)max_vec,
@@ -506,7 +528,10 @@ extern "C" int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs
     if (!jobs_host || !jobs_dev) return TQ_ERR_NULL;
     if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
     if ((uintptr_t)workspace & 63u) return TQ_ERR_ALIGN;
-    return decompress_batched(jobs_host, jobs_dev, n_jobs, head_dim, workspace, stream);
+    long long max_vec = 0;
+    const int rc = check_batch(jobs_host, n_jobs, head_dim, &max_vec);
+    if (rc || max_vec == 0) return rc;
+    return launch_batch(jobs_host, jobs_dev, n_jobs, head_dim, max_vec, workspace, stream);
 }
 
 extern "C" int tq_decompress_batched_noalloc(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
@@ -515,8 +540,12 @@ extern "C" int tq_decompress_batched_noalloc(const tq_job *jobs_host, const tq_j
     if (!jobs_host || !jobs_dev) return TQ_ERR_NULL;
     if (n_jobs < 0) return TQ_ERR_SIZE;
     if (n_jobs > TQ_NOALLOC_MAX_JOBS) return TQ_ERR_CAPACITY;
+    // every argument is checked before anything is launched: an argument error leaves the stream untouched
+    long long max_vec = 0;
+    int rc = check_batch(jobs_host, n_jobs, head_dim, &max_vec);
+    if (rc || max_vec == 0) return rc;
     uint32_t *counters = nullptr;
-    const int rc = static_counters(&counters);
+    rc = static_counters(&counters);
     if (rc) return rc;
     // The array keeps what the last call left.  A launch that completed left zeros, one that failed half-way
     // may not have: the words this call uses are cleared first, on the same stream.
@@ -525,5 +554,5 @@ extern "C" int tq_decompress_batched_noalloc(const tq_job *jobs_host, const tq_j
                        counters, words);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    return decompress_batched(jobs_host, jobs_dev, n_jobs, head_dim, counters, stream);
+    return launch_batch(jobs_host, jobs_dev, n_jobs, head_dim, max_vec, counters, stream);
 }

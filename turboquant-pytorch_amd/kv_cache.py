@@ -419,7 +419,7 @@ def hf_cache_class():
             # means the model's attention ran over one token (another attention implementation is selected, or the
             # tag on the key tensor was lost on the way), and that must not pass silently.
             self._pending_layer = None
-            self._mask_checked = None      # (address, version) of the last attention mask found free of padding
+            self._mask_checked = None      # (address, version, shape, cache length) of the last attention mask found free of padding
 
         def _no_pending(self, what: str) -> None:
             if self._pending_layer is not None:
@@ -474,8 +474,15 @@ def packed_attention_forward(module, query, key, value, attention_mask, scaling=
     if tag is not None and query.shape[2] == 1:
         cache, layer_idx = tag
         if attention_mask is not None:
-            ident = (attention_mask.data_ptr(), attention_mask._version, tuple(attention_mask.shape))
+            # One inspection per decode step: the key carries the cache length of this step, so that a new mask that the
+            # allocator happens to place at the address of the last one (fixed-length masks) is looked at again.
+            ident = (attention_mask.data_ptr(), attention_mask._version, tuple(attention_mask.shape),
+                     V3Cache.get_seq_length(cache, layer_idx))
             if cache._mask_checked != ident:
+                if torch.cuda.is_current_stream_capturing():
+                    # the inspection reads a device value on the host, which a stream capture cannot record
+                    raise RuntimeError("packed_attention: an attention mask cannot be inspected while a graph is being captured; "
+                                       "capture decode steps without a mask (unpadded batches need none) or use packed_attention=False.")
                 if not _mask_hides_nothing(attention_mask):
                     raise RuntimeError("packed_attention: the attention mask hides cached tokens (padded batch?); attention from "
                                        "the packed store counts every cached token.  Use packed_attention=False for such batches.")
