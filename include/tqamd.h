@@ -221,6 +221,47 @@ int tq_qjl_signs(const void *states, int dtype, long long n_vec, long long token
                  uint8_t *sign_bytes, uint16_t *residual_norm, void *stream);
 
 /*
+ * TurboQuantCompressorV2.compress (compressors.py:84-122) as one call: packed MSE codes and fp16 norms (what tq_compress
+ * writes with mse_bits and `table_dev`), the 16 sign bytes and the fp16 residual norm of every vector (what tq_qjl_signs
+ * writes).  The n_vec vectors lie token_stride elements apart; all four outputs are dense ([n_vec, G], [n_vec],
+ * [n_vec, 16], [n_vec]).  For 16-bit inputs and codes of up to TQ_QJL_ONE_PASS_MAX_BITS bits the vectors are read once, by a
+ * kernel that works on the residual in rotated coordinates ((Pi x)[k] - ||x|| centroid(code_k), projected by S Pi^T
+ * from the table of tq_qjl_table_build); float32 inputs, wider codes and the last n_vec % 32 vectors of a job take
+ * tq_compress followed by tq_qjl_signs.  Both forms write the same codes and norms; their sign bits agree wherever a
+ * projection is further than 1e-5 of |S row| |residual| from zero.
+ * The batched form is one launch for many (layer) jobs that share dtype and mse_bits; `jobs_dev` is a device copy of the
+ * same records, uploaded once by the caller (the per-layer loop of validate.py:96-111).
+ */
+#define TQ_QJL_ONE_PASS_MAX_BITS 4
+typedef struct tq_qjl_job {
+    const void *states;          /* input vectors                                        */
+    uint8_t *idx_bytes;          /* out: packed MSE codes, dense [n_vec, G]              */
+    uint16_t *vec_norms;         /* out: fp16 norms [n_vec]                              */
+    uint8_t *sign_bytes;         /* out: [n_vec, 16]                                     */
+    uint16_t *residual_norm;     /* out: fp16 [n_vec]                                    */
+    const void *table_dev;       /* tq_table_build(Pi, centroids, mse_bits)              */
+    const void *qjl_table_dev;   /* tq_qjl_table_build(Pi, S, centroids, mse_bits)       */
+    long long n_vec;
+    long long token_stride;      /* elements                                             */
+    int mse_bits;                /* 1..7, the same in all jobs of a call                 */
+    int dtype;                   /* element type of `states`, the same in all jobs       */
+} tq_qjl_job;
+int tq_qjl_compress(const void *states, int dtype, long long n_vec, long long token_stride, const void *table_dev,
+                    const void *qjl_table_dev, int head_dim, int mse_bits, uint8_t *idx_bytes, uint16_t *vec_norms,
+                    uint8_t *sign_bytes, uint16_t *residual_norm, void *stream);
+int tq_qjl_compress_batched(const tq_qjl_job *jobs_host, const tq_qjl_job *jobs_dev, int n_jobs, int head_dim, void *stream);
+/*
+ * Both terms of asymmetric_attention_scores (compressors.py:124-158) in one launch, from the packed form (dense buffers
+ * of `rows` rows x `tokens` tokens) for any number of query tokens per row:
+ *   scores[(r * n_queries + q) * tokens + t] = norm_t * q_rot[r][q] . centroids[codes_t] + residual_norm_t * q_sign[r][q] . signs_t
+ * with q_rot = Pi q and q_sign = sqrt(pi/2) / head_dim * S q (float32 [rows, n_queries, head_dim], contiguous), `table_dev`
+ * the codec table of the MSE stage.  rows <= 65535.
+ */
+int tq_qjl_scores(const uint8_t *idx_bytes, const uint16_t *vec_norms, const uint8_t *sign_bytes, const uint16_t *residual_norm,
+                  long long rows, long long tokens, const void *table_dev, int head_dim, int mse_bits,
+                  const float *q_rot, const float *q_sign, long long n_queries, float *scores, void *stream);
+
+/*
  * tq_decompress_batched for callers that cannot allocate device memory and have no workspace to pass: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments, checks and output bytes as tq_decompress_batched; the ticket counters live in a

@@ -141,3 +141,47 @@ def test_v2_value_compressor_against_reference_vectors(pkg, oracle, fx):
         assert rec.dtype == torch.float32 and rec.shape == ref.shape
         err = np.linalg.norm(rec.cpu().numpy() - ref) / np.linalg.norm(ref)
         assert err < 1e-3, (bits, err)
+
+
+@pytest.mark.parametrize("bits,dtype", [(3, torch.bfloat16), (5, torch.float16), (2, torch.bfloat16)])
+def test_v2_one_pass_form_against_the_two_kernel_form(pkg, oracle, bits, dtype):
+    """The one-pass kernel (residual in rotated coordinates, projection by S Pi^T) against tq_compress followed by
+    tq_qjl_signs on the same vectors: identical codes and norms, sign bits that differ only where a projection lies
+    within 1e-5 of |S row| |residual| of zero, residual norms within one fp16 unit; single call and batched list."""
+    import ctypes
+    native = pkg._native
+    L, n = 3, 4096 + 32 * 7 + 11                 # full tiles for the one-pass kernel, a ragged end for the other form
+    comps = [pkg.TurboQuantCompressorV2(128, bits, seed=31 * l + bits, device=DEV) for l in range(L)]
+    xs = [outlier_kv((1, 1, n, 128), seed=300 + l, dtype=dtype).to(DEV) for l in range(L)]
+    packed = [c.empty_packed(1, 1, n, DEV) for c in comps]
+    for p in packed:
+        for k in ("idx_bytes", "vec_norms", "sign_bytes", "residual_norm"):
+            p[k].fill_(0x55 if p[k].dtype == torch.uint8 else 3.0)
+    native.QjlJobList([c.job(x, p) for c, x, p in zip(comps, xs, packed)], torch.device(DEV)).compress()
+    torch.cuda.synchronize()
+    for c, x, p in zip(comps, xs, packed):
+        single = c.compress(x)
+        for k in ("idx_bytes", "vec_norms", "sign_bytes", "residual_norm"):
+            assert torch.equal(single[k].view(torch.uint8), p[k].view(torch.uint8)), k       # the list and the single call agree
+        # the two-kernel form through the C entry points
+        first = c._mse.compress(x)
+        sb = torch.empty_like(p["sign_bytes"])
+        rn = torch.empty_like(p["residual_norm"])
+        rc = native.lib().tq_qjl_signs(x.data_ptr(), native.dtype_code(x.dtype), n, 128, first["idx_bytes"].data_ptr(),
+                                       c._table(DEV).data_ptr(), 128, c.mse_bits, sb.data_ptr(), rn.data_ptr(),
+                                       ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(first["idx_bytes"], p["idx_bytes"]) and torch.equal(first["vec_norms"].view(torch.int16), p["vec_norms"].view(torch.int16))
+        a = np.unpackbits(p["sign_bytes"].cpu().numpy().reshape(-1, 16), axis=-1, bitorder="big")
+        b = np.unpackbits(sb.cpu().numpy().reshape(-1, 16), axis=-1, bitorder="big")
+        diff = a != b
+        orc = oracle.QjlOracle(c.Pi.cpu().numpy(), c.S.cpu().numpy(), c.centroids.cpu().numpy())
+        ref = orc.compress(x.float().cpu().numpy().reshape(-1, 128))
+        srow = np.linalg.norm(orc.S, axis=1)
+        margin = np.abs(ref["projected"]) / (srow[None, :] * np.maximum(ref["residual_norm_f32"][:, None], 1e-30))
+        print(f"[v2] one pass vs two kernels, {bits} bits {dtype}: {int(diff.sum())} of {diff.size} sign bits differ, "
+              f"largest margin {float(margin[diff].max()) if diff.any() else 0:.1e}")
+        assert diff.sum() <= max(4, 5e-5 * diff.size) and (margin[diff] < 1e-5).all()
+        ulp = oracle.fp16_ulp_distance(bits16(p["residual_norm"]).reshape(-1), bits16(rn).reshape(-1))
+        assert ulp.max() <= 1 and (ulp > 0).mean() < 0.02

@@ -134,11 +134,28 @@ class TqJob(ctypes.Structure):
     ]
 
 
+class TqQjlJob(ctypes.Structure):
+    _fields_ = [
+        ("states", ctypes.c_void_p),
+        ("idx_bytes", ctypes.c_void_p),
+        ("vec_norms", ctypes.c_void_p),
+        ("sign_bytes", ctypes.c_void_p),
+        ("residual_norm", ctypes.c_void_p),
+        ("table_dev", ctypes.c_void_p),
+        ("qjl_table_dev", ctypes.c_void_p),
+        ("n_vec", ctypes.c_longlong),
+        ("token_stride", ctypes.c_longlong),
+        ("mse_bits", ctypes.c_int),
+        ("dtype", ctypes.c_int),
+    ]
+
+
 EXPORTS = (
     "tq_abi_version", "tq_status_string", "tq_device_count", "tq_bytes_per_vector",
     "tq_decision_thresholds", "tq_table_bytes", "tq_table_build", "tq_table_check", "tq_table_quantize_host",
     "tq_compress", "tq_decompress", "tq_compress_batched", "tq_decompress_batched", "tq_workspace_bytes",
     "tq_decompress_batched_noalloc", "tq_qjl_table_bytes", "tq_qjl_table_build", "tq_qjl_signs",
+    "tq_qjl_compress", "tq_qjl_compress_batched", "tq_qjl_scores",
     "tq_scores", "tq_weighted_values", "tq_weighted_values_splits", "tq_attend_partials", "tq_attend_splits",
     "tq_attend_prepare", "tq_attend_merge", "tq_append_token", "tq_attend_step",
 )
@@ -186,6 +203,9 @@ def lib() -> ctypes.CDLL:
     L.tq_qjl_table_bytes.argtypes = [ci, ci]
     L.tq_qjl_table_build.argtypes = [vp, vp, vp, ci, ci, vp, ctypes.c_size_t]
     L.tq_qjl_signs.argtypes = [vp, ci, ll, ll, vp, vp, ci, ci, vp, vp, vp]
+    L.tq_qjl_compress.argtypes = [vp, ci, ll, ll, vp, vp, ci, ci, vp, vp, vp, vp, vp]
+    L.tq_qjl_compress_batched.argtypes = [vp, vp, ci, ci, vp]
+    L.tq_qjl_scores.argtypes = [vp, vp, vp, vp, ll, ll, vp, ci, ci, vp, vp, ll, vp, vp]
     L.tq_append_token.argtypes = [vp, vp, ci, ll, ll, vp, vp, ll, ll, ll, vp, vp, ci, ci, ci, vp, vp, vp, vp, ll, ll, ll, vp]
     L.tq_attend_step.argtypes = [vp, ci, ll, ci, ctypes.c_float, vp, vp, vp, vp, ci, ll, ll, vp, vp, vp, vp, ll, ll,
                                  vp, vp, ci, ci, ci, vp, vp, vp, ci, vp, ci, vp]
@@ -765,6 +785,43 @@ class JobList:
         if rc:
             self.workspace.zero_()      # counters of a launch that did not complete are not trusted
         check(rc, "tq_decompress_batched")
+
+
+class QjlJobList:
+    """A fixed list of V2 key jobs (one per layer) of one width and element type, uploaded once and compressed by a
+    single tq_qjl_compress_batched call.  Every job: {"states" [.., 128] dense vectors, "idx_bytes", "vec_norms",
+    "sign_bytes", "residual_norm" (dense outputs), "table" (codec table of the MSE stage), "qjl_table", "mse_bits"}."""
+
+    def __init__(self, jobs: Sequence[dict], device: torch.device):
+        if not jobs:
+            raise ValueError("empty job list")
+        self.n = len(jobs)
+        self.device = torch.device(device)
+        self.host = (TqQjlJob * self.n)()
+        self._keep = []
+        for i, j in enumerate(jobs):
+            t = j["states"]
+            _require_gpu(t, "states")
+            if not t.is_contiguous() or t.data_ptr() % 16:
+                raise TqError("batched V2 jobs need contiguous, 16-byte aligned inputs")
+            for name in ("idx_bytes", "vec_norms", "sign_bytes", "residual_norm"):
+                if not j[name].is_contiguous():
+                    raise TqError(f"batched V2 jobs need dense outputs ({name})")
+            D = t.shape[-1]
+            check_table(j["table"], D, int(j["mse_bits"]))
+            self.host[i] = TqQjlJob(t.data_ptr(), j["idx_bytes"].data_ptr(), j["vec_norms"].data_ptr(), j["sign_bytes"].data_ptr(),
+                                    j["residual_norm"].data_ptr(), j["table"].data_ptr(), j["qjl_table"].data_ptr(),
+                                    t.numel() // D, D, int(j["mse_bits"]), dtype_code(t.dtype))
+            self._keep.append(tuple(j[k] for k in ("states", "idx_bytes", "vec_norms", "sign_bytes", "residual_norm", "table", "qjl_table")))
+        self.head_dim = int(jobs[0]["states"].shape[-1])
+        raw = np.frombuffer(bytes(self.host), dtype=np.uint8).copy()
+        self.dev = torch.from_numpy(raw).to(self.device)
+
+    def compress(self) -> None:
+        with _on(self.device):
+            rc = lib().tq_qjl_compress_batched(ctypes.addressof(self.host), self.dev.data_ptr(), self.n, self.head_dim,
+                                               _stream_handle(self.device))
+        check(rc, "tq_qjl_compress_batched")
 
 
 # ------------------------------------------------------------------------------------

@@ -68,8 +68,6 @@ class TurboQuantCompressorV2:
         self.S = s_host.to(dev).contiguous()
         self.centroids = cent_host.to(dev)
         self._mse = MSECompressor.from_tensors(pi_host, cent_host, self.mse_bits, device=dev)
-        # the sign bits are a 1-bit store over the codebook (-1, +1) in an un-rotated space: the score kernels read them as such
-        self._sign = MSECompressor.from_tensors(torch.eye(self.head_dim), torch.tensor([-1.0, 1.0]), 1, device=dev)
         L = _native.lib()
         n = L.tq_qjl_table_bytes(self.head_dim, self.mse_bits)
         if n < 0:
@@ -106,26 +104,40 @@ class TurboQuantCompressorV2:
     @torch.no_grad()
     def compress(self, states: torch.Tensor) -> dict:
         """(B, H, S, D) -> {"idx_bytes" u8 [B,H,S,G], "vec_norms" f16 [B,H,S], "sign_bytes" u8 [B,H,S,D/8],
-        "residual_norm" f16 [B,H,S], "shape"}.  Two launches: MSE codes and norms, then residual signs and norms."""
+        "residual_norm" f16 [B,H,S], "shape"}.  One call (tq_qjl_compress): a single pass over the input for 16-bit
+        elements and MSE codes of up to 4 bits, MSE codes and norms followed by residual signs and norms otherwise."""
         B, H, S, D = states.shape
         _native._require_gpu(states, "states")
         if not states.is_contiguous():
             states = states.contiguous()
         if states.data_ptr() % 16:       # a contiguous view into the middle of a buffer: contiguous() would hand it back as it is
             states = states.clone(memory_format=torch.contiguous_format)
-        first = self._mse.compress(states)
-        sign_bytes = torch.empty((B, H, S, D // 8), dtype=torch.uint8, device=states.device)
-        residual_norm = torch.empty((B, H, S), dtype=torch.float16, device=states.device)
+        out = self.empty_packed(B, H, S, states.device)
         n_vec = B * H * S
         if n_vec:
             with _native._on(states.device):
-                rc = _native.lib().tq_qjl_signs(states.data_ptr(), _native.dtype_code(states.dtype), n_vec, D,
-                                                first["idx_bytes"].data_ptr(), self._table(states.device).data_ptr(), D, self.mse_bits,
-                                                sign_bytes.data_ptr(), residual_norm.data_ptr(),
-                                                _native._stream_handle(states.device))
-            _native.check(rc, "tq_qjl_signs")
-        return {"idx_bytes": first["idx_bytes"], "vec_norms": first["vec_norms"], "sign_bytes": sign_bytes,
-                "residual_norm": residual_norm, "shape": (B, H, S, D)}
+                rc = _native.lib().tq_qjl_compress(states.data_ptr(), _native.dtype_code(states.dtype), n_vec, D,
+                                                   self._mse.table(states.device).data_ptr(), self._table(states.device).data_ptr(),
+                                                   D, self.mse_bits, out["idx_bytes"].data_ptr(), out["vec_norms"].data_ptr(),
+                                                   out["sign_bytes"].data_ptr(), out["residual_norm"].data_ptr(),
+                                                   _native._stream_handle(states.device))
+            _native.check(rc, "tq_qjl_compress")
+        return out
+
+    def empty_packed(self, B: int, H: int, S: int, device) -> dict:
+        """The packed dictionary `compress` fills, with uninitialised buffers."""
+        D = self.head_dim
+        G = -(-D // (8 // self.mse_bits))
+        return {"idx_bytes": torch.empty((B, H, S, G), dtype=torch.uint8, device=device),
+                "vec_norms": torch.empty((B, H, S), dtype=torch.float16, device=device),
+                "sign_bytes": torch.empty((B, H, S, D // 8), dtype=torch.uint8, device=device),
+                "residual_norm": torch.empty((B, H, S), dtype=torch.float16, device=device), "shape": (B, H, S, D)}
+
+    def job(self, states: torch.Tensor, packed: dict) -> dict:
+        """A record for `_native.QjlJobList` (one launch for the keys of many layers): `states` compressed into `packed`."""
+        return {"states": states, "idx_bytes": packed["idx_bytes"], "vec_norms": packed["vec_norms"], "sign_bytes": packed["sign_bytes"],
+                "residual_norm": packed["residual_norm"], "table": self._mse.table(states.device), "qjl_table": self._table(states.device),
+                "mse_bits": self.mse_bits}
 
     @torch.no_grad()
     def reference_format(self, compressed: dict) -> dict:
@@ -158,16 +170,21 @@ class TurboQuantCompressorV2:
         out = torch.empty((B, H, S_q, S_k), dtype=torch.float32, device=queries.device)
         if out.numel() == 0:
             return out
+        _native._require_gpu(queries, "queries")
         q = queries.float()
-        q_sign = torch.matmul(q, self._s(q.device).T) * corr
-        step = 32                                   # query tokens per key row and launch
-        for lo in range(0, S_q, step):
-            hi = min(lo + step, S_q)
-            n = hi - lo
-            first = self._mse.packed_scores(compressed["idx_bytes"], compressed["vec_norms"], q[:, :, lo:hi].reshape(B, H * n, D))
-            second = self._sign.packed_scores(compressed["sign_bytes"], compressed["residual_norm"],
-                                              q_sign[:, :, lo:hi].reshape(B, H * n, D))
-            out[:, :, lo:hi] = (first + second).reshape(B, H, n, S_k)
+        dev = q.device
+        q_rot = torch.matmul(q, self._mse.pi_transposed(dev)).contiguous()          # Pi q for every query token
+        st = self._s_on.get(("t", dev))
+        if st is None:
+            st = self._s_on[("t", dev)] = (self._s(dev).T * corr).contiguous()      # sqrt(pi/2)/m S^T, made once per device
+        q_sign = torch.matmul(q, st).contiguous()
+        packed = [compressed[k] if compressed[k].is_contiguous() else compressed[k].contiguous()
+                  for k in ("idx_bytes", "vec_norms", "sign_bytes", "residual_norm")]
+        with _native._on(dev):
+            rc = _native.lib().tq_qjl_scores(packed[0].data_ptr(), packed[1].data_ptr(), packed[2].data_ptr(), packed[3].data_ptr(),
+                                             B * H, S_k, self._mse.table(dev).data_ptr(), D, self.mse_bits,
+                                             q_rot.data_ptr(), q_sign.data_ptr(), S_q, out.data_ptr(), _native._stream_handle(dev))
+        _native.check(rc, "tq_qjl_scores")
         return out
 
 

@@ -134,6 +134,156 @@ __global__ __launch_bounds__(SC_WAVES *TQ_WAVE) void tq_scores_kernel(ScoreArgs 
     }
 }
 
+// ---- both terms of the V2 key estimate in one pass (upstream turboquant/compressors.py:124-158) ----------------------
+//   score[row][q][t] = norm_t * (Pi q) . centroids[codes_t]  +  residual_norm_t * (c S q) . signs_t ,  c = sqrt(pi/2) / 128
+// The first term is tq_scores_kernel's; the second reads the 16 sign bytes of a token as 1-bit codes over (-1, +1)
+// (byte -> eight fp16 values from a table built here) against one fp16 term of the projected query (the term is a
+// correction of the size of the quantisation residual: 2^-12 of it disappears under the tolerance of the first).
+// Query tokens beyond 32 per row go to further blocks (blockIdx.z): one launch for any number of them.
+struct QjlScoreArgs {
+    const uint8_t *idx_bytes;
+    const uint16_t *vec_norms;
+    const uint8_t *sign_bytes;
+    const uint16_t *residual_norm;
+    const uint8_t *table;
+    const float *q_rot;      // [rows, n_q, 128]
+    const float *q_sign;     // [rows, n_q, 128]
+    float *scores;           // [rows, n_q, tokens]
+    uint32_t tokens, n_q;
+};
+
+template <int IPB>
+__global__ __launch_bounds__(SC_WAVES *TQ_WAVE) void tq_qjl_scores_kernel(QjlScoreArgs a) {
+    constexpr int NB = 64 / IPB;   // packed bytes per lane (half a vector)
+    constexpr int NW = NB / 4;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_lut[4096];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_sign[4096];
+    __shared__ float lds_rowscale[2][32];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t row = blockIdx.y, q0 = blockIdx.z * 32u;
+    const uint32_t group = a.n_q - q0 < 32u ? a.n_q - q0 : 32u;      // query tokens of this block
+    const uint32_t n = lane & 31u, hk = lane >> 5;
+    const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(a.table);
+    tq_copy_to_lds(lds_lut, a.table + hd->off_lut, 256u * 2u * IPB, tid, SC_WAVES * TQ_WAVE);
+    for (uint32_t v = tid; v < 256u; v += SC_WAVES * TQ_WAVE) {     // bit 7 - k of a sign byte belongs to coordinate k
+        tq_half8 e;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) e[k] = ((v >> (7 - k)) & 1u) ? (_Float16)1.0f : (_Float16)-1.0f;
+        *reinterpret_cast<tq_u4 *>(lds_sign + 16u * v) = __builtin_bit_cast(tq_u4, e);
+    }
+
+    // ---- A operands: query n of this block, contraction slice (step s, half hk) = coordinates 64*hk + 8*s + i
+    tq_u4 ahi[TQ_STEPS], alo[TQ_STEPS], shi[TQ_STEPS];
+    {
+        const bool live = n < group;
+        const size_t qoff = ((size_t)row * a.n_q + q0 + (live ? n : 0u)) * TQ_HEAD_DIM + 64u * hk;
+        auto exponent_of = [&](const TQ_GLOBAL float *q) {
+            float big = 0.f;
+            for (int i = 0; i < 64; ++i) big = fmaxf(big, fabsf(q[i]));
+            big = fmaxf(big, __shfl_xor(big, 32));
+            int e = 0;
+            if (big > 0.f && big < __builtin_inff()) (void)frexpf(big, &e);
+            return e < -100 ? -100 : e;   // rows that small give zero scores either way; keeps 2^(10-e) finite
+        };
+        const TQ_GLOBAL float *q = (const TQ_GLOBAL float *)a.q_rot + qoff;
+        const TQ_GLOBAL float *qs = (const TQ_GLOBAL float *)a.q_sign + qoff;
+        const int e1 = exponent_of(q), e2 = exponent_of(qs);
+        const float up1 = ldexpf(1.f, TQ_F16_PI_SHIFT - e1), up2 = ldexpf(1.f, TQ_F16_PI_SHIFT - e2);
+        if (hk == 0u) {
+            lds_rowscale[0][n] = live ? ldexpf(1.f, e1 - TQ_F16_PI_SHIFT) : 0.f;
+            lds_rowscale[1][n] = live ? ldexpf(1.f, e2 - TQ_F16_PI_SHIFT) : 0.f;
+        }
+#pragma unroll
+        for (int s = 0; s < TQ_STEPS; ++s) {
+            tq_half8 h, l, g;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float x = live ? q[8 * s + i] * up1 : 0.f;
+                const _Float16 xh = (_Float16)x;
+                h[i] = xh;
+                l[i] = (_Float16)(x - (float)xh);
+                g[i] = (_Float16)(live ? qs[8 * s + i] * up2 : 0.f);
+            }
+            ahi[s] = __builtin_bit_cast(tq_u4, h);
+            alo[s] = __builtin_bit_cast(tq_u4, l);
+            shi[s] = __builtin_bit_cast(tq_u4, g);
+        }
+    }
+    __syncthreads();
+    // accumulator register r of lane (n, h = hk) belongs to query 8*(r/4) + 4*h + r%4
+    float scale1[16], scale2[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        scale1[r] = lds_rowscale[0][8 * (r / 4) + 4 * hk + (r % 4)];
+        scale2[r] = lds_rowscale[1][8 * (r / 4) + 4 * hk + (r % 4)];
+    }
+
+    const uint32_t n_tiles = (a.tokens + 31u) / 32u;
+    const uint32_t tile_stride = gridDim.x * SC_WAVES;
+    uint32_t tile = blockIdx.x * SC_WAVES + wave;
+    const size_t slot0 = (size_t)row * a.tokens;
+
+    uint32_t raw[NW], sraw[2];
+    uint16_t norm_bits = 0, rnorm_bits = 0;
+    auto issue_loads = [&](uint32_t tl) {
+        const uint32_t t = tl * 32u + n;
+        const bool ok = t < a.tokens;
+        const size_t slot = slot0 + (ok ? t : 0u);
+        const uint8_t *src = a.idx_bytes + slot * (2 * NB) + hk * NB;
+        if constexpr (NW == 2) {
+            tq_u2 v = {0u, 0u};
+            if (ok) v = tq_gload8(src);
+            raw[0] = v[0]; raw[1] = v[1];
+        } else {
+#pragma unroll
+            for (int q = 0; q < NW / 4; ++q) {
+                tq_u4 v = {0u, 0u, 0u, 0u};
+                if (ok) v = tq_gload16(src + 16 * q);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) raw[4 * q + i] = v[i];
+            }
+        }
+        tq_u2 sv = {0u, 0u};
+        if (ok) sv = tq_gload8(a.sign_bytes + slot * 16u + hk * 8u);
+        sraw[0] = sv[0]; sraw[1] = sv[1];
+        norm_bits = ok ? tq_gload2(a.vec_norms + slot) : (uint16_t)0;
+        rnorm_bits = ok ? tq_gload2(a.residual_norm + slot) : (uint16_t)0;
+    };
+    if (tile < n_tiles) issue_loads(tile);
+    while (tile < n_tiles) {
+        uint32_t cur[NW], scur[2];
+#pragma unroll
+        for (int i = 0; i < NW; ++i) cur[i] = raw[i];
+        scur[0] = sraw[0]; scur[1] = sraw[1];
+        const float nrm = (float)__builtin_bit_cast(_Float16, norm_bits);
+        const float rnrm = (float)__builtin_bit_cast(_Float16, rnorm_bits);
+        const uint32_t next = tile + tile_stride;
+        if (next < n_tiles) issue_loads(next);
+
+        tq_f16v acc = tq_zero16(), sacc = tq_zero16();
+#pragma unroll
+        for (int s = 0; s < TQ_STEPS; ++s) {
+            const tq_u4 b = decode_step<IPB, NW>(cur, s, lds_lut);
+            const tq_u4 sb = decode_step<8, 2>(scur, s, lds_sign);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, ahi[s]), __builtin_bit_cast(tq_half8, b), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, alo[s]), __builtin_bit_cast(tq_half8, b), acc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(tq_half8, shi[s]), __builtin_bit_cast(tq_half8, sb), sacc, 0, 0, 0);
+        }
+        const uint32_t t = tile * 32u + n;
+        if (t < a.tokens) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t m = 8u * (r / 4) + 4u * hk + (r % 4);
+                if (m < group)
+                    ((TQ_GLOBAL float *)a.scores)[((size_t)row * a.n_q + q0 + m) * a.tokens + t] =
+                        fmaf(sacc[r] * scale2[r], rnrm, acc[r] * scale1[r] * nrm);
+            }
+        }
+        tile = next;
+    }
+}
+
 struct WvArgs {
     const uint8_t *idx_bytes;
     const uint16_t *vec_norms;
@@ -1154,6 +1304,50 @@ extern "C" int tq_scores(const uint8_t *idx_bytes, const uint16_t *vec_norms, lo
         case 4: hipLaunchKernelGGL(tq_scores_kernel<4>, grid, block, 0, s, a); break;
         case 2: hipLaunchKernelGGL(tq_scores_kernel<2>, grid, block, 0, s, a); break;
         default: hipLaunchKernelGGL(tq_scores_kernel<1>, grid, block, 0, s, a); break;
+    }
+    return (int)hipGetLastError();
+}
+
+extern "C" int tq_qjl_scores(const uint8_t *idx_bytes, const uint16_t *vec_norms, const uint8_t *sign_bytes, const uint16_t *residual_norm,
+                             long long rows, long long tokens, const void *table_dev, int head_dim, int mse_bits,
+                             const float *q_rot, const float *q_sign, long long n_queries, float *scores, void *stream) {
+    int rc = check_packed(idx_bytes, vec_norms, 0, rows, tokens, table_dev, head_dim, mse_bits);
+    if (rc) return rc;
+    if (n_queries < 0 || n_queries > 32ll * 65535) return TQ_ERR_SIZE;
+    if (rows == 0 || tokens == 0 || n_queries == 0) return TQ_OK;
+    if (!sign_bytes || !residual_norm || !q_rot || !q_sign || !scores) return TQ_ERR_NULL;
+    if (((uintptr_t)sign_bytes & 15u) || ((uintptr_t)residual_norm & 1u) || ((uintptr_t)q_rot & 3u) || ((uintptr_t)q_sign & 3u) ||
+        ((uintptr_t)scores & 3u))
+        return TQ_ERR_ALIGN;
+    int cus = 0;
+    rc = device_cus(cus);
+    if (rc) return rc;
+    QjlScoreArgs a;
+    a.idx_bytes = idx_bytes;
+    a.vec_norms = vec_norms;
+    a.sign_bytes = sign_bytes;
+    a.residual_norm = residual_norm;
+    a.table = static_cast<const uint8_t *>(table_dev);
+    a.q_rot = q_rot;
+    a.q_sign = q_sign;
+    a.scores = scores;
+    a.tokens = (uint32_t)tokens;
+    a.n_q = (uint32_t)n_queries;
+    const uint32_t chunks = (uint32_t)((n_queries + 31) / 32);
+    const uint32_t tiles = (uint32_t)((tokens + 31) / 32);
+    const uint32_t want = (tiles + SC_WAVES - 1) / SC_WAVES;
+    // about two four-wave blocks per compute unit: a block spends several microseconds on its query operands and
+    // tables before its first tile, so it should have many tiles to walk
+    uint32_t bx = (uint32_t)(((long long)cus * 2 + rows * chunks - 1) / (rows * chunks));
+    if (bx > want) bx = want;
+    if (bx < 1) bx = 1;
+    dim3 grid(bx, (unsigned)rows, chunks), block(SC_WAVES * TQ_WAVE, 1, 1);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (8 / mse_bits) {
+        case 8: hipLaunchKernelGGL(tq_qjl_scores_kernel<8>, grid, block, 0, s, a); break;
+        case 4: hipLaunchKernelGGL(tq_qjl_scores_kernel<4>, grid, block, 0, s, a); break;
+        case 2: hipLaunchKernelGGL(tq_qjl_scores_kernel<2>, grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL(tq_qjl_scores_kernel<1>, grid, block, 0, s, a); break;
     }
     return (int)hipGetLastError();
 }

@@ -176,6 +176,48 @@ static __device__ __forceinline__ void split_f32x8(const float (&x)[8], tq_u4 &t
     }
 }
 
+// ---- packing geometry -------------------------------------------------------------------
+// A lane owns 16 consecutive codes = NB packed bytes, handled as NW words of WB bytes (a full
+// dword, or the lane's 2 bytes for 1-bit codes).  Inside a word, code number i (in the order
+// "highest byte first, most significant code of the byte first") sits at bit shift_of(i);
+// FIELD is the spacing the sign-collecting funnel shift uses.
+template <int BITS> struct Pack {
+    static constexpr int IPB = 8 / BITS;                 // codes per byte
+    static constexpr int NB = 16 / IPB;                  // bytes per lane: 2, 4, 8, 8, 16
+    static constexpr int WB = NB < 4 ? NB : 4;           // bytes per word
+    static constexpr int NW = NB / WB;                   // words per lane
+    static constexpr int CPW = WB * IPB;                 // codes per word
+    static constexpr int FIELD = IPB == 1 ? 8 : BITS;    // bits the funnel shift advances per code
+    static constexpr int COPIES = TQ_GRID_COPIES(BITS);
+    static constexpr int COPY_STRIDE = TQ_GRID_COPY_STRIDE(BITS);
+    static constexpr int byte_of(int i) { return WB - 1 - i / IPB; }
+    static constexpr int k_of(int i) { return i % IPB; }
+    static constexpr int shift_of(int i) { return 8 * byte_of(i) + BITS * (IPB - 1 - k_of(i)); }
+    static constexpr int local_code(int w, int i) { return w * CPW + byte_of(i) * IPB + k_of(i); }
+    // grid copy used for the i-th code: its base is pre-shifted to the code's bit position
+    // (one-code-per-byte widths use two copies, shifts 0 and 8, and merge halves with one shift)
+    static constexpr int copy_of(int i) {
+        return IPB == 1 ? (byte_of(i) & 1) : byte_of(i) * IPB + (IPB - 1 - k_of(i));
+    }
+    static constexpr uint32_t sign_mask() {
+        uint32_t m = 0;
+        for (int i = 0; i < CPW; ++i) m |= 1u << (shift_of(i) + FIELD - 1);
+        return m;
+    }
+};
+
+template <int BITS>
+__device__ __forceinline__ uint32_t copy_shift_rt(uint32_t c) {
+    constexpr int IPB = 8 / BITS;
+    return IPB == 1 ? 8u * c : 8u * (c / IPB) + (uint32_t)BITS * (c % IPB);
+}
+
+// s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
 // Norm of a vector from the fp32 sum of its squares.  Reciprocal square root plus one Newton step is correctly
 // rounded except for a vanishing fraction of inputs.  Sums below 1e-35 (norm < 1e-17: it vanishes both in
 // norm + 1e-8 and in fp16) count as zero; infinite and NaN sums pass through.

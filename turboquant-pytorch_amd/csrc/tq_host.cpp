@@ -308,7 +308,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
 long long tq_qjl_table_bytes(int head_dim, int mse_bits) {
     if (head_dim != TQ_HEAD_DIM) return TQ_ERR_HEAD_DIM;
     if (mse_bits < 1 || mse_bits > 7) return TQ_ERR_BITS;
-    return (long long)sizeof(TqQjlHeader) + 4ll * TQ_OPERAND_BYTES + 1024;
+    return (long long)sizeof(TqQjlHeader) + 6ll * TQ_OPERAND_BYTES + 2048;
 }
 
 int tq_qjl_table_build(const float *Pi, const float *S, const float *centroids, int head_dim, int mse_bits,
@@ -348,6 +348,8 @@ int tq_qjl_table_build(const float *Pi, const float *S, const float *centroids, 
     hd.off_pit = sizeof(TqQjlHeader);
     hd.off_s = hd.off_pit + 2 * TQ_OPERAND_BYTES;
     hd.off_centroids = hd.off_s + 2 * TQ_OPERAND_BYTES;
+    hd.off_m = hd.off_centroids + 1024;
+    hd.off_cent_f32 = hd.off_m + 2 * TQ_OPERAND_BYTES;
     hd.total_bytes = (uint32_t)need;
     hd.k_scale = std::ldexp(1.0f, -(sh_pit + sh_c));
     uint16_t *pit = reinterpret_cast<uint16_t *>(blob + hd.off_pit);
@@ -367,10 +369,39 @@ int tq_qjl_table_build(const float *Pi, const float *S, const float *centroids, 
                 }
             }
     uint32_t *pairs = reinterpret_cast<uint32_t *>(blob + hd.off_centroids);
+    float *cent_f32 = reinterpret_cast<float *>(blob + hd.off_cent_f32);
     for (int i = 0; i < levels; ++i) {
         uint16_t hi, lo;
         split(centroids[i], sh_c, hi, lo);
         pairs[i] = (uint32_t)hi | ((uint32_t)lo << 16);
+        cent_f32[i] = centroids[i];
+    }
+    {   // M = S Pi^T in double precision, then the same two-term tiles (only the sign of the projection is used: any scale does)
+        std::vector<double> m((size_t)D * D);
+        std::vector<float> mf((size_t)D * D);
+        for (int out = 0; out < D; ++out)
+            for (int k = 0; k < D; ++k) {
+                double acc = 0.0;
+                for (int j = 0; j < D; ++j) acc += (double)S[out * D + j] * (double)Pi[k * D + j];
+                m[(size_t)out * D + k] = acc;
+                mf[(size_t)out * D + k] = (float)acc;
+            }
+        const int sh_m = shift_for(mf.data(), (size_t)D * D);
+        uint16_t *mm = reinterpret_cast<uint16_t *>(blob + hd.off_m);
+        for (int t = 0; t < TQ_TILES; ++t)
+            for (int s = 0; s < TQ_STEPS; ++s)
+                for (int l = 0; l < 64; ++l) {
+                    const int mrow = l % 32, hk = l / 32;
+                    const int a = mrow / 8, h = (mrow / 4) % 2, b = mrow % 4;
+                    const int out = 32 * t + 16 * h + 4 * a + b;
+                    for (int i = 0; i < 8; ++i) {
+                        const size_t o = (((size_t)t * TQ_STEPS + s) * 64 + l) * 8 + i;
+                        const int k = 16 * s + 8 * hk + i;
+                        const double x = std::ldexp(m[(size_t)out * D + k], sh_m);
+                        mm[o] = to_f16((float)x);
+                        mm[term + o] = to_f16((float)(x - (double)from_f16(mm[o])));
+                    }
+                }
     }
     std::memcpy(blob, &hd, sizeof(hd));
     return TQ_OK;

@@ -97,8 +97,14 @@ static_assert(sizeof(TqTableHeader) == 256, "header is one 256-byte block");
 //   S    : projected[out] = sum_k residual[k] * S[out][k]      (only its sign is used: any positive scale does)
 // The centroids come as pairs of fp16 terms of centroid * 2^cent_shift, one 32-bit word per code (hi | lo << 16);
 // k_scale = 2^-(pit_shift + cent_shift) takes the product back.
+// For the one-pass kernel (codes, norms, signs and residual norms from a single read of the input) the table also holds
+//   M = S Pi^T : projected[out] = sum_k (Pi residual)[k] * M[out][k]
+// in the same tiling and term format: with the rotated input y = Pi x that the code search works on anyway, the residual
+// in rotated coordinates is y - norm * centroid(code), coordinate by coordinate (Pi (centroids @ Pi) = centroids up to the
+// rotation's departure from orthogonality, 1e-6 of the residual's own projection), so the inverse rotation never
+// has to be formed.  M is computed in double precision from Pi and S.  The centroids are there as plain floats as well.
 #define TQ_QJL_MAGIC 0x54514a4cu /* "TQJL" */
-#define TQ_QJL_VERSION 2u
+#define TQ_QJL_VERSION 3u
 struct TqQjlHeader {
     uint32_t magic;
     uint32_t version;
@@ -110,6 +116,8 @@ struct TqQjlHeader {
     uint32_t off_centroids;  // uint32[256], the first `levels` used
     uint32_t total_bytes;
     float k_scale;
-    uint32_t reserved[54];
+    uint32_t off_m;          // 2 x TQ_OPERAND_BYTES
+    uint32_t off_cent_f32;   // float[256], the first `levels` used
+    uint32_t reserved[52];
 };
 static_assert(sizeof(TqQjlHeader) == 256, "header is one 256-byte block");
