@@ -165,3 +165,71 @@ def test_v3_orchestration_and_cache_at_head_dim_64(pkg, oracle):
     assert torch.equal(fk[:, :, :144], want)
     with pytest.raises(pkg._native.TqError):
         cache.attend(torch.randn((1, 4, 1, D), device=DEV, dtype=torch.float16), 5)
+
+
+@pytest.mark.parametrize("bits,dtype", [(4, torch.bfloat16), (2, torch.float16), (8, torch.float32), (3, torch.bfloat16)])
+def test_head_dim_64_in_pairs_equals_the_one_by_one_form(pkg, oracle, bits, dtype):
+    """64-wide vectors go through the 128-wide kernels two at a time (as rows rotated by diag(Pi, Pi)) whenever every
+    row of the job holds an even number of tokens that lie 64 elements apart; otherwise one by one through the
+    run-time-dimension kernels.  Both forms against the oracle, and against each other: the same codes (outside the
+    boundary window), norms within one fp16 unit, the same de-quantised values; dense tensors, token slices of a
+    preallocated store at even and odd offsets, job lists that mix both kinds."""
+    native = pkg._native
+    D = 64
+    comp = pkg.MSECompressor(D, bits, seed=11 + bits, device=DEV)
+    Pi, cent = comp.Pi.cpu().numpy(), comp.centroids.cpu().numpy()
+    G = D // (8 // bits)
+    B, H, S = 2, 3, 347                          # odd token count: slices decide which form runs
+    x = outlier_kv((B, H, S, D), seed=40 + bits, dtype=dtype).to(DEV)
+    orc = oracle.COracle(Pi, cent, bits, accum_double=True)
+    ref = orc.compress(x.float().cpu().numpy().reshape(-1, D))
+    ref_idx = ref["idx_bytes"].reshape(B, H, S, G)
+    ref_nrm = ref["vec_norms"].reshape(B, H, S)
+    ref_rot = ref["rotated"].reshape(B, H, S, D)
+
+    def check(out_idx, out_nrm, sl, label):
+        rep = oracle.code_mismatch_report(out_idx.cpu().numpy().reshape(-1, G), np.ascontiguousarray(ref_idx[:, :, sl]).reshape(-1, G),
+                                          np.ascontiguousarray(ref_rot[:, :, sl]).reshape(-1, D), cent, bits, 1e-5)
+        assert rep["outside_window"] == 0 and rep["differ"] <= max(4, 3e-4 * rep["coords"]), (label, rep)
+        ulp = oracle.fp16_ulp_distance(bits16(out_nrm).reshape(-1), np.ascontiguousarray(ref_nrm[:, :, sl]).reshape(-1))
+        assert ulp.max() <= 1, label
+
+    even = comp.compress(x[:, :, :346])          # rows of 346 tokens, 64 apart: pairs
+    odd = comp.compress(x[:, :, :345])           # 345 tokens per row: one by one
+    check(even["idx_bytes"], even["vec_norms"], slice(0, 346), "pairs")
+    check(odd["idx_bytes"], odd["vec_norms"], slice(0, 345), "one by one")
+    whole = comp.compress(x)                     # contiguous: 2 * 3 * 347 = 2082 vectors in one row: pairs across the rows' ends
+    check(whole["idx_bytes"], whole["vec_norms"], slice(0, S), "contiguous")
+    same_codes = (even["idx_bytes"][:, :, :345] == odd["idx_bytes"]).all(-1)
+    assert same_codes.float().mean() > 0.995
+    # a preallocated store: even and odd slot offsets and capacities
+    for cap, t0, n_tok in ((400, 6, 346), (401, 6, 346), (400, 7, 346), (400, 6, 345)):
+        idx = torch.zeros((B, H, cap, G), dtype=torch.uint8, device=DEV)
+        nrm = torch.zeros((B, H, cap), dtype=torch.float16, device=DEV)
+        comp.compress_into(x[:, :, :n_tok], idx[:, :, t0:t0 + n_tok], nrm[:, :, t0:t0 + n_tok])
+        check(idx[:, :, t0:t0 + n_tok], nrm[:, :, t0:t0 + n_tok], slice(0, n_tok), f"store cap {cap} at {t0}, {n_tok} tokens")
+        assert not idx[:, :, :t0].any() and not idx[:, :, t0 + n_tok:].any() and not nrm[:, :, t0 + n_tok:].any()
+        out = torch.zeros((B, H, cap + 3, D), dtype=torch.bfloat16 if dtype == torch.float32 else dtype, device=DEV)
+        comp.decompress_packed(idx[:, :, t0:t0 + n_tok], nrm[:, :, t0:t0 + n_tok], out[:, :, t0:t0 + n_tok])
+        want = oracle.NumpyOracle(Pi, cent, bits).decompress(idx[:, :, t0:t0 + n_tok].cpu().numpy().reshape(-1, G),
+                                                             bits16(nrm[:, :, t0:t0 + n_tok]).reshape(-1))
+        err, _ = rel_l2(out[:, :, t0:t0 + n_tok].float().cpu().numpy().reshape(-1, D), torch.from_numpy(want).to(out.dtype).float().numpy())
+        assert err <= 4e-3, (cap, t0, n_tok, err)
+        assert not out[:, :, :t0].any() and not out[:, :, t0 + n_tok:].any()
+    # job lists: all jobs in pairs; one job that cannot be paired sends the whole launch through the one-by-one kernels
+    for counts in ((64, 2, 258), (64, 1, 257)):
+        jobs = []
+        for k, tokens in enumerate(counts):
+            t = outlier_kv((1, 2, tokens, D), seed=60 + k, dtype=dtype).to(DEV)
+            jobs.append({"states": t, "idx_bytes": torch.empty((1, 2, tokens, G), dtype=torch.uint8, device=DEV),
+                         "vec_norms": torch.empty((1, 2, tokens), dtype=torch.float16, device=DEV), "table": comp.table(),
+                         "bits": bits, "out": torch.empty_like(t)})
+        native.JobList(jobs, torch.device(DEV)).compress()
+        native.JobList([dict(j, states=j["out"]) for j in jobs], torch.device(DEV)).decompress()
+        for j in jobs:
+            r = orc.compress(j["states"].float().cpu().numpy().reshape(-1, D))
+            rep = oracle.code_mismatch_report(j["idx_bytes"].cpu().numpy().reshape(-1, G), r["idx_bytes"], r["rotated"], cent, bits, 1e-5)
+            assert rep["outside_window"] == 0 and rep["differ"] <= max(4, 3e-4 * rep["coords"]), (counts, rep)
+            want = oracle.NumpyOracle(Pi, cent, bits).decompress(j["idx_bytes"].cpu().numpy().reshape(-1, G), bits16(j["vec_norms"]).reshape(-1))
+            err, _ = rel_l2(j["out"].float().cpu().numpy().reshape(-1, D), torch.from_numpy(want).to(j["out"].dtype).float().numpy())
+            assert err <= 4e-3, (counts, err)

@@ -308,7 +308,8 @@ def test_c_abi_argument_errors(pkg):
     # compress / decompress take every multiple of 32 up to 256
     assert lib.tq_table_bytes(80, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(288, 4) == E["HEAD_DIM"]
     assert lib.tq_table_bytes(0, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(128, 9) == E["BITS"]
-    assert 0 < lib.tq_table_bytes(64, 4) < lib.tq_table_bytes(128, 4) < lib.tq_table_bytes(256, 4)
+    assert 0 < lib.tq_table_bytes(32, 4) < lib.tq_table_bytes(128, 4) < lib.tq_table_bytes(256, 4)
+    assert lib.tq_table_bytes(64, 4) > lib.tq_table_bytes(96, 4)      # 64: also the operands of diag(Pi, Pi) for the 128-wide kernels
     cent = np.array([0.1, -0.1], np.float32)
     thr = np.zeros(1, np.float32)
     assert lib.tq_decision_thresholds(cent.ctypes.data, 2, thr.ctypes.data) == E["CODEBOOK"]

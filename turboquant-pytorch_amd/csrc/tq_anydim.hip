@@ -380,6 +380,300 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_ke
     }
 }
 
+// ====================================================================================================================
+// Head dimension 256 with 16-bit elements: the rotation resident in registers, as in the 128-wide kernels.
+//
+// compress: a block is eight waves that share tiles of 32 vectors (16 KiB); wave w keeps the 32 rows [32w, 32w+32) of
+// Pi as MFMA A operands for all 16 steps of the contraction, two 16-bit terms (128 registers).  A tile is fetched with
+// coalesced 16-byte loads one tile ahead, parked in a double-buffered XOR-swizzled LDS tile (one barrier per tile) and
+// read back by every wave as the B operand of 32 matrix instructions.  The sum of squares of a vector is reduced over the
+// 32 lanes that hold its 32 pieces while they park them (a butterfly: the same order for every vector, whatever the
+// launch shape).  The code search of tile j-1 is written between the matrix instructions of tile j (one coordinate per
+// step, from the other accumulator set), so that the vector work runs in their shadow.  65 536 x 4 flop per vector
+// against 640 bytes puts this width on the matrix side of the roofline: the kernel is bound by the matrix rate the part
+// sustains, not by memory.
+template <int DTYPE, int BITS>
+__global__ __launch_bounds__(512, 1) void tq_d256_compress_kernel(TqDevJob job0, const tq_job *jobs) {
+    static_assert(DTYPE == TQ_F16 || DTYPE == TQ_BF16, "16-bit inputs");
+    constexpr int D = 256, STEPS = D / 16, PIECES = D * 2 / 16;     // 32 pieces of 16 bytes per vector
+    constexpr int IPB = 8 / BITS, NB = 16 / IPB, NW = NB < 4 ? 1 : NB / 4;
+    constexpr int TILE_BYTES = 32 * D * 2;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t *lds_grid = lds;                                                        // single copy, bases unshifted
+    uint8_t (*lds_stage)[TILE_BYTES] = reinterpret_cast<uint8_t (*)[TILE_BYTES]>(lds + TQ_GRID_LDS_BYTES);
+    float (*lds_ss)[32] = reinterpret_cast<float (*)[32]>(lds + TQ_GRID_LDS_BYTES + 2 * TILE_BYTES);     // [3][32]
+
+    const TqDevJob job = tq_uniform_job(tq_load_job(job0, jobs, blockIdx.y, 2));
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = tq_uniform32(tid >> 6);
+    const uint32_t n = lane & 31u, hk = lane >> 5;
+    const uint32_t n_tiles = (job.n_vec + 31u) / 32u;
+    if (blockIdx.x >= n_tiles) return;        // also: an empty job of a batch, whose table may be NULL
+    const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
+
+    // loads of a tile: piece i = l * 512 + tid of the tile's 1024 is piece i % 32 of vector i / 32, so that the 32 pieces
+    // of a vector sit in 32 consecutive lanes; vectors past the end re-read the job's last one (never stored)
+    const uint32_t ld_vec = tid >> 5, ld_piece = tid & 31u;
+    tq_u4 pre[2];
+    auto issue_loads = [&](uint32_t tl) {
+#pragma unroll
+        for (int l = 0; l < 2; ++l) {
+            uint32_t v = tl * 32u + l * 16u + ld_vec;
+            v = v < job.n_vec ? v : job.n_vec - 1u;
+            pre[l] = tq_gload16(job.states + tq_vec_offset(job, v) + ld_piece * 16u);
+        }
+    };
+    issue_loads(blockIdx.x);
+
+    tq_u4 areg[2][STEPS];
+    {
+        const uint8_t *src = job.table + (DTYPE == TQ_F16 ? hd->off_a_f16 : hd->off_a_bf16);
+#pragma unroll
+        for (int term = 0; term < 2; ++term)
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+                areg[term][s] = tq_gload16(src + (size_t)term * TQ_OPERAND_BYTES_FOR(D) + (((size_t)wave * STEPS + s) * 64 + lane) * 16);
+    }
+    tq_copy_to_lds(lds_grid, job.table + hd->off_grid, hd->grid_cells * 8u, tid, 512u);
+    const float grid_scale = hd->grid_scale, grid_bias = hd->grid_bias;
+
+    // park the prefetched tile in buffer b and leave the vectors' sums of squares in slot `slot`
+    auto park = [&](uint32_t b, uint32_t slot) {
+#pragma unroll
+        for (int l = 0; l < 2; ++l) {
+            const uint32_t v = l * 16u + ld_vec;
+            *reinterpret_cast<tq_u4 *>(lds_stage[b] + v * (D * 2) + ((ld_piece ^ (v & 31u)) << 4)) = pre[l];
+            float s = sumsq8<DTYPE>(pre[l], 0.f);
+#pragma unroll
+            for (int m = 1; m < 32; m <<= 1) s += __shfl_xor(s, m);
+            if (ld_piece == 0u) lds_ss[slot][v] = s;
+        }
+    };
+    // B operand of step s: piece (2 s + hk) ^ (n & 31) of row n = the piece of step 0 with 32 s toggled in its byte offset
+    const uint32_t op_base = n * (D * 2) + ((hk ^ (n & 31u)) << 4);
+    const uint32_t g_bytes = D / IPB;
+
+    // iteration j: rotate tile j into acc_new, search tile j-1 from acc_old
+    auto iteration = [&](auto rot_tag, auto search_tag, uint32_t j, tq_f16v &acc_new, const tq_f16v &acc_old) {
+        constexpr bool ROT = decltype(rot_tag)::value, SEARCH = decltype(search_tag)::value;
+        const uint8_t *stage = lds_stage[j & 1u];
+        float nrm = 0.f, inv = 0.f, inv_cell = 0.f;
+        if constexpr (SEARCH) {
+            nrm = tq_norm_from_sumsq(lds_ss[(j + 2u) % 3u][n]);       // tile j-1 sits in slot (j-1) % 3
+            inv = __builtin_amdgcn_rcpf(nrm + 1e-8f);
+            if (DTYPE == TQ_F16) inv *= 1.0f / (float)(1 << TQ_F16_PI_SHIFT);
+            inv_cell = inv * grid_scale;
+        }
+        if constexpr (ROT) acc_new = tq_zero16();
+        uint32_t words[NW];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) words[w] = 0u;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            if constexpr (ROT) {
+                const tq_u4 bop = *reinterpret_cast<const tq_u4 *>(stage + (op_base ^ (32u * s)));
+                acc_new = (DTYPE == TQ_F16) ? mfma_f16(areg[0][s], bop, acc_new) : mfma_bf16(areg[0][s], bop, acc_new);
+                acc_new = (DTYPE == TQ_F16) ? mfma_f16(areg[1][s], bop, acc_new) : mfma_bf16(areg[1][s], bop, acc_new);
+            }
+            if constexpr (SEARCH) {     // coordinate 32 w + 16 hk + s of vector n
+                const float a = acc_old[s];
+                const uint32_t addr = __float_as_uint(fmaf(a, inv_cell, grid_bias)) & TQ_GRID_ADDR_MASK;
+                const tq_u2 cell = *reinterpret_cast<const tq_u2 *>(lds_grid + addr);
+                const float t = fmaf(a, inv, -__uint_as_float(cell[0]));
+                const uint32_t code = cell[1] + (~__float_as_uint(t) >> 31);          // base + !(rho < threshold)
+                const int byte = s / IPB, k = s % IPB;                                // most significant code of a byte first
+                words[byte / 4] |= code << (8 * (byte % 4) + BITS * (IPB - 1 - k));
+            }
+            // keep the steps in this order: with all 16 operand reads and table lookups hoisted to the top the kernel
+            // runs out of registers (the rotation alone holds 128)
+            if (s % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (SEARCH) {
+            const uint32_t v = (blockIdx.x + (j - 1u) * gridDim.x) * 32u + n;
+            if (v < job.n_vec) {
+                const uint32_t slot = tq_packed_slot(job, v);
+                uint8_t *dst = job.idx_bytes + (size_t)slot * g_bytes + (2u * wave + hk) * NB;
+                if constexpr (NB == 2) tq_gstore2(reinterpret_cast<uint16_t *>(dst), (uint16_t)words[0]);
+                else if constexpr (NB == 4) *reinterpret_cast<TQ_GLOBAL uint32_t *>((TQ_GLOBAL uint8_t *)dst) = words[0];
+                else if constexpr (NB == 8) { const tq_u2 o = {words[0], words[1]}; tq_gstore8(dst, o); }
+                else { const tq_u4 o = {words[0], words[1], words[2], words[3]}; tq_gstore16(dst, o); }
+                if (wave == 0u && hk == 0u) {
+                    const _Float16 hn = (_Float16)nrm;
+                    tq_gstore2(job.vec_norms + slot, __builtin_bit_cast(uint16_t, hn));
+                }
+            }
+        }
+    };
+
+    const uint32_t m = (n_tiles - blockIdx.x + gridDim.x - 1u) / gridDim.x;     // this block's tiles
+    // one trip: the tile after this one sets out while this one is rotated, and is parked behind the trip's work
+    auto trip = [&](auto rot_tag, auto search_tag, uint32_t j, tq_f16v &acc_new, const tq_f16v &acc_old) {
+        const bool more = j + 1u < m;
+        if (more) issue_loads(blockIdx.x + (j + 1u) * gridDim.x);
+        __syncthreads();        // tile j and its sums are parked, and nobody reads buffer (j + 1) & 1 any more
+        iteration(rot_tag, search_tag, j, acc_new, acc_old);
+        if (more) park((j + 1u) & 1u, (j + 1u) % 3u);
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    park(0u, 0u);
+    tq_f16v acc_a, acc_b;       // tiles with an even index rotate into acc_a, the others into acc_b
+    trip(T{}, F{}, 0u, acc_a, acc_a);
+    uint32_t j = 1;
+    for (; j + 1u < m; j += 2u) {
+        trip(T{}, T{}, j, acc_b, acc_a);
+        trip(T{}, T{}, j + 1u, acc_a, acc_b);
+    }
+    if (j < m) {
+        trip(T{}, T{}, j, acc_b, acc_a);
+        ++j;
+    }
+    if (m & 1u) trip(F{}, T{}, m, acc_b, acc_a);        // the last tile's codes
+    else trip(F{}, T{}, m, acc_a, acc_b);
+}
+
+// decompress: a block is four waves that share tiles of 32 vectors; wave w keeps the rows [64w, 64w+64) of Pi^T as A
+// operands for all 16 steps (the leading fp16 term: 128 registers).  The packed bytes of a tile are fetched one tile
+// ahead (every thread the bytes of 32 codes), turned into fp16 centroids through the byte -> centroids table and parked
+// in a double-buffered swizzled LDS tile that all four waves read as B operands; the scaled, rounded results go through
+// a second LDS tile so that the stores are 512 contiguous bytes per vector.
+template <int DTYPE, int IPB>
+__global__ __launch_bounds__(256, 2) void tq_d256_decompress_kernel(TqDevJob job0, const tq_job *jobs) {
+    static_assert(DTYPE == TQ_F16 || DTYPE == TQ_BF16, "16-bit outputs");
+    constexpr int D = 256, STEPS = D / 16;
+    constexpr int TILE_BYTES = 32 * D * 2;
+    constexpr int ENTRY = 2 * IPB;                 // bytes of a table entry: the fp16 centroids of one packed byte
+    constexpr int RAW = 32 / IPB;                  // packed bytes of a thread's 32 codes: 4, 8, 16, 32
+    constexpr int RW = RAW / 4;                    // as dwords
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t *lds_lut = lds;
+    uint8_t (*lds_y)[TILE_BYTES] = reinterpret_cast<uint8_t (*)[TILE_BYTES]>(lds + 4096);
+    uint8_t *lds_out = lds + 4096 + 2 * TILE_BYTES;
+    float (*lds_norm)[32] = reinterpret_cast<float (*)[32]>(lds + 4096 + 3 * TILE_BYTES);       // [2][32]
+
+    const TqDevJob job = tq_uniform_job(tq_load_job(job0, jobs, blockIdx.y, 2));
+    uint8_t *out_base = const_cast<uint8_t *>(job.states);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = tq_uniform32(tid >> 6);
+    const uint32_t n = lane & 31u, hk = lane >> 5;
+    const uint32_t n_tiles = (job.n_vec + 31u) / 32u;
+    if (blockIdx.x >= n_tiles) return;
+    const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
+    const uint32_t g_bytes = D / IPB;
+
+    // a thread's share of a tile: codes [32 c, 32 c + 32) of vector dv, c = tid % 8
+    const uint32_t dv = tid >> 3, chunk = tid & 7u;
+    uint32_t raw[RW];
+    uint16_t norm_bits = 0;
+    auto issue_loads = [&](uint32_t tl) {
+        uint32_t v = tl * 32u + dv;
+        v = v < job.n_vec ? v : job.n_vec - 1u;
+        const uint32_t slot = tq_packed_slot(job, v);
+        const uint8_t *src = job.idx_bytes + (size_t)slot * g_bytes + chunk * RAW;
+        if constexpr (RW == 1) raw[0] = *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)src);
+        else if constexpr (RW == 2) { const tq_u2 t = tq_gload8(src); raw[0] = t[0]; raw[1] = t[1]; }
+        else {
+#pragma unroll
+            for (int q = 0; q < RW / 4; ++q) {
+                const tq_u4 t = tq_gload16(src + 16 * q);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) raw[4 * q + i] = t[i];
+            }
+        }
+        if (chunk == 0u) norm_bits = tq_gload2(job.vec_norms + slot);
+    };
+    issue_loads(blockIdx.x);
+
+    tq_u4 areg[2][STEPS];       // row tiles 2w, 2w + 1
+    {
+        const uint8_t *src = job.table + hd->off_at_f16;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+                areg[t][s] = tq_gload16(src + (((size_t)(2u * wave + t) * STEPS + s) * 64 + lane) * 16);
+    }
+    tq_copy_to_lds(lds_lut, job.table + hd->off_lut, 256u * ENTRY, tid, 256u);
+    __syncthreads();
+
+    // the prefetched bytes -> 32 fp16 centroids = pieces 4 chunk .. 4 chunk + 3 of row dv of buffer b
+    auto decode = [&](uint32_t b) {
+        uint32_t h[16];         // 32 halves
+#pragma unroll
+        for (int byte = 0; byte < RAW; ++byte) {
+            const uint32_t v = (raw[byte / 4] >> (8 * (byte % 4))) & 0xffu;
+            const uint8_t *e = lds_lut + v * ENTRY;
+            if constexpr (IPB == 1) {
+                const uint32_t c = *reinterpret_cast<const uint16_t *>(e);
+                if (byte & 1) h[byte / 2] |= c << 16; else h[byte / 2] = c;
+            } else if constexpr (IPB == 2) {
+                h[byte] = *reinterpret_cast<const uint32_t *>(e);
+            } else if constexpr (IPB == 4) {
+                const tq_u2 c = *reinterpret_cast<const tq_u2 *>(e);
+                h[2 * byte] = c[0]; h[2 * byte + 1] = c[1];
+            } else {
+                const tq_u4 c = *reinterpret_cast<const tq_u4 *>(e);
+                h[4 * byte] = c[0]; h[4 * byte + 1] = c[1]; h[4 * byte + 2] = c[2]; h[4 * byte + 3] = c[3];
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const tq_u4 o = {h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3]};
+            *reinterpret_cast<tq_u4 *>(lds_y[b] + dv * (D * 2) + (((4u * chunk + q) ^ (dv & 31u)) << 4)) = o;
+        }
+        if (chunk == 0u) lds_norm[b][dv] = (float)__builtin_bit_cast(_Float16, norm_bits);
+    };
+    const uint32_t op_base = n * (D * 2) + ((hk ^ (n & 31u)) << 4);     // B operand of step s: at op_base ^ (32 s)
+
+    const uint32_t m = (n_tiles - blockIdx.x + gridDim.x - 1u) / gridDim.x;
+    decode(0u);
+    for (uint32_t j = 0; j < m; ++j) {
+        const uint32_t tl = blockIdx.x + j * gridDim.x;
+        if (j + 1u < m) issue_loads(tl + gridDim.x);
+        __syncthreads();        // tile j is decoded; the output tile of the last iteration has been read
+        const uint8_t *ys = lds_y[j & 1u];
+        tq_f16v acc[2] = {tq_zero16(), tq_zero16()};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            const tq_u4 b = *reinterpret_cast<const tq_u4 *>(ys + (op_base ^ (32u * s)));
+            acc[0] = mfma_f16(areg[0][s], b, acc[0]);
+            acc[1] = mfma_f16(areg[1][s], b, acc[1]);
+        }
+        // lane (n, hk) holds elements 32 t + 16 hk + r of vector n for its row tiles t = 2w, 2w + 1: pieces 4 t + 2 hk + c
+        const float nrm = lds_norm[j & 1u][n];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                tq_u4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float x0 = acc[t][8 * c + 2 * e] * nrm, x1 = acc[t][8 * c + 2 * e + 1] * nrm;
+                    if constexpr (DTYPE == TQ_F16) {
+                        const tq_half2 hh = {(_Float16)x0, (_Float16)x1};
+                        o[e] = __builtin_bit_cast(uint32_t, hh);
+                    } else {
+                        const tq_bf2 hh = {(__bf16)x0, (__bf16)x1};
+                        o[e] = __builtin_bit_cast(uint32_t, hh);
+                    }
+                }
+                const uint32_t piece = 4u * (2u * wave + t) + 2u * hk + c;
+                *reinterpret_cast<tq_u4 *>(lds_out + n * (D * 2) + ((piece ^ (n & 31u)) << 4)) = o;
+            }
+        __syncthreads();        // the output tile is complete
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {       // 1024 pieces, 256 threads: piece i % 32 of vector i / 32, 512 contiguous bytes per vector
+            const uint32_t i = k * 256u + tid, vl = i >> 5, p = i & 31u;
+            const tq_u4 val = *reinterpret_cast<const tq_u4 *>(lds_out + vl * (D * 2) + ((p ^ (vl & 31u)) << 4));
+            const uint32_t v = tl * 32u + vl;
+            if (v < job.n_vec) tq_gstore16_stream(out_base + tq_vec_offset(job, v) + p * 16u, val);
+        }
+        if (j + 1u < m) decode((j + 1u) & 1u);
+    }
+}
+
 // ---- host side --------------------------------------------------------------------------
 
 constexpr int MAX_DEVICES = 64;
@@ -430,8 +724,36 @@ int launch(K kernel, uint32_t (&raised)[MAX_DEVICES], L lds_for, uint32_t nt_max
     return (int)hipGetLastError();
 }
 
+// Launch of one of the 256-wide kernels: `threads` per block, `resident` blocks per compute unit, `lds` bytes of dynamic LDS.
+template <typename K>
+int launch_d256(K kernel, bool (&raised)[MAX_DEVICES], uint32_t lds, uint32_t threads, int resident, const TqDevJob &job,
+                const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, hipStream_t stream) {
+    int dev = 0, cus = 0;
+    const int rc = device_cus(dev, cus);
+    if (rc) return rc;
+    {
+        std::lock_guard<std::mutex> lock(host_state_mutex);
+        if (!raised[dev]) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return (int)e;
+            raised[dev] = true;
+        }
+    }
+    const uint32_t tiles = (max_vec + 31u) / 32u;
+    const uint32_t bx = tq_blocks_per_job(tiles, cus * resident, n_jobs);
+    hipLaunchKernelGGL(kernel, dim3(bx, (unsigned)n_jobs, 1), dim3(threads, 1, 1), lds, stream, job, jobs_dev);
+    return (int)hipGetLastError();
+}
+
 template <int DTYPE, int BITS>
 int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, hipStream_t s) {
+    if constexpr (DTYPE != TQ_F32) {
+        if (d == 256u) {
+            static bool raised256[MAX_DEVICES] = {};
+            constexpr uint32_t lds = TQ_GRID_LDS_BYTES + 2u * 32u * 256u * 2u + 3u * 32u * 4u;
+            return launch_d256(&tq_d256_compress_kernel<DTYPE, BITS>, raised256, lds, 512u, 1, job, jobs_dev, n_jobs, max_vec, s);
+        }
+    }
     static uint32_t raised[MAX_DEVICES] = {};
     return launch(&tq_anydim_compress_kernel<DTYPE, BITS>, raised, compress_lds_bytes<DTYPE>, AnyIn<DTYPE>::NT, job, jobs_dev,
                   n_jobs, max_vec, d, s);
@@ -451,6 +773,13 @@ int compress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_j
 
 template <int DTYPE, int IPB>
 int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, hipStream_t s) {
+    if constexpr (DTYPE != TQ_F32) {
+        if (d == 256u) {
+            static bool raised256[MAX_DEVICES] = {};
+            constexpr uint32_t lds = 4096u + 3u * 32u * 256u * 2u + 2u * 32u * 4u;
+            return launch_d256(&tq_d256_decompress_kernel<DTYPE, IPB>, raised256, lds, 256u, 2, job, jobs_dev, n_jobs, max_vec, s);
+        }
+    }
     static uint32_t raised[MAX_DEVICES] = {};
     return launch(&tq_anydim_decompress_kernel<DTYPE, IPB>, raised, decompress_lds_bytes, DEC_NT, job, jobs_dev, n_jobs, max_vec, d, s);
 }

@@ -72,7 +72,7 @@ __device__ __forceinline__ bool run_tail(F &step) {
 
 template <int DTYPE, int BITS>
 __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t *workspace,
-                                                                                          uint32_t tshift) {
+                                                                                          uint32_t tshift, uint32_t paired) {
     using T = InTraits<DTYPE>;
     using P = Pack<BITS>;
     constexpr int ELEM = T::ELEM;
@@ -88,9 +88,13 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     __shared__ __attribute__((aligned(16))) uint8_t lds_grid[TQ_GRID_LDS_BYTES];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_stage[RING][STAGE];
     __shared__ float lds_ss[2][32];   // sum of squares of the tile's vectors (16-bit inputs)
+    __shared__ float lds_ssh[2][32][2];   // the same per half of a row (rows that are pairs of 64-wide vectors)
     __shared__ __attribute__((aligned(16))) float lds_part[2][32][4];   // the same, one share per wave (pipelined path)
 
-    const TqDevJob job = tq_uniform_job(tq_load_job(job0, jobs, blockIdx.y, ELEM));
+    // paired: the job's vectors are 64 wide and the kernel works on pairs of them as 128-wide rows (diag(Pi, Pi) from the
+    // table's pair sections).  Everything is as for 128-wide vectors except the norm: one per half of a row; the
+    // coordinates of wave w belong to half w / 2.
+    const TqDevJob job = tq_uniform_job(tq_pair_job(tq_load_job(job0, jobs, blockIdx.y, ELEM), paired != 0u));
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
@@ -137,7 +141,8 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     // Every cell is fetched once and written to all its copies; the fetches of a thread are issued together.
     // Called once per block: behind the first tile loads on the pipelined path, so that their latencies overlap.
     auto load_tables = [&]() {
-        const uint8_t *src = job.table + (DTYPE == TQ_F16 ? hd->off_a_f16 : hd->off_a_bf16);
+        const uint8_t *src = job.table + (paired ? (DTYPE == TQ_F16 ? hd->off_pair_a_f16 : hd->off_pair_a_bf16)
+                                                 : (DTYPE == TQ_F16 ? hd->off_a_f16 : hd->off_a_bf16));
 #pragma unroll
         for (int term = 0; term < T::TERMS; ++term)
 #pragma unroll
@@ -169,6 +174,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
 
     const uint32_t ld_vec = lane / PIECES, ld_piece = lane % PIECES;  // role in the coalesced loads
     const uint32_t n = lane & 31u, hk = lane >> 5;                    // role in the MFMA: column, half
+    const uint32_t half = wave >> 1;                                  // paired rows: the 64-wide vector this wave's coordinates belong to
 
     // LDS offset of this lane's piece of load j (computed where it is used: these paths are not the hot one)
     auto st_off = [&](int j) {
@@ -212,6 +218,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
                 const float pair = share + row_shr(share, std::integral_constant<int, 4>{});                // at p == 7, 15
                 const float total = pair + row_shr(pair, std::integral_constant<int, 8>{});                 // at p == 15
                 if ((lane & 15u) == 15u) lds_ss[b][(wave * NLOAD + j) * VEC_PER_LOAD + ld_vec] = total;
+                if ((lane & 7u) == 7u) lds_ssh[b][(wave * NLOAD + j) * VEC_PER_LOAD + ld_vec][(lane >> 3) & 1u] = pair;   // pieces 0..7, 8..15
             }
         }
     };
@@ -236,8 +243,10 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             float x[8];
 #pragma unroll
             for (int i = 0; i < 4; ++i) { x[i] = __uint_as_float(q0[i]); x[4 + i] = __uint_as_float(q1[i]); }
+            if (!paired || (sg >> 2) == half) {      // (a half row: the four steps that cover it)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) { if (i & 1) ss1 = fmaf(x[i], x[i], ss1); else ss0 = fmaf(x[i], x[i], ss0); }
+                for (int i = 0; i < 8; ++i) { if (i & 1) ss1 = fmaf(x[i], x[i], ss1); else ss0 = fmaf(x[i], x[i], ss0); }
+            }
             tq_u4 xt[3];
             split_f32x8(x, xt[0], xt[1], xt[2]);
             // all products whose weight is >= 2^-24 of the leading one: (x term i, Pi term j), i + j <= 2
@@ -262,7 +271,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
     auto scale_of = [&](uint32_t b, float ss0, float ss1) {
         float ss;
         if constexpr (ELEM == 2) {
-            ss = lds_ss[b][n];
+            ss = paired ? lds_ssh[b][n][half] : lds_ss[b][n];
         } else {
             ss = ss0 + ss1;                 // both lanes of a vector hold half of the squares
             ss += __shfl_xor(ss, 32);
@@ -343,6 +352,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
         tq_gstore2(ndst, __builtin_bit_cast(uint16_t, hn));
     };
     const uint32_t lane_slot = (2u * wave + hk) * NB;   // this lane's bytes inside a vector's G = 8 * NB
+    auto norm_slot = [&](size_t slot) { return paired ? 2u * slot + half : slot; };     // where the norm of this wave's half of row `slot` goes
 
     uint32_t buf = 0;
     uint32_t words[NW];
@@ -449,12 +459,13 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             // output addresses: a base per tile that is the same in every lane, plus a per-lane constant
             const uint32_t cd_lane = n * (8 * NB) + lane_slot, nd_lane = n;
             auto store_tile = [&](uint32_t tl, const uint32_t (&w)[NW], float nrm_of_tile) {
-                store(job.idx_bytes + (size_t)tl * (32u * (8 * NB)) + cd_lane, job.vec_norms + (size_t)tl * 32u + nd_lane, w, nrm_of_tile);
+                store(job.idx_bytes + (size_t)tl * (32u * (8 * NB)) + cd_lane, job.vec_norms + norm_slot((size_t)tl * 32u + nd_lane), w, nrm_of_tile);
             };
 
             auto scale_from_shares = [&](uint32_t par) {
                 const float4 q = *reinterpret_cast<const float4 *>(&lds_part[par][n][0]);
-                return scale_from_ss((q.x + q.y) + (q.z + q.w));
+                const float lo_half = q.x + q.y, hi_half = q.z + q.w;
+                return scale_from_ss(paired ? (half ? hi_half : lo_half) : lo_half + hi_half);
             };
             // iteration j: slot = j % P; `acc_new` receives t_j, `acc_old` holds t_{j-1}
             auto iteration = [&](auto with_search, auto slot_tag, bool warm, uint32_t par, tq_f16v &acc_new, const tq_f16v &acc_old) {
@@ -617,7 +628,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
             __syncthreads();
             compute(buf, words, nrm);
             const uint32_t slot = tq_packed_slot(job, tile * 32u + n);
-            store(job.idx_bytes + (size_t)slot * (8 * NB) + lane_slot, job.vec_norms + slot, words, nrm);
+            store(job.idx_bytes + (size_t)slot * (8 * NB) + lane_slot, job.vec_norms + norm_slot(slot), words, nrm);
             buf ^= 1u;
             park(buf, pre);
             tile = next;
@@ -632,7 +643,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
         const uint32_t v = tile * 32u + n;
         if (v < job.n_vec) {
             const uint32_t slot = tq_packed_slot(job, v);
-            store(job.idx_bytes + (size_t)slot * (8 * NB) + lane_slot, job.vec_norms + slot, words, nrm);
+            store(job.idx_bytes + (size_t)slot * (8 * NB) + lane_slot, job.vec_norms + norm_slot(slot), words, nrm);
         }
     }
     report_done();
@@ -674,7 +685,7 @@ int query_device(DeviceInfo &info) {
 #endif
 
 template <int DTYPE, int BITS>
-int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *workspace, hipStream_t stream) {
+int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *workspace, bool paired, hipStream_t stream) {
     DeviceInfo info;
     int rc = query_device(info);
     if (rc) return rc;
@@ -707,28 +718,28 @@ int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uin
         }
     }
     dim3 grid(bx, (unsigned)n_jobs, 1), block(CTHREADS, 1, 1);
-    hipLaunchKernelGGL((tq_compress_kernel<DTYPE, BITS>), grid, block, 0, stream, job, jobs_dev, counters, tshift);
+    hipLaunchKernelGGL((tq_compress_kernel<DTYPE, BITS>), grid, block, 0, stream, job, jobs_dev, counters, tshift, paired ? 1u : 0u);
     return (int)hipGetLastError();
 }
 
 template <int DTYPE>
-int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, hipStream_t s) {
+int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, bool paired, hipStream_t s) {
     switch (bits) {
-        case 1: return launch_compress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case 2: return launch_compress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case 3: return launch_compress<DTYPE, 3>(job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case 4: return launch_compress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case 1: return launch_compress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case 2: return launch_compress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case 3: return launch_compress<DTYPE, 3>(job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case 4: return launch_compress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
         case 5: case 6: case 7: case 8:  // one code per byte: identical packing
-            return launch_compress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, ws, s);
+            return launch_compress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
         default: return TQ_ERR_BITS;
     }
 }
 
-int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, hipStream_t s) {
+int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, bool paired, hipStream_t s) {
     switch (dtype) {
-        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
         default: return TQ_ERR_DTYPE;
     }
 }
@@ -779,9 +790,11 @@ extern "C" int tq_compress(const void *states, int dtype, long long rows, long l
     job.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     job.row_stride = row_stride * elem_bytes(dtype);
     job.token_stride = token_stride * elem_bytes(dtype);
+    if (head_dim == TQ_HEAD_DIM / 2 && tq_pairable(rows, tokens, token_stride, packed_row_stride, head_dim))
+        return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec / 2 + 31) / 32), workspace, true, static_cast<hipStream_t>(stream));
     if (head_dim != TQ_HEAD_DIM)
         return tq_anydim_compress(dtype, bits, head_dim, job, nullptr, 1, (uint32_t)n_vec, static_cast<hipStream_t>(stream));
-    return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), workspace, static_cast<hipStream_t>(stream));
+    return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), workspace, false, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
@@ -791,6 +804,7 @@ extern "C" int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_d
     if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
     if ((uintptr_t)workspace & 63u) return TQ_ERR_ALIGN;
     long long max_vec = 0;
+    bool paired = head_dim == TQ_HEAD_DIM / 2;     // 64-wide vectors in pairs, if every job of the launch allows it
     for (int i = 0; i < n_jobs; ++i) {
         const tq_job &j = jobs_host[i];
         if (j.bits != jobs_host[0].bits) return TQ_ERR_BITS;
@@ -800,12 +814,16 @@ extern "C" int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_d
                                  head_dim, j.bits, j.idx_bytes, j.vec_norms, j.packed_row_stride, &n_vec);
         if (rc) return rc;
         if (n_vec > max_vec) max_vec = n_vec;
+        if (n_vec && !tq_pairable(j.rows, j.tokens, j.token_stride, j.packed_row_stride, head_dim)) paired = false;
     }
     if (max_vec == 0) return TQ_OK;
     TqDevJob none{};
+    if (paired)
+        return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec / 2 + 31) / 32),
+                        workspace, true, static_cast<hipStream_t>(stream));
     if (head_dim != TQ_HEAD_DIM)
         return tq_anydim_compress(jobs_host[0].dtype, jobs_host[0].bits, head_dim, none, jobs_dev, n_jobs, (uint32_t)max_vec,
                                   static_cast<hipStream_t>(stream));
     return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec + 31) / 32),
-                    workspace, static_cast<hipStream_t>(stream));
+                    workspace, false, static_cast<hipStream_t>(stream));
 }

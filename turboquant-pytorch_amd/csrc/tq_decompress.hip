@@ -61,7 +61,7 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
 }
 
 template <int DTYPE, int IPB>
-__global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t *workspace) {
+__global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t *workspace, uint32_t paired) {
     using T = OutTraits<DTYPE>;
     constexpr int ELEM = T::ELEM;
     constexpr int VEC_BYTES = TQ_HEAD_DIM * ELEM;   // 256 or 512
@@ -74,7 +74,9 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    const TqDevJob job = tq_load_job(job0, jobs, blockIdx.y, ELEM);
+    // paired: the job's vectors are 64 wide; two neighbours are one 128-wide row here (diag(Pi, Pi)^T from the table's pair
+    // section).  Lane half hk decodes and produces the second vector of the pair; only its norm is its own.
+    const TqDevJob job = tq_pair_job(tq_load_job(job0, jobs, blockIdx.y, ELEM), paired != 0u);
     uint8_t *out_base = const_cast<uint8_t *>(job.states);
 
     const uint32_t tid = threadIdx.x;
@@ -114,7 +116,7 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
         constexpr int NT = T::WAVES * TQ_WAVE;
         constexpr int A_TRIPS = TQ_OPERAND_BYTES / 16 / NT;
         static_assert(A_TRIPS * NT * 16 == TQ_OPERAND_BYTES, "whole trips");
-        const uint8_t *a_src = job.table + hd->off_at_f16;
+        const uint8_t *a_src = job.table + (paired ? hd->off_pair_at_f16 : hd->off_at_f16);
         tq_u4 v[A_TRIPS];
 #pragma unroll
         for (int k = 0; k < A_TRIPS; ++k) v[k] = tq_gload16(a_src + 16u * (tid + k * NT));
@@ -185,7 +187,7 @@ __global__ __launch_bounds__(OutTraits<DTYPE>::WAVES *TQ_WAVE) void tq_decompres
                 for (int i = 0; i < 4; ++i) raw[4 * q + i] = t[i];
             }
         }
-        norm_bits = tq_gload2(job.vec_norms + slot);
+        norm_bits = tq_gload2(job.vec_norms + (paired ? 2u * (size_t)slot + hk : (size_t)slot));
     };
 
     // one tile: decode + rotate + scale + transpose + store
@@ -388,7 +390,7 @@ int static_counters(uint32_t **out) {
 }
 
 template <int DTYPE, int IPB>
-int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *workspace,
+int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *workspace, bool paired,
                       hipStream_t stream) {
     using T = OutTraits<DTYPE>;
     int cus = 0;
@@ -414,26 +416,26 @@ int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, u
     dim3 grid(bx, (unsigned)n_jobs, 1), block(T::WAVES * TQ_WAVE, 1, 1);
     // tickets pay off once every block has several to draw; below that the fixed assignment starts sooner
     uint32_t *counters = want >= 4u * bx ? static_cast<uint32_t *>(workspace) : nullptr;
-    hipLaunchKernelGGL((tq_decompress_kernel<DTYPE, IPB>), grid, block, lds, stream, job, jobs_dev, counters);
+    hipLaunchKernelGGL((tq_decompress_kernel<DTYPE, IPB>), grid, block, lds, stream, job, jobs_dev, counters, paired ? 1u : 0u);
     return (int)hipGetLastError();
 }
 
 template <int DTYPE>
-int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, hipStream_t s) {
+int dispatch_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, bool paired, hipStream_t s) {
     switch (8 / bits) {
-        case 8: return launch_decompress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case 4: return launch_decompress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case 2: return launch_decompress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case 1: return launch_decompress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case 8: return launch_decompress<DTYPE, 8>(job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case 4: return launch_decompress<DTYPE, 4>(job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case 2: return launch_decompress<DTYPE, 2>(job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case 1: return launch_decompress<DTYPE, 1>(job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
         default: return TQ_ERR_BITS;
     }
 }
 
-int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, hipStream_t s) {
+int dispatch(int dtype, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_tiles, void *ws, bool paired, hipStream_t s) {
     switch (dtype) {
-        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
-        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, s);
+        case TQ_F32: return dispatch_bits<TQ_F32>(bits, job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case TQ_F16: return dispatch_bits<TQ_F16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
+        case TQ_BF16: return dispatch_bits<TQ_BF16>(bits, job, jobs_dev, n_jobs, max_tiles, ws, paired, s);
         default: return TQ_ERR_DTYPE;
     }
 }
@@ -483,9 +485,11 @@ extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms
     job.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     job.row_stride = row_stride * elem_bytes(out_dtype);
     job.token_stride = token_stride * elem_bytes(out_dtype);
+    if (head_dim == TQ_HEAD_DIM / 2 && tq_pairable(rows, tokens, token_stride, packed_row_stride, head_dim))
+        return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec / 2 + 31) / 32), workspace, true, static_cast<hipStream_t>(stream));
     if (head_dim != TQ_HEAD_DIM)     // the run-time-dimension kernel assigns its tiles statically: no counters
         return tq_anydim_decompress(out_dtype, bits, head_dim, job, nullptr, 1, (uint32_t)n_vec, static_cast<hipStream_t>(stream));
-    return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), workspace, static_cast<hipStream_t>(stream));
+    return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec + 31) / 32), workspace, false, static_cast<hipStream_t>(stream));
 }
 
 extern "C" long long tq_workspace_bytes(int n_jobs) {
@@ -495,8 +499,9 @@ extern "C" long long tq_workspace_bytes(int n_jobs) {
 
 namespace {
 // Argument checks of a batch; max_vec = vectors of its largest job (0: nothing to launch).
-int check_batch(const tq_job *jobs_host, int n_jobs, int head_dim, long long *max_vec) {
+int check_batch(const tq_job *jobs_host, int n_jobs, int head_dim, long long *max_vec, bool *paired) {
     *max_vec = 0;
+    *paired = head_dim == TQ_HEAD_DIM / 2;       // 64-wide vectors in pairs, if every job of the launch allows it
     for (int i = 0; i < n_jobs; ++i) {
         const tq_job &j = jobs_host[i];
         if (8 / (j.bits < 1 || j.bits > 8 ? 1 : j.bits) != 8 / (jobs_host[0].bits < 1 || jobs_host[0].bits > 8 ? 1 : jobs_host[0].bits))
@@ -507,18 +512,22 @@ int check_batch(const tq_job *jobs_host, int n_jobs, int head_dim, long long *ma
                                  head_dim, j.bits, j.idx_bytes, j.vec_norms, j.packed_row_stride, &n_vec);
         if (rc) return rc;
         if (n_vec > *max_vec) *max_vec = n_vec;
+        if (n_vec && !tq_pairable(j.rows, j.tokens, j.token_stride, j.packed_row_stride, head_dim)) *paired = false;
     }
     return TQ_OK;
 }
 
-int launch_batch(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs, int head_dim, long long max_vec,
+int launch_batch(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs, int head_dim, long long max_vec, bool paired,
                  void *workspace, void *stream) {
     TqDevJob none{};
+    if (paired)
+        return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec / 2 + 31) / 32),
+                        workspace, true, static_cast<hipStream_t>(stream));
     if (head_dim != TQ_HEAD_DIM)
         return tq_anydim_decompress(jobs_host[0].dtype, jobs_host[0].bits, head_dim, none, jobs_dev, n_jobs, (uint32_t)max_vec,
                                     static_cast<hipStream_t>(stream));
     return dispatch(jobs_host[0].dtype, jobs_host[0].bits, none, jobs_dev, n_jobs, (uint32_t)((max_vec + 31) / 32),
-                    workspace, static_cast<hipStream_t>(stream));
+                    workspace, false, static_cast<hipStream_t>(stream));
 }
 }  // namespace
 
@@ -529,9 +538,10 @@ extern "C" int tq_decompress_batched(const tq_job *jobs_host, const tq_job *jobs
     if (n_jobs < 0 || n_jobs > TQ_MAX_JOBS) return TQ_ERR_SIZE;
     if ((uintptr_t)workspace & 63u) return TQ_ERR_ALIGN;
     long long max_vec = 0;
-    const int rc = check_batch(jobs_host, n_jobs, head_dim, &max_vec);
+    bool paired = false;
+    const int rc = check_batch(jobs_host, n_jobs, head_dim, &max_vec, &paired);
     if (rc || max_vec == 0) return rc;
-    return launch_batch(jobs_host, jobs_dev, n_jobs, head_dim, max_vec, workspace, stream);
+    return launch_batch(jobs_host, jobs_dev, n_jobs, head_dim, max_vec, paired, workspace, stream);
 }
 
 extern "C" int tq_decompress_batched_noalloc(const tq_job *jobs_host, const tq_job *jobs_dev, int n_jobs,
@@ -542,7 +552,8 @@ extern "C" int tq_decompress_batched_noalloc(const tq_job *jobs_host, const tq_j
     if (n_jobs > TQ_NOALLOC_MAX_JOBS) return TQ_ERR_CAPACITY;
     // every argument is checked before anything is launched: an argument error leaves the stream untouched
     long long max_vec = 0;
-    int rc = check_batch(jobs_host, n_jobs, head_dim, &max_vec);
+    bool paired = false;
+    int rc = check_batch(jobs_host, n_jobs, head_dim, &max_vec, &paired);
     if (rc || max_vec == 0) return rc;
     uint32_t *counters = nullptr;
     rc = static_counters(&counters);
@@ -554,5 +565,5 @@ extern "C" int tq_decompress_batched_noalloc(const tq_job *jobs_host, const tq_j
                        counters, words);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    return launch_batch(jobs_host, jobs_dev, n_jobs, head_dim, max_vec, counters, stream);
+    return launch_batch(jobs_host, jobs_dev, n_jobs, head_dim, max_vec, paired, counters, stream);
 }

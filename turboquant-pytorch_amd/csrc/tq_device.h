@@ -46,6 +46,18 @@ __device__ __forceinline__ TqDevJob tq_load_job(const TqDevJob &single, const tq
     return job;
 }
 
+// Two 64-wide vectors that lie next to each other are one 128-wide row to the 128-wide kernels (rotated by diag(Pi, Pi)):
+// the job seen that way.  The host has checked that every row holds an even number of tokens, 64 elements apart.
+__device__ __forceinline__ TqDevJob tq_pair_job(TqDevJob j, bool paired) {
+    if (paired) {
+        j.n_vec >>= 1;
+        j.tokens >>= 1;
+        j.packed_row_stride >>= 1;
+        j.token_stride <<= 1;
+    }
+    return j;
+}
+
 // The job's fields are the same in every lane of a block, but a record fetched from the job array arrives in vector
 // registers (the compiler cannot prove that nobody writes the array).  Moving every field into scalar registers keeps
 // them out of the vector register budget and lets the address arithmetic on them run on the scalar unit.
@@ -318,6 +330,14 @@ __device__ __forceinline__ tq_u4 decode_rep(const uint32_t (&raw)[NW], int s, co
         out = *reinterpret_cast<const tq_u4 *>(lut + (b << 7));
     }
     return out;
+}
+
+// 64-wide vectors can go through the 128-wide kernels two at a time when the two vectors of every pair are neighbours in
+// memory and in the packed store, and no pair straddles two rows: an even number of tokens per row, 64 elements apart,
+// an even packed row stride.
+static inline bool tq_pairable(long long rows, long long tokens, long long token_stride, long long packed_row_stride, int head_dim) {
+    (void)rows;
+    return head_dim == TQ_HEAD_DIM / 2 && tokens > 0 && (tokens & 1) == 0 && token_stride == head_dim && (packed_row_stride & 1) == 0;
 }
 
 // Blocks per job for a (blocks_per_job x n_jobs) grid of equal-cost blocks on `cus` compute units

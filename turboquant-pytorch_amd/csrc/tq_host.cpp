@@ -96,6 +96,7 @@ inline uint32_t grid_cell(float r, float scale, float bias) {
 struct Layout {
     uint32_t off_a_f16, off_a_bf16, off_grid, off_at_f16, off_lut, off_centroids, off_thresholds, total;
     uint32_t lut_entry_bytes;
+    uint32_t off_pair_a_f16, off_pair_a_bf16, off_pair_at_f16;     // head_dim 64: room for the operands of diag(Pi, Pi)
 };
 // head dimensions the kernels take: 128 (the tuned kernels) and the other multiples of 32 up to 256
 bool supported_head_dim(int d) { return d >= TQ_ANYDIM_MIN && d <= TQ_ANYDIM_MAX && d % 32 == 0; }
@@ -113,6 +114,11 @@ Layout layout_for(int head_dim, int bits) {
     L.off_lut = off;        off += round_up(256 * L.lut_entry_bytes, 256);
     L.off_centroids = off;  off += round_up(levels * 4, 256);
     L.off_thresholds = off; off += round_up(levels * 4, 256);
+    if (head_dim == TQ_HEAD_DIM / 2) {
+        L.off_pair_a_f16 = off;  off += 2 * TQ_OPERAND_BYTES;
+        L.off_pair_a_bf16 = off; off += 3 * TQ_OPERAND_BYTES;
+        L.off_pair_at_f16 = off; off += 2 * TQ_OPERAND_BYTES;
+    }
     L.total = off;
     return L;
 }
@@ -182,6 +188,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     const int levels = 1 << bits;
     const int D = head_dim;
     const bool tuned = D == TQ_HEAD_DIM;   // the 128-wide kernels have their own decompress tiling and keep shifted grid copies
+    const bool tuned_grid = tuned || D == TQ_HEAD_DIM / 2;     // 64-wide vectors go through them in pairs: the same grid limit
     if (!valid_codebook(centroids, levels)) return TQ_ERR_CODEBOOK;
     for (int i = 0; i < D * D; ++i)
         if (!std::isfinite(Pi[i])) return TQ_ERR_SIZE;
@@ -210,7 +217,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     for (int lg = 3; lg <= 12 && !ok; ++lg) {
         scale = (float)(1 << lg);
         cells = 2u * (uint32_t)std::ceil(range * scale);
-        if (cells > (uint32_t)(tuned ? TQ_GRID_MAX_CELLS(bits) : TQ_GRID_LDS_BYTES / 8)) break;
+        if (cells > (uint32_t)(tuned_grid ? TQ_GRID_MAX_CELLS(bits) : TQ_GRID_LDS_BYTES / 8)) break;
         bias = (float)(cells / 2) + TQ_GRID_MAGIC;
         grid.assign(cells, TqGridCell{INFINITY, 0});
         auto edge = [&](uint32_t k) { return ((double)k - (double)(cells / 2) - 0.0625) / (double)scale; };
@@ -273,6 +280,48 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
                 }
             }
 
+    // ---- head_dim 64: the same operand sets for diag(Pi, Pi) in the tilings of the 128-wide kernels ----
+    const bool paired = D == TQ_HEAD_DIM / 2 && cells <= (uint32_t)TQ_GRID_MAX_CELLS(bits);
+    if (paired) {
+        const int W = TQ_HEAD_DIM;
+        auto pp = [&](int row, int col) { return (row / D == col / D) ? Pi[(row % D) * D + (col % D)] : 0.0f; };   // diag(Pi, Pi)[row][col]
+        uint16_t *pa_f16 = reinterpret_cast<uint16_t *>(blob + L.off_pair_a_f16);
+        uint16_t *pa_bf16 = reinterpret_cast<uint16_t *>(blob + L.off_pair_a_bf16);
+        uint16_t *pat_f16 = reinterpret_cast<uint16_t *>(blob + L.off_pair_at_f16);
+        const size_t pterm = (size_t)TQ_OPERAND_BYTES / 2;
+        for (int t = 0; t < TQ_TILES; ++t)
+            for (int s = 0; s < TQ_STEPS; ++s)
+                for (int l = 0; l < 64; ++l) {
+                    const int m = l % 32, hk = l / 32;
+                    const int a = m / 8, h = (m / 4) % 2, b = m % 4;
+                    const int out_c = 32 * t + 16 * h + 4 * a + b;
+                    const int out_d = 64 * h + 16 * t + 4 * a + b;
+                    for (int i = 0; i < 8; ++i) {
+                        const size_t o = (((size_t)t * TQ_STEPS + s) * 64 + l) * 8 + i;
+                        {
+                            const float p = pp(out_c, 16 * s + 8 * hk + i);
+                            const double ps = (double)p * pi_scale;
+                            const uint16_t hi = to_f16((float)ps);
+                            pa_f16[o] = hi;
+                            pa_f16[pterm + o] = to_f16((float)(ps - (double)from_f16(hi)));
+                            const uint16_t b0 = to_bf16(p);
+                            const float r1 = p - from_bf16(b0);
+                            const uint16_t b1 = to_bf16(r1);
+                            pa_bf16[o] = b0;
+                            pa_bf16[pterm + o] = b1;
+                            pa_bf16[2 * pterm + o] = to_bf16((r1 - from_bf16(b1)));
+                        }
+                        {
+                            const float p = pp(64 * hk + 8 * s + i, out_d);
+                            const uint16_t hi = to_f16(p);
+                            pat_f16[o] = hi;
+                            pat_f16[pterm + o] = to_f16((float)((double)p - (double)from_f16(hi)));
+                        }
+                    }
+                }
+        (void)W;
+    }
+
     // ---- decode table: byte value -> the ipb centroids it holds (MSB-first), as fp16 ----
     const int ipb = 8 / bits;
     const unsigned mask = (1u << bits) - 1u;
@@ -298,6 +347,9 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     hd.off_grid = L.off_grid;
     hd.off_at_f16 = L.off_at_f16;
     hd.off_lut = L.off_lut;
+    hd.off_pair_a_f16 = paired ? L.off_pair_a_f16 : 0u;
+    hd.off_pair_a_bf16 = paired ? L.off_pair_a_bf16 : 0u;
+    hd.off_pair_at_f16 = paired ? L.off_pair_at_f16 : 0u;
     hd.off_centroids = L.off_centroids;
     hd.off_thresholds = L.off_thresholds;
     hd.lut_entry_bytes = L.lut_entry_bytes;

@@ -6,7 +6,7 @@
 #include <stdint.h>
 
 #define TQ_TABLE_MAGIC 0x54514d49u /* "TQMI" */
-#define TQ_TABLE_VERSION 6u
+#define TQ_TABLE_VERSION 7u
 #define TQ_HEAD_DIM 128
 
 // --- MFMA operand tiling (v_mfma_f32_32x32x16_{f16,bf16}) --------------------------------
@@ -85,7 +85,15 @@ struct TqTableHeader {
     uint32_t off_centroids;  // float[levels]
     uint32_t off_thresholds; // float[levels - 1]
     uint32_t lut_entry_bytes; // 2 * ipb
-    uint32_t reserved[45];
+    // head_dim 64 only, and only when the quantiser grid fits the shifted copies of the 128-wide kernels (0 otherwise):
+    // operand sets of the 128 x 128 block-diagonal matrix diag(Pi, Pi) in the tilings of those kernels.  Two consecutive
+    // 64-wide vectors that lie next to each other in memory are one 128-wide row to them; rotated by diag(Pi, Pi), searched
+    // and packed per coordinate, they come out as the two vectors' codes one after the other, which is the packed layout
+    // of two 64-wide vectors.  Only the norm is per half.
+    uint32_t off_pair_a_f16;  // compress operand of diag(Pi, Pi) * 2^shift as fp16 hi, lo     (2 x 32 KiB)
+    uint32_t off_pair_a_bf16; // compress operand of diag(Pi, Pi) as bf16 hi, mid, lo          (3 x 32 KiB)
+    uint32_t off_pair_at_f16; // decompress operand of diag(Pi, Pi)^T as fp16 hi, lo           (2 x 32 KiB)
+    uint32_t reserved[42];
 };
 static_assert(sizeof(TqTableHeader) == 256, "header is one 256-byte block");
 
