@@ -144,8 +144,7 @@ def test_strided_store_and_batched_jobs(pkg, oracle):
 
 
 def test_v3_orchestration_and_cache_at_head_dim_64(pkg, oracle):
-    """TurboQuantV3 and the streaming cache at head_dim 64 (compress_kv / decompress_kv / update); the attention
-    kernels read 128-wide stores only and say so."""
+    """TurboQuantV3 and the streaming cache at head_dim 64 (compress_kv / decompress_kv / update / attend)."""
     D = 64
     tq = pkg.TurboQuantV3(D, key_bits=4, value_bits=2, residual_window=0, layer_idx=5, n_layers=12, protected_layers=2, device=DEV)
     k = outlier_kv((1, 2, 200, D), seed=1, dtype=torch.float16).to(DEV)
@@ -163,8 +162,10 @@ def test_v3_orchestration_and_cache_at_head_dim_64(pkg, oracle):
     assert torch.equal(fk[:, :, -16:], k[:, :, 144:160]) and torch.equal(fv[:, :, -16:], v[:, :, 144:160])
     want = tq.key_compressor.decompress_into(tq.key_compressor.compress(k[:, :, :144]), torch.empty_like(k[:, :, :144]))
     assert torch.equal(fk[:, :, :144], want)
-    with pytest.raises(pkg._native.TqError):
-        cache.attend(torch.randn((1, 4, 1, D), device=DEV, dtype=torch.float16), 5)
+    q = torch.randn((1, 4, 1, D), device=DEV, dtype=torch.float16)
+    got = cache.attend(q, 5)                    # other head dimensions: de-quantised history, then plain attention
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), fk.float().repeat_interleave(2, dim=1), fv.float().repeat_interleave(2, dim=1))
+    assert got.shape == q.shape and float((got.float() - want).norm() / want.norm()) < 5e-3
 
 
 @pytest.mark.parametrize("bits,dtype", [(4, torch.bfloat16), (2, torch.float16), (8, torch.float32), (3, torch.bfloat16)])

@@ -275,12 +275,14 @@ def test_packed_weighted_values_against_oracle(pkg, oracle, bits, group, S):
     assert torch.equal(again, got)                               # fixed summation order
 
 
-@pytest.mark.parametrize("rw,dtype", [(128, torch.bfloat16), (0, torch.float16), (16, torch.bfloat16)])
-def test_v3cache_attend_equals_attention_over_the_cache(pkg, oracle, rw, dtype):
+@pytest.mark.parametrize("rw,dtype,D", [(128, torch.bfloat16, 128), (0, torch.float16, 128), (16, torch.bfloat16, 128),
+                                         (16, torch.bfloat16, 64), (128, torch.float16, 256), (0, torch.bfloat16, 96)])
+def test_v3cache_attend_equals_attention_over_the_cache(pkg, oracle, rw, dtype, D):
     """append() leaves the cache in the state update() leaves it in, and attend() equals one-query
     attention over (oracle-decoded packed tokens ++ window) in float64; it also agrees with attention
-    over the bf16 / fp16 tensors update() hands to the model within their rounding."""
-    B, H, G, D, L = 2, 2, 4, 128, 2
+    over the bf16 / fp16 tensors update() hands to the model within their rounding.  128-wide heads are read
+    straight from the packed codes; other head dimensions are de-quantised by the codec kernels first."""
+    B, H, G, L = 2, 2, 4, 2
     a = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=rw, n_layers=L)
     b = pkg.V3Cache(key_bits=4, value_bits=2, residual_window=rw, n_layers=L)
     steps = [300, 1, 1, 5, 1] + [1] * 20
@@ -322,7 +324,9 @@ def test_v3cache_attend_equals_attention_over_the_cache(pkg, oracle, rw, dtype):
                     q.float(), fk.float().repeat_interleave(G, dim=1), fv.float().repeat_interleave(G, dim=1)).squeeze(2)
                 err_model = float((out.squeeze(2).float() - model).norm() / model.norm())
                 print(f"[attend] rw={rw} step {i} layer {l}: vs oracle {err:.2e}, vs attention over update() tensors {err_model:.2e}")
-                assert err < 6e-3 and err_model < 2e-2           # output rounded to bf16 / fp16: 2^-9 / 2^-11
+                # output rounded to bf16 / fp16: 2^-9 / 2^-11.  (The tensors update() returns are rounded to 16 bits; with 64-wide
+                # heads the softmax scale is 1/8 and the same rounding of a key moves a weight further.)
+                assert err < 6e-3 and err_model < (2e-2 if D >= 128 else 4e-2)
         seen += n_new
     with pytest.raises(ValueError):
         b.attend(torch.zeros(B, H * G, 2, D, device=DEV), 0)

@@ -25,7 +25,7 @@ def _check_key_path(oracle, comp, x_f32, packed, label, ref_signs=None, ref_rnor
     """Packed output of TurboQuantCompressorV2.compress against the oracle on the same float32 inputs (and, when given,
     against the reference's own signs and residual norms).  Vectors in which a code moved (a coordinate within 1e-5
     of a decision boundary) have another residual and are left out of the sign comparison."""
-    D = 128
+    D = x_f32.shape[-1]
     orc = oracle.QjlOracle(comp.Pi.cpu().numpy(), comp.S.cpu().numpy(), comp.centroids.cpu().numpy())
     ref = orc.compress(x_f32)
     G = packed["idx_bytes"].shape[-1]
@@ -185,3 +185,24 @@ def test_v2_one_pass_form_against_the_two_kernel_form(pkg, oracle, bits, dtype):
         assert diff.sum() <= max(4, 5e-5 * diff.size) and (margin[diff] < 1e-5).all()
         ulp = oracle.fp16_ulp_distance(bits16(p["residual_norm"]).reshape(-1), bits16(rn).reshape(-1))
         assert ulp.max() <= 1 and (ulp > 0).mean() < 0.02
+
+
+@pytest.mark.parametrize("D,bits,dtype", [(64, 3, torch.bfloat16), (256, 4, torch.float16), (96, 2, torch.float32)])
+def test_v2_keys_at_other_head_dimensions(pkg, oracle, D, bits, dtype):
+    """Head dimensions other than 128: codes and norms from the MSE kernels, the residual part as float32 tensor
+    operations on the device.  Same checks as for 128-wide heads."""
+    n_tok = 333
+    comp = pkg.TurboQuantCompressorV2(D, bits, seed=17 * bits + D, device=DEV)
+    x = outlier_kv((2, 2, n_tok, D), seed=70 + bits, dtype=dtype)
+    packed = comp.compress(x.to(DEV))
+    assert packed["sign_bytes"].shape == (2, 2, n_tok, D // 8) and packed["idx_bytes"].shape[-1] == D // (8 // comp.mse_bits)
+    orc, ref, same = _check_key_path(oracle, comp, x.float().numpy().reshape(-1, D), packed, f"d{D} b{bits} {dtype}")
+    g = torch.Generator().manual_seed(bits)
+    q = torch.randn(2, 2, 9, D, generator=g)
+    got = comp.asymmetric_attention_scores(q.to(DEV), packed).cpu().numpy()
+    k16 = ref["k_mse_f16"].reshape(4, n_tok, D)
+    want = orc.scores(q.numpy().reshape(4, 9, D), k16, ref["signs"].reshape(4, n_tok, D), ref["residual_norm"].reshape(4, n_tok))
+    scale = np.linalg.norm(q.numpy().reshape(4, 9, 1, D), axis=-1) * np.linalg.norm(x.float().numpy().reshape(4, 1, n_tok, D), axis=-1)
+    keep = same.reshape(4, 1, n_tok).repeat(9, axis=1)
+    err = (np.abs(got.reshape(4, 9, n_tok) - want) / scale)[keep]
+    assert err.max() < 1e-3

@@ -68,6 +68,14 @@ class TurboQuantCompressorV2:
         self.S = s_host.to(dev).contiguous()
         self.centroids = cent_host.to(dev)
         self._mse = MSECompressor.from_tensors(pi_host, cent_host, self.mse_bits, device=dev)
+        self._qjl_host = None
+        self._qjl_tables = {}
+        self._s_on = {}
+        if self.head_dim != _native.HEAD_DIM:
+            # The residual kernels are built for 128-wide heads.  Other head dimensions (the multiples of 32 up to 256 that
+            # the MSE stage takes) get their codes and norms from the same kernels and the residual part (reconstruction,
+            # projection by S, signs, norm) from float32 tensor operations on the device: the reference's own arithmetic.
+            return
         L = _native.lib()
         n = L.tq_qjl_table_bytes(self.head_dim, self.mse_bits)
         if n < 0:
@@ -79,8 +87,6 @@ class TurboQuantCompressorV2:
         _native.check(L.tq_qjl_table_build(pi.ctypes.data, s.ctypes.data, c.ctypes.data, self.head_dim, self.mse_bits,
                                            blob.ctypes.data, blob.size), "tq_qjl_table_build")
         self._qjl_host = blob
-        self._qjl_tables = {}
-        self._s_on = {}
 
     def _table(self, device) -> torch.Tensor:
         """The QJL table on `device` (the compressor itself may sit on the CPU, the reference's default)."""
@@ -112,6 +118,8 @@ class TurboQuantCompressorV2:
             states = states.contiguous()
         if states.data_ptr() % 16:       # a contiguous view into the middle of a buffer: contiguous() would hand it back as it is
             states = states.clone(memory_format=torch.contiguous_format)
+        if D != _native.HEAD_DIM:
+            return self._compress_by_tensor_ops(states)
         out = self.empty_packed(B, H, S, states.device)
         n_vec = B * H * S
         if n_vec:
@@ -123,6 +131,29 @@ class TurboQuantCompressorV2:
                                                    _native._stream_handle(states.device))
             _native.check(rc, "tq_qjl_compress")
         return out
+
+    def _unpacked_codes(self, idx_bytes: torch.Tensor) -> torch.Tensor:
+        """[.., G] packed bytes -> [.., D] codes (most significant code of a byte first)."""
+        ipb = 8 // self.mse_bits
+        shifts = torch.arange(ipb - 1, -1, -1, device=idx_bytes.device, dtype=torch.uint8) * self.mse_bits
+        codes = (idx_bytes.unsqueeze(-1) >> shifts) & ((1 << self.mse_bits) - 1)
+        return codes.reshape(*idx_bytes.shape[:-1], -1)[..., :self.head_dim].long()
+
+    def _compress_by_tensor_ops(self, states: torch.Tensor) -> dict:
+        """compress for head dimensions other than 128: codes and norms from the MSE kernels, then compressors.py:107-121
+        as float32 tensor operations (reconstruction with the float32 norm, residual, its norm, projection, signs)."""
+        B, H, S, D = states.shape
+        dev = states.device
+        first = self._mse.compress(states)
+        x = states.reshape(-1, D).float()
+        norms = torch.norm(x, dim=-1, keepdim=True)
+        k_mse = (self._mse.centroids.to(dev)[self._unpacked_codes(first["idx_bytes"]).reshape(-1, D)] @ self._mse.pi(dev)) * norms
+        residual = x - k_mse
+        signs = (residual @ self._s(dev).T) >= 0
+        weights = torch.tensor([128, 64, 32, 16, 8, 4, 2, 1], device=dev, dtype=torch.int32)      # coordinate 8b + k in bit 7 - k
+        sign_bytes = (signs.reshape(-1, D // 8, 8).to(torch.int32) * weights).sum(-1).to(torch.uint8)
+        return {"idx_bytes": first["idx_bytes"], "vec_norms": first["vec_norms"], "sign_bytes": sign_bytes.reshape(B, H, S, D // 8),
+                "residual_norm": torch.norm(residual, dim=-1).to(torch.float16).reshape(B, H, S), "shape": (B, H, S, D)}
 
     def empty_packed(self, B: int, H: int, S: int, device) -> dict:
         """The packed dictionary `compress` fills, with uninitialised buffers."""
@@ -173,6 +204,11 @@ class TurboQuantCompressorV2:
         _native._require_gpu(queries, "queries")
         q = queries.float()
         dev = q.device
+        if D != _native.HEAD_DIM:       # other head dimensions: the reconstruction from the MSE kernels, the rest as tensor operations
+            exp = self.reference_format(compressed)
+            term1 = torch.matmul(q, exp["k_mse"].float().transpose(-2, -1))
+            ip = torch.matmul(torch.matmul(q, self._s(dev).T), exp["qjl_signs"].float().transpose(-2, -1))
+            return term1 + corr * ip * compressed["residual_norm"].float().unsqueeze(-2)
         q_rot = torch.matmul(q, self._mse.pi_transposed(dev)).contiguous()          # Pi q for every query token
         st = self._s_on.get(("t", dev))
         if st is None:

@@ -762,7 +762,7 @@ int check_job(const void *states, int dtype, long long rows, long long tokens, l
     if (token_stride < head_dim && tokens > 1) return TQ_ERR_SIZE;
     if (rows > 1 && row_stride < 0) return TQ_ERR_SIZE;
     if (packed_row_stride != 0 && (packed_row_stride < tokens || packed_row_stride > (long long)0x7fffffff / rows)) return TQ_ERR_SIZE;
-    if (((uintptr_t)states & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & 15u) || ((uintptr_t)vec_norms & 1u))
+    if (((uintptr_t)states & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & (tq_packed_alignment(head_dim, bits) - 1u)) || ((uintptr_t)vec_norms & 1u))
         return TQ_ERR_ALIGN;
     if (((token_stride * eb) & 15) || (rows > 1 && ((row_stride * eb) & 15))) return TQ_ERR_ALIGN;
     return TQ_OK;
@@ -790,7 +790,7 @@ extern "C" int tq_compress(const void *states, int dtype, long long rows, long l
     job.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     job.row_stride = row_stride * elem_bytes(dtype);
     job.token_stride = token_stride * elem_bytes(dtype);
-    if (head_dim == TQ_HEAD_DIM / 2 && tq_pairable(rows, tokens, token_stride, packed_row_stride, head_dim))
+    if (head_dim == TQ_HEAD_DIM / 2 && tq_pairable(rows, tokens, token_stride, packed_row_stride, head_dim, idx_bytes))
         return dispatch(dtype, bits, job, nullptr, 1, (uint32_t)((n_vec / 2 + 31) / 32), workspace, true, static_cast<hipStream_t>(stream));
     if (head_dim != TQ_HEAD_DIM)
         return tq_anydim_compress(dtype, bits, head_dim, job, nullptr, 1, (uint32_t)n_vec, static_cast<hipStream_t>(stream));
@@ -814,7 +814,7 @@ extern "C" int tq_compress_batched(const tq_job *jobs_host, const tq_job *jobs_d
                                  head_dim, j.bits, j.idx_bytes, j.vec_norms, j.packed_row_stride, &n_vec);
         if (rc) return rc;
         if (n_vec > max_vec) max_vec = n_vec;
-        if (n_vec && !tq_pairable(j.rows, j.tokens, j.token_stride, j.packed_row_stride, head_dim)) paired = false;
+        if (n_vec && !tq_pairable(j.rows, j.tokens, j.token_stride, j.packed_row_stride, head_dim, j.idx_bytes)) paired = false;
     }
     if (max_vec == 0) return TQ_OK;
     TqDevJob none{};

@@ -457,7 +457,7 @@ int check_job(const void *out, int dtype, long long rows, long long tokens, long
     if (token_stride < head_dim && tokens > 1) return TQ_ERR_SIZE;
     if (rows > 1 && row_stride < 0) return TQ_ERR_SIZE;
     if (packed_row_stride != 0 && (packed_row_stride < tokens || packed_row_stride > (long long)0x7fffffff / rows)) return TQ_ERR_SIZE;
-    if (((uintptr_t)out & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & 15u) || ((uintptr_t)vec_norms & 1u))
+    if (((uintptr_t)out & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & (tq_packed_alignment(head_dim, bits) - 1u)) || ((uintptr_t)vec_norms & 1u))
         return TQ_ERR_ALIGN;
     if (((token_stride * eb) & 15) || (rows > 1 && ((row_stride * eb) & 15))) return TQ_ERR_ALIGN;
     return TQ_OK;
@@ -485,7 +485,7 @@ extern "C" int tq_decompress(const uint8_t *idx_bytes, const uint16_t *vec_norms
     job.packed_row_stride = (uint32_t)(packed_row_stride ? packed_row_stride : tokens);
     job.row_stride = row_stride * elem_bytes(out_dtype);
     job.token_stride = token_stride * elem_bytes(out_dtype);
-    if (head_dim == TQ_HEAD_DIM / 2 && tq_pairable(rows, tokens, token_stride, packed_row_stride, head_dim))
+    if (head_dim == TQ_HEAD_DIM / 2 && tq_pairable(rows, tokens, token_stride, packed_row_stride, head_dim, idx_bytes))
         return dispatch(out_dtype, bits, job, nullptr, 1, (uint32_t)((n_vec / 2 + 31) / 32), workspace, true, static_cast<hipStream_t>(stream));
     if (head_dim != TQ_HEAD_DIM)     // the run-time-dimension kernel assigns its tiles statically: no counters
         return tq_anydim_decompress(out_dtype, bits, head_dim, job, nullptr, 1, (uint32_t)n_vec, static_cast<hipStream_t>(stream));
@@ -512,7 +512,7 @@ int check_batch(const tq_job *jobs_host, int n_jobs, int head_dim, long long *ma
                                  head_dim, j.bits, j.idx_bytes, j.vec_norms, j.packed_row_stride, &n_vec);
         if (rc) return rc;
         if (n_vec > *max_vec) *max_vec = n_vec;
-        if (n_vec && !tq_pairable(j.rows, j.tokens, j.token_stride, j.packed_row_stride, head_dim)) *paired = false;
+        if (n_vec && !tq_pairable(j.rows, j.tokens, j.token_stride, j.packed_row_stride, head_dim, j.idx_bytes)) *paired = false;
     }
     return TQ_OK;
 }

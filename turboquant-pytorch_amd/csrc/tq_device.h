@@ -335,9 +335,21 @@ __device__ __forceinline__ tq_u4 decode_rep(const uint32_t (&raw)[NW], int s, co
 // 64-wide vectors can go through the 128-wide kernels two at a time when the two vectors of every pair are neighbours in
 // memory and in the packed store, and no pair straddles two rows: an even number of tokens per row, 64 elements apart,
 // an even packed row stride.
-static inline bool tq_pairable(long long rows, long long tokens, long long token_stride, long long packed_row_stride, int head_dim) {
+static inline bool tq_pairable(long long rows, long long tokens, long long token_stride, long long packed_row_stride, int head_dim,
+                               const void *idx_bytes) {
     (void)rows;
-    return head_dim == TQ_HEAD_DIM / 2 && tokens > 0 && (tokens & 1) == 0 && token_stride == head_dim && (packed_row_stride & 1) == 0;
+    return head_dim == TQ_HEAD_DIM / 2 && tokens > 0 && (tokens & 1) == 0 && token_stride == head_dim && (packed_row_stride & 1) == 0 &&
+           ((uintptr_t)idx_bytes & 15u) == 0;      // (the 128-wide kernels move packed bytes 16 at a time)
+}
+
+// Alignment the packed codes need: 16 bytes for the 128-wide kernels; the kernels of the other head dimensions move them
+// in pieces no larger than the largest power of two that divides a vector's packed bytes (a token slice of a store of
+// 24-byte vectors starts on a multiple of 8).
+static inline uintptr_t tq_packed_alignment(int head_dim, int bits) {
+    if (head_dim == TQ_HEAD_DIM) return 16;
+    const uintptr_t g = (uintptr_t)((head_dim + (8 / bits) - 1) / (8 / bits));
+    const uintptr_t low = g & (~g + 1);
+    return low < 16 ? low : 16;
 }
 
 // Blocks per job for a (blocks_per_job x n_jobs) grid of equal-cost blocks on `cus` compute units

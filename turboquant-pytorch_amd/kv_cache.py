@@ -292,6 +292,22 @@ class V3Cache:
         scale = D ** -0.5 if scale is None else scale
         n_c, n_w = st.n_compressed, st.n_recent
         kc, vc = st.comp.key_compressor, st.comp.val_compressor
+        if D != _native.HEAD_DIM:
+            # The kernels that read packed codes directly are built for 128-wide heads.  Other head dimensions: the history
+            # is de-quantised by the codec kernels (into float32: rounding the keys to 16 bits would move logits of the size
+            # this cache sees by several per cent of a softmax weight) and attended to together with the window.
+            k = torch.empty((B, st.H, n_c + n_w, D), dtype=torch.float32, device=query_states.device)
+            v = torch.empty_like(k)
+            if n_c:
+                kc.decompress_packed(st.k_idx[:, :, :n_c], st.k_nrm[:, :, :n_c], k[:, :, :n_c])
+                vc.decompress_packed(st.v_idx[:, :, :n_c], st.v_nrm[:, :, :n_c], v[:, :, :n_c])
+            if n_w:
+                kw, vw = st.window()
+                k[:, :, n_c:] = kw
+                v[:, :, n_c:] = vw
+            q5 = query_states.reshape(B, st.H, G, D).float()
+            probs = torch.softmax(torch.matmul(q5, k.transpose(-2, -1)) * scale, dim=-1)
+            return torch.matmul(probs, v).to(query_states.dtype).reshape(B, Hq, 1, D)
         if fused is None:
             fused = G <= 16
         if fused and n_w <= 512 and not torch.compiler.is_compiling():
