@@ -44,6 +44,10 @@ WORKLOADS = {
     "llama3-8b-32k": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2, protected=4),
     "llama3-8b-32k-k4v2": dict(layers=32, batch=1, heads=8, tokens=32768, dtype="bf16", key_bits=4, value_bits=2, protected=0),
     "qwen2.5-3b-8k": dict(layers=36, batch=1, heads=2, tokens=8192, dtype="f16", key_bits=4, value_bits=2, protected=0),
+    # the same amount of data as one third of the headline cache, in heads of 64 and of 256 elements (K4/V2, bf16):
+    # 64-wide vectors go through the 128-wide kernels two at a time, 256-wide ones through kernels of their own
+    "d64-k4v2-64k": dict(layers=8, batch=1, heads=8, tokens=65536, dtype="bf16", key_bits=4, value_bits=2, protected=0, head_dim=64),
+    "d256-k4v2-16k": dict(layers=8, batch=1, heads=8, tokens=16384, dtype="bf16", key_bits=4, value_bits=2, protected=0, head_dim=256),
     # streaming decode: 64 sequences with 16384 compressed + 128 window tokens; a step is
     # one new token through V3Cache.update on all 32 layers (compress what leaves the window, de-quantise all)
     "decode-64x16k": dict(layers=32, batch=64, heads=8, tokens=16384, dtype="bf16", key_bits=4, value_bits=2,
@@ -61,14 +65,14 @@ WORKLOADS = {
 }
 
 
-def packed_bytes(bits: int) -> int:
-    return -(-128 // (8 // bits))
+def packed_bytes(bits: int, head_dim: int = 128) -> int:
+    return -(-head_dim // (8 // bits))
 
 
-def algorithmic_bytes(bits: int, elem: int, direction: str) -> int:
+def algorithmic_bytes(bits: int, elem: int, direction: str, head_dim: int = 128) -> int:
     """Bytes per vector that must cross HBM: the vector itself plus packed codes plus the fp16 norm.
     Rotation tiles and codebook tables stay in L2/LDS and are not counted."""
-    return 128 * elem + packed_bytes(bits) + 2
+    return head_dim * elem + packed_bytes(bits, head_dim) + 2
 
 
 def synth_kv(torch, shape, seed, dtype, device):
@@ -132,7 +136,7 @@ def _timed_sample(run, make_input, share, budget_s, probe_n=2048, cap=4_000_000)
     return n / (time.perf_counter() - t0), n
 
 
-def cpu_baseline(pkg, widths, budget_s=20.0):
+def cpu_baseline(pkg, widths, budget_s=20.0, head_dim=128):
     """The reference's CPU path on this machine's host cores, on a bounded sample: `widths` = {bits: share of
     vectors}.  Primary figure: the reference's op sequence issued as torch CPU operators on all cores
     (oracle.TorchCpuOracle: fp32 cast, norm, divide, sgemm, [n,D,L] broadcast / abs / argmin, int64 pack; unpack,
@@ -145,10 +149,10 @@ def cpu_baseline(pkg, widths, budget_s=20.0):
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     rng = np.random.default_rng(0)
-    make = lambda n: rng.standard_normal((n, 128), dtype=np.float32)
+    make = lambda n: rng.standard_normal((n, head_dim), dtype=np.float32)
     seq, port, seq_desc, port_desc = {}, {}, [], []
     for bits, share in sorted(widths.items()):
-        comp = pkg.MSECompressor(128, bits, seed=42, device="cpu")
+        comp = pkg.MSECompressor(head_dim, bits, seed=42, device="cpu")
         pi, cent = comp.Pi.numpy(), comp.centroids.numpy()
         tor = O.TorchCpuOracle(pi, cent, bits)
 
@@ -375,6 +379,8 @@ def main():
     if w.get("v2"):
         return run_v2(args, torch, pkg, w, dev)
     L, B, H, S = w["layers"], w["batch"], w["heads"], w["tokens"]
+    D = w.get("head_dim", 128)
+    rotation_flop = 2 * D * D                 # the rotation is a D x D contraction
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16}[w["dtype"]]
     n_vec = B * H * S
 
@@ -382,17 +388,17 @@ def main():
     groups = {}   # bits -> list of job dicts
     layers = []
     for l in range(L):
-        tq = pkg.TurboQuantV3(128, key_bits=w["key_bits"], value_bits=w["value_bits"], residual_window=0,
+        tq = pkg.TurboQuantV3(D, key_bits=w["key_bits"], value_bits=w["value_bits"], residual_window=0,
                               layer_idx=l, n_layers=L, protected_layers=w["protected"], device=str(dev))
         layers.append(tq)
         for which, comp in (("k", tq.key_compressor), ("v", tq.val_compressor)):
-            x = synth_kv(torch, (B, H, S, 128), seed=4_000_000 + 10 * l + (0 if which == "k" else 1), dtype=dtype, device=dev)
+            x = synth_kv(torch, (B, H, S, D), seed=4_000_000 + 10 * l + (0 if which == "k" else 1), dtype=dtype, device=dev)
             job = {
                 "states": x,
-                "idx_bytes": torch.empty((B, H, S, packed_bytes(comp.bits)), dtype=torch.uint8, device=dev),
+                "idx_bytes": torch.empty((B, H, S, packed_bytes(comp.bits, D)), dtype=torch.uint8, device=dev),
                 "vec_norms": torch.empty((B, H, S), dtype=torch.float16, device=dev),
                 "table": comp.table(), "bits": comp.bits,
-                "out": torch.empty((B, H, S, 128), dtype=dtype, device=dev),
+                "out": torch.empty((B, H, S, D), dtype=dtype, device=dev),
             }
             groups.setdefault(comp.bits, []).append(job)
     comp_lists = {b: native.JobList(jobs, dev) for b, jobs in groups.items()}
@@ -488,11 +494,11 @@ def main():
     step_bytes = 0
     for (direction, b), table_avg in table_ms.items():
         jobs = len(groups[b])
-        bytes_per_launch = jobs * n_vec * algorithmic_bytes(b, elem, direction)
+        bytes_per_launch = jobs * n_vec * algorithmic_bytes(b, elem, direction, D)
         live = (direction, b) == dominant_launch
         avg_ms = live_ms if live else table_avg          # the dominant launch: measured inside the timed region
         step_bytes += bytes_per_launch
-        flop = jobs * n_vec * ROTATION_FLOP * MFMA_PASSES[direction]
+        flop = jobs * n_vec * rotation_flop * MFMA_PASSES[direction]
         kernels[f"{direction}_b{b}"] = {
             "launches_per_step": 1, "jobs": jobs, "vectors_per_launch": jobs * n_vec,
             "algorithmic_bytes_per_launch": bytes_per_launch, "avg_ms": avg_ms,
@@ -520,9 +526,21 @@ def main():
         """the rotation's matrix-core rate in the slowest launch of one direction"""
         name = max((k for k in kernels if k.startswith(direction)), key=lambda k: kernels[k]["avg_ms"])
         k = kernels[name]
-        return {"kernel": name, "flop_per_vector": ROTATION_FLOP * MFMA_PASSES[direction],
+        return {"kernel": name, "flop_per_vector": rotation_flop * MFMA_PASSES[direction],
                 "flop_per_launch": k["mfma_flop_per_launch"], "achieved": k["mfma_PFLOPs"], "peak": MFMA_PEAK_PFLOPS,
                 "unit": "PFLOP/s", "frac": k["frac_of_mfma_peak"]}
+
+    # The bound is the one the dominant launch is nearer to.  At 128 elements a vector it is the memory system (about 6
+    # matrix flop per byte); at 256 the rotation does four times the flop per vector on twice the bytes and the
+    # two-pass split-precision product makes compress matrix-bound.
+    if dk["frac_of_mfma_peak"] > dk["frac_of_hbm_peak"]:
+        roofline = {"bound": "mfma", "kernel": dominant, "achieved": dk["mfma_PFLOPs"] * 1e3, "peak": MFMA_PEAK_PFLOPS * 1e3,
+                    "unit": "TFLOP/s", "frac": dk["frac_of_mfma_peak"], "traffic": traffic, "traffic_source": traffic_source,
+                    "hbm": {"achieved": dk["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dk["frac_of_hbm_peak"]}}
+    else:
+        roofline = {"bound": "hbm", "kernel": dominant, "achieved": dk["achieved_GBps"], "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": dk["frac_of_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source}
+    roofline["mfma"] = {"compress": mfma_of("compress"), "decompress": mfma_of("decompress")}
 
     widths = {}
     for b, jobs in groups.items():
@@ -537,7 +555,7 @@ def main():
         "dtype": w["dtype"], "data": "synthetic",
         "untimed_steps_after_warmup": 3 + conditioning_steps + table_steps,
         "warmup_total": args.warmup + 3 + conditioning_steps + table_steps,      # every untimed step before the timed region
-        "config": {"workload": args.workload, "layers": L, "batch": B, "kv_heads": H, "tokens": S, "head_dim": 128,
+        "config": {"workload": args.workload, "layers": L, "batch": B, "kv_heads": H, "tokens": S, "head_dim": D,
                    "key_bits": w["key_bits"], "value_bits": w["value_bits"], "protected_layers": w["protected"],
                    "residual_window": 0, "width_groups": {str(b): len(groups[b]) for b in order},
                    "vectors_per_step": total_vec},
@@ -545,9 +563,7 @@ def main():
         "step_algorithmic_GB": step_bytes / 1e9,
         "step_GBps": step_bytes / (wall / args.steps) / 1e9,
         "step_frac_of_hbm_peak": step_bytes / (wall / args.steps) / 1e9 / HBM_PEAK_GBS,
-        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dk["achieved_GBps"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": dk["frac_of_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source,
-                     "mfma": {"compress": mfma_of("compress"), "decompress": mfma_of("decompress")}},
+        "roofline": roofline,
         "kernels": kernels,
         "round_trip_rel_error": rel,
     }
@@ -559,7 +575,7 @@ def main():
         result["roofline"]["stream_GBps"] = stream_rates(torch, dev)
         result["roofline"]["step_frac_of_copy_rate"] = result["step_GBps"] / result["roofline"]["stream_GBps"]["copy"]
     if not args.no_cpu_baseline and not args.skeleton:
-        result["cpu_baseline"] = cpu_baseline(pkg, widths, args.cpu_seconds)
+        result["cpu_baseline"] = cpu_baseline(pkg, widths, args.cpu_seconds, head_dim=D)
     print(json.dumps(result))
 
 
