@@ -39,7 +39,8 @@ struct TermPair { uint32_t hi, lo; };
 __device__ __forceinline__ TermPair split_pair(float x0, float x1) {
     typedef __fp16 pk_half2 __attribute__((ext_vector_type(2)));
     const pk_half2 h = __builtin_amdgcn_cvt_pkrtz(x0, x1);
-    const pk_half2 l = __builtin_amdgcn_cvt_pkrtz(x0 - (float)h[0], x1 - (float)h[1]);
+    // x - hi written as a fused multiply-add with the 16-bit operand widened inside the instruction (same value: one rounding)
+    const pk_half2 l = __builtin_amdgcn_cvt_pkrtz(__builtin_fmaf((float)h[0], -1.0f, x0), __builtin_fmaf((float)h[1], -1.0f, x1));
     return {__builtin_bit_cast(uint32_t, h), __builtin_bit_cast(uint32_t, l)};
 }
 
@@ -324,7 +325,6 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_fused_kernel(TqQjlDevJob j
     constexpr int VEC_BYTES = TQ_HEAD_DIM * 2;
     constexpr int STAGE = 32 * VEC_BYTES;       // one tile of 16-bit values: 8 KiB
     constexpr int NLOAD = 2;                    // direct-to-LDS loads per wave and tile
-    constexpr int SLOTS = 2;
 
     // LDS (dynamic: more than the 64 KiB a kernel may declare statically): input ring | residual terms | grid | tables | shares
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds_all[];
@@ -434,7 +434,13 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_fused_kernel(TqQjlDevJob j
     auto iteration = [&](auto rot_tag, auto search_tag, auto project_tag, auto par_tag, uint32_t j, tq_f16v &acc_new, const tq_f16v &acc_old) {
         constexpr bool ROT = decltype(rot_tag)::value, SEARCH = decltype(search_tag)::value, PROJECT = decltype(project_tag)::value;
         constexpr uint32_t PAR = decltype(par_tag)::value;
-        wait_vmcnt<0>();        // this wave's loads of tile j (issued an iteration ago) and its stores
+        // this wave's loads of tile j, issued at the start of the iteration before.  Younger than them are only that
+        // iteration's stores (codes and norm of a searched tile, the signs of a projected one; the residual norm, which
+        // wave 0 alone stores, comes last): two of them in iteration 1, three from then on, and they may stay in flight
+        // (which measures the same as waiting for them: the kernel is bound by its matrix and vector instructions).
+        // A third ring slot, which would let the loads run two iterations ahead, costs the second block of a compute
+        // unit its LDS and a third of the rate.
+        if (j >= 3u) wait_vmcnt<3>(); else if (j == 2u) wait_vmcnt<2>(); else wait_vmcnt<0>();
         __syncthreads();
         if constexpr (ROT) issue(PAR ^ 1u, tile_of(j + 1u));
         const uint8_t *stage = lds_stage[PAR];
@@ -544,9 +550,13 @@ __global__ __launch_bounds__(QTHREADS, 2) void tq_qjl_fused_kernel(TqQjlDevJob j
         }
         if constexpr (PROJECT) {
             const uint32_t tl = tile_of(j - 2u);
-            uint32_t word = 0;             // byte 0: coordinates 0..7 of the lane, most significant bit first; byte 1: 8..15
+            // byte 0: coordinates 0..7 of the lane, most significant bit first; byte 1: 8..15.  The sign bits are shifted
+            // in one instruction each (8..15 first, so that they end up in the upper byte) and inverted at the end: a
+            // sum that starts from +0 is never -0, so "sign bit clear" is ">= 0".
+            uint32_t neg = 0;
 #pragma unroll
-            for (int k = 0; k < 16; ++k) word |= (prj[k] >= 0.f ? 1u : 0u) << (8 * (k / 8) + 7 - (k % 8));
+            for (int k = 0; k < 16; ++k) neg = __builtin_amdgcn_alignbit(neg, __float_as_uint(prj[(k + 8) & 15]), 31);
+            const uint32_t word = ~neg;
             const size_t v = (size_t)tl * 32u + n;
             tq_gstore2(reinterpret_cast<uint16_t *>(job.sign_bytes + v * 16u + 4u * wave + 2u * hk), (uint16_t)word);
             if (wave == 0) {
