@@ -105,11 +105,15 @@ int tq_table_quantize_host(const void *table_host, const float *r, long long n, 
  *               and its head_dim elements are contiguous.  A contiguous
  *               [B,H,S,D] tensor is rows=1, tokens=B*H*S, token_stride=D; a slice
  *               [:, :, :s, :] of one is rows=B*H, tokens=s, row_stride=S*D.
- *               Base address and strides must keep every vector 16-byte aligned.
+ *               Base address and strides must keep every vector 16-byte aligned (head dimensions that are
+ *               not a multiple of 32: aligned to the element size).
  *   head_dim    128 runs the tuned kernels; tq_compress, tq_decompress and their batched forms also take
- *               every other multiple of 32 from 32 to 256 (compressors_v3.py:37-43 accepts any head_dim),
- *               through one pair of kernels that reads the dimension at run time.  Everything else in this
- *               header (scores, weighted values, attention, token append, QJL signs) is 128 only.
+ *               every other head dimension from 8 to 256 (compressors_v3.py:37-43 accepts any head_dim):
+ *               64 and 256 through kernels of their own, the rest through one pair of kernels that reads the
+ *               dimension at run time and works on a dimension that is not a multiple of 32 as the next
+ *               multiple (zero elements in, zero codes up to a whole byte out: compressors_v3.py:64-68).
+ *               Everything else in this header (scores, weighted values, attention, token append, QJL signs)
+ *               is 128 only.
  *   table_dev   device copy of the blob from tq_table_build
  *   idx_bytes   device, uint8, bytes_per_vector per packed slot
  *   vec_norms   device, one IEEE fp16 bit pattern per packed slot (norm of the fp32-widened vector)

@@ -32,7 +32,7 @@ def oracle():
 def golden():
     """Outputs of the upstream reference on seeded inputs (written by tests/golden/make_fixtures.py)."""
     out = {name: np.load(os.path.join(GOLDEN, name + ".npz")) for name in
-           ("codebooks", "rotations", "mse_roundtrip", "config1", "v3")}
+           ("codebooks", "rotations", "mse_roundtrip", "config1", "v3", "odd_dims")}
     with open(os.path.join(GOLDEN, "fixtures.json")) as f:
         out["json"] = json.load(f)
     return out

@@ -18,7 +18,7 @@ static float rnd() {
 
 int main() {
     if (tq_abi_version() <= 0 || !tq_status_string(0) || !tq_status_string(-3) || !tq_status_string(-99)) return 1;
-    const int dims[] = {32, 64, 96, 128, 160, 256};
+    const int dims[] = {8, 32, 45, 64, 80, 96, 100, 128, 160, 255, 256};
     for (int D : dims) {
         std::vector<float> Pi((size_t)D * D), S((size_t)D * D);
         for (auto &v : Pi) v = rnd() / std::sqrt((float)D);
@@ -58,7 +58,7 @@ int main() {
             }
         }
     }
-    if (tq_table_bytes(80, 4) >= 0 || tq_table_bytes(128, 9) >= 0 || tq_qjl_table_bytes(64, 3) >= 0) return 1;
+    if (tq_table_bytes(7, 4) >= 0 || tq_table_bytes(257, 4) >= 0 || tq_table_bytes(128, 9) >= 0 || tq_qjl_table_bytes(64, 3) >= 0) return 1;
     std::puts("ok");
     return 0;
 }

@@ -1,5 +1,6 @@
-"""GPU parity for head dimensions other than 128 (compress / decompress take every multiple of 32 up to 256;
-upstream turboquant/compressors_v3.py:37-43 builds rotation and codebook for any head_dim).  Same bars as the
+"""GPU parity for head dimensions other than 128 (compress / decompress take every head dimension from 8 to 256;
+upstream turboquant/compressors_v3.py:37-43 builds rotation and codebook for any head_dim, :64-68 pads the codes of a
+vector to a whole byte).  Same bars as the
 128-wide tests: codes bit-exact outside a 1e-5 window around a decision boundary, fp16 norms within one ulp,
 reconstruction within 1e-3 relative L2 of the oracle's.
 """
@@ -29,13 +30,14 @@ def _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, label, max_f
     dn = {torch.float32: "f32", torch.float16: "f16", torch.bfloat16: "bf16"}[x.dtype]
     D = x.shape[-1]
     out = comp.compress(x.to(DEV))
-    assert out["idx_bytes"].shape[-1] == D // (8 // bits) and out["idx_pad"] == 0
+    ipb = 8 // bits
+    assert out["idx_bytes"].shape[-1] == -(-D // ipb) and out["idx_pad"] == (ipb - D % ipb) % ipb
     ref, _ = check_codes(oracle, out["idx_bytes"].cpu().numpy(), x.float().numpy().reshape(-1, D), Pi, cent, bits, label, max_frac)
     check_norms(oracle, bits16(out["vec_norms"]), ref["vec_norms"], label)
     # de-quantise the ORACLE's packed form, so that a code on the other side of a boundary does not enter
     packed = {"idx_bytes": torch.from_numpy(ref["idx_bytes"].reshape(out["idx_bytes"].shape)).to(DEV),
               "vec_norms": torch.from_numpy(ref["vec_norms"].view(np.int16).reshape(out["vec_norms"].shape)).view(torch.float16).to(DEV),
-              "shape": tuple(x.shape), "idx_pad": 0}
+              "shape": tuple(x.shape), "idx_pad": out["idx_pad"]}
     want = oracle.NumpyOracle(Pi, cent, bits).decompress(ref["idx_bytes"], ref["vec_norms"])
     rec = comp.decompress(packed)
     assert rec.dtype == torch.float32 and rec.shape == x.shape
@@ -80,6 +82,85 @@ def test_other_dimensions_and_widths(pkg, oracle, D, bits):
     for dn, shape in (("f32", (1, 2, 211, D)), ("bf16", (3, 1, 129, D)), ("f16", (1, 1, 31, D))):
         x = outlier_kv(shape, seed=D + bits, dtype=TORCH_DT[dn])
         _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, f"d{D} b{bits} {dn}", max_frac=2.5e-4 if bits > 4 else None)
+
+
+ODD_DIM_CASES = ((45, 2), (45, 3), (45, 4), (80, 2), (80, 4), (100, 1), (100, 3), (112, 4), (200, 2))
+
+
+@pytest.mark.parametrize("D,bits", ODD_DIM_CASES)
+def test_reference_fixtures_at_head_dimensions_that_are_not_multiples_of_32(pkg, oracle, golden, D, bits):
+    """The reference's own outputs at head dimensions 45, 80, 100, 112 and 200 (tests/golden/odd_dims.npz), among them
+    ones whose codes do not fill the last byte of a vector: the reference's bytes except on a decision boundary (the
+    padding bits among them: zero), its norms to one fp16 step, its reconstruction from its own packed form."""
+    fx = golden["odd_dims"]
+    Pi, cent = fx[f"Pi_d{D}_b{bits}"], fx[f"centroids_d{D}_b{bits}"]
+    comp = pkg.MSECompressor.from_tensors(torch.from_numpy(Pi), torch.from_numpy(cent), bits, device=DEV)
+    ipb = 8 // bits
+    for dn in ("f32", "f16", "bf16"):
+        key = f"d{D}_b{bits}_{dn}"
+        raw = fx[key + "_x"]
+        x = torch.from_numpy(raw) if dn == "f32" else torch.from_numpy(raw.view(np.int16)).view(TORCH_DT[dn])
+        out = comp.compress(x.to(DEV))
+        ref_bytes = fx[key + "_idx_bytes"]
+        assert tuple(out["idx_bytes"].shape) == ref_bytes.shape and out["idx_pad"] == int(fx[key + "_idx_pad"][0])
+        got = out["idx_bytes"].cpu().numpy().reshape(-1, ref_bytes.shape[-1])
+        ref2 = ref_bytes.reshape(got.shape)
+        if not np.array_equal(got, ref2):
+            rot = oracle.NumpyOracle(Pi, cent, bits).rotate(oracle.widen(raw, dn))[1]
+            rep = oracle.code_mismatch_report(got, ref2, rot, cent, bits)
+            assert rep["outside_window"] == 0 and rep["differ"] <= 3, (key, rep)
+        pad = out["idx_pad"]
+        if pad:      # the bits of the codes a vector does not have
+            assert not (got[:, -1] & ((1 << (bits * pad)) - 1)).any(), key
+        check_norms(oracle, bits16(out["vec_norms"]), fx[key + "_vec_norms"], key)
+        packed = {"idx_bytes": torch.from_numpy(ref_bytes).to(DEV),
+                  "vec_norms": torch.from_numpy(fx[key + "_vec_norms"].view(np.int16)).view(torch.float16).to(DEV),
+                  "shape": tuple(x.shape), "idx_pad": pad}
+        rec = comp.decompress(packed).cpu().numpy()
+        want = fx[key + "_recon"]
+        err, fin = rel_l2(rec, want)
+        assert err <= REL_L2, (key, err)
+        assert np.array_equal(np.isfinite(rec).all(-1).reshape(-1), np.isfinite(want).all(-1).reshape(-1)), key
+        assert not rec.reshape(-1, D)[0].any()       # the zero vector comes back as zeros
+
+
+@pytest.mark.parametrize("D,bits", [(8, 4), (17, 2), (40, 8), (72, 5), (120, 3), (136, 4), (250, 1), (255, 2)])
+def test_any_head_dimension_from_8_to_256(pkg, oracle, D, bits):
+    """Dimensions on both sides of every multiple of 32, every packing, against the oracle; also as token-axis slices
+    of a preallocated store (vectors and packed rows at addresses with no particular alignment) and as a job list."""
+    Pi_t = _orthogonal(D, seed=3 * D + bits)
+    cent_t = pkg.LloydMaxCodebook(D, bits).centroids
+    comp = pkg.MSECompressor.from_tensors(Pi_t, cent_t, bits, device=DEV)
+    Pi, cent = Pi_t.numpy(), cent_t.numpy()
+    for dn, shape in (("f32", (1, 2, 77, D)), ("bf16", (2, 1, 129, D)), ("f16", (1, 1, 33, D))):
+        x = outlier_kv(shape, seed=D + bits, dtype=TORCH_DT[dn])
+        _roundtrip_against_oracle(pkg, oracle, comp, Pi, cent, bits, x, f"d{D} b{bits} {dn}", max_frac=2.5e-4 if bits > 4 else None)
+    # a store with room for 50 tokens per row, filled from token 3 on
+    B, H, S, cap = 2, 2, 21, 50
+    G = -(-D // (8 // bits))
+    x = outlier_kv((B, H, S, D), seed=9, dtype=torch.bfloat16).to(DEV)
+    plain = comp.compress(x)
+    idx = torch.zeros((B, H, cap, G), dtype=torch.uint8, device=DEV)
+    nrm = torch.zeros((B, H, cap), dtype=torch.float16, device=DEV)
+    comp.compress_into(x, idx[:, :, 3:3 + S], nrm[:, :, 3:3 + S])
+    assert torch.equal(idx[:, :, 3:3 + S], plain["idx_bytes"]) and torch.equal(nrm[:, :, 3:3 + S], plain["vec_norms"])
+    assert not idx[:, :, :3].any() and not idx[:, :, 3 + S:].any()
+    big = torch.full((B, H, cap, D), 7.0, dtype=torch.bfloat16, device=DEV)
+    comp.decompress_into({"idx_bytes": idx[:, :, 3:3 + S], "vec_norms": nrm[:, :, 3:3 + S], "shape": (B, H, S, D), "idx_pad": plain["idx_pad"]},
+                         big[:, :, 5:5 + S])
+    direct = torch.empty((B, H, S, D), dtype=torch.bfloat16, device=DEV)
+    comp.decompress_into(plain, direct)
+    assert torch.equal(big[:, :, 5:5 + S], direct)
+    assert (big[:, :, :5] == 7.0).all() and (big[:, :, 5 + S:] == 7.0).all()       # nothing written past a vector's end
+    # several tensors in one launch
+    native = pkg._native
+    xs = [outlier_kv((1, 2, 40 + 3 * i, D), seed=20 + i, dtype=torch.float16).to(DEV) for i in range(3)]
+    jobs = [{"states": t, "idx_bytes": torch.zeros((1, 2, t.shape[2], G), dtype=torch.uint8, device=DEV),
+             "vec_norms": torch.zeros((1, 2, t.shape[2]), dtype=torch.float16, device=DEV), "table": comp.table(DEV), "bits": bits} for t in xs]
+    native.JobList(jobs, torch.device(DEV)).compress()
+    for t, j in zip(xs, jobs):
+        one = comp.compress(t)
+        assert torch.equal(j["idx_bytes"], one["idx_bytes"]) and torch.equal(j["vec_norms"], one["vec_norms"])
 
 
 def test_edge_inputs(pkg, oracle):

@@ -276,7 +276,8 @@ def test_packed_weighted_values_against_oracle(pkg, oracle, bits, group, S):
 
 
 @pytest.mark.parametrize("rw,dtype,D", [(128, torch.bfloat16, 128), (0, torch.float16, 128), (16, torch.bfloat16, 128),
-                                         (16, torch.bfloat16, 64), (128, torch.float16, 256), (0, torch.bfloat16, 96)])
+                                         (16, torch.bfloat16, 64), (128, torch.float16, 256), (0, torch.bfloat16, 96),
+                                         (16, torch.float16, 80), (8, torch.bfloat16, 45)])
 def test_v3cache_attend_equals_attention_over_the_cache(pkg, oracle, rw, dtype, D):
     """append() leaves the cache in the state update() leaves it in, and attend() equals one-query
     attention over (oracle-decoded packed tokens ++ window) in float64; it also agrees with attention

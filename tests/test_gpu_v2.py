@@ -36,8 +36,10 @@ def _check_key_path(oracle, comp, x_f32, packed, label, ref_signs=None, ref_rnor
     ulp = oracle.fp16_ulp_distance(bits16(packed["vec_norms"]).reshape(-1), ref["norms_f32"].astype(np.float16).view(np.uint16))
     assert ulp.max() <= 1, label
     want_signs = ref["signs"] if ref_signs is None else ref_signs
-    got_bytes = packed["sign_bytes"].cpu().numpy().reshape(-1, D // 8)
-    got_signs = np.unpackbits(got_bytes, axis=-1, bitorder="big").astype(np.int8) * 2 - 1
+    got_bytes = packed["sign_bytes"].cpu().numpy().reshape(-1, -(-D // 8))
+    if D % 8:       # the bits a vector does not fill stay clear
+        assert not (got_bytes[:, -1] & ((1 << (8 - D % 8)) - 1)).any(), label
+    got_signs = np.unpackbits(got_bytes, axis=-1, bitorder="big")[:, :D].astype(np.int8) * 2 - 1
     diff = (got_signs != want_signs) & same[:, None]
     srow = np.linalg.norm(orc.S, axis=1)
     margin = np.abs(ref["projected"]) / (srow[None, :] * np.maximum(ref["residual_norm_f32"][:, None], 1e-30))
@@ -187,7 +189,8 @@ def test_v2_one_pass_form_against_the_two_kernel_form(pkg, oracle, bits, dtype):
         assert ulp.max() <= 1 and (ulp > 0).mean() < 0.02
 
 
-@pytest.mark.parametrize("D,bits,dtype", [(64, 3, torch.bfloat16), (256, 4, torch.float16), (96, 2, torch.float32)])
+@pytest.mark.parametrize("D,bits,dtype", [(64, 3, torch.bfloat16), (256, 4, torch.float16), (96, 2, torch.float32),
+                                          (80, 3, torch.float16), (45, 3, torch.bfloat16)])
 def test_v2_keys_at_other_head_dimensions(pkg, oracle, D, bits, dtype):
     """Head dimensions other than 128: codes and norms from the MSE kernels, the residual part as float32 tensor
     operations on the device.  Same checks as for 128-wide heads."""
@@ -195,7 +198,7 @@ def test_v2_keys_at_other_head_dimensions(pkg, oracle, D, bits, dtype):
     comp = pkg.TurboQuantCompressorV2(D, bits, seed=17 * bits + D, device=DEV)
     x = outlier_kv((2, 2, n_tok, D), seed=70 + bits, dtype=dtype)
     packed = comp.compress(x.to(DEV))
-    assert packed["sign_bytes"].shape == (2, 2, n_tok, D // 8) and packed["idx_bytes"].shape[-1] == D // (8 // comp.mse_bits)
+    assert packed["sign_bytes"].shape == (2, 2, n_tok, -(-D // 8)) and packed["idx_bytes"].shape[-1] == -(-D // (8 // comp.mse_bits))
     orc, ref, same = _check_key_path(oracle, comp, x.float().numpy().reshape(-1, D), packed, f"d{D} b{bits} {dtype}")
     g = torch.Generator().manual_seed(bits)
     q = torch.randn(2, 2, 9, D, generator=g)

@@ -305,9 +305,10 @@ def test_c_abi_argument_errors(pkg):
     assert lib.tq_bytes_per_vector(128, 6) == 128 and lib.tq_bytes_per_vector(128, 1) == 16
     assert lib.tq_bytes_per_vector(6, 2) == 2
     assert lib.tq_bytes_per_vector(128, 0) == E["BITS"] and lib.tq_bytes_per_vector(128, 9) == E["BITS"]
-    # compress / decompress take every multiple of 32 up to 256
-    assert lib.tq_table_bytes(80, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(288, 4) == E["HEAD_DIM"]
+    # compress / decompress take every head dimension from 8 to 256; one that is not a multiple of 32 has the table of the next multiple
+    assert lib.tq_table_bytes(7, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(257, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(288, 4) == E["HEAD_DIM"]
     assert lib.tq_table_bytes(0, 4) == E["HEAD_DIM"] and lib.tq_table_bytes(128, 9) == E["BITS"]
+    assert lib.tq_table_bytes(80, 4) == lib.tq_table_bytes(96, 4) == lib.tq_table_bytes(65, 4) and lib.tq_table_bytes(8, 2) == lib.tq_table_bytes(32, 2)
     assert 0 < lib.tq_table_bytes(32, 4) < lib.tq_table_bytes(128, 4) < lib.tq_table_bytes(256, 4)
     assert lib.tq_table_bytes(64, 4) > lib.tq_table_bytes(96, 4)      # 64: also the operands of diag(Pi, Pi) for the 128-wide kernels
     cent = np.array([0.1, -0.1], np.float32)
@@ -331,7 +332,9 @@ def test_c_abi_argument_errors(pkg):
         states, dtype, kw.get("rows", 1), kw.get("tokens", 4), kw.get("rs", 0), kw.get("ts", 128), table, hd, bits,
         idx, norms, kw.get("prs", 0), kw.get("ws", None), None)
     assert call(p, 1, 0, 128) == E["BITS"]
-    assert call(p, 1, 4, 80) == E["HEAD_DIM"]
+    assert call(p, 1, 4, 300) == E["HEAD_DIM"] and call(p, 1, 4, 4) == E["HEAD_DIM"]
+    assert call(p, 1, 4, 80, ts=64) == E["SIZE"]
+    assert call(p + 1, 1, 4, 80, ts=80) == E["ALIGN"]      # fp16 vectors of 80 elements may start on any even address, not on an odd one
     assert call(p, 1, 4, 64, ts=48) == E["SIZE"]
     assert call(p, 7, 4, 128) == E["DTYPE"]
     assert call(None, 1, 4, 128) == E["NULL"]
@@ -462,13 +465,32 @@ def test_tables_for_other_head_dimensions(pkg):
                    [("grid_scale", ctypes.c_float), ("grid_bias", ctypes.c_float)] + \
                    [(n, ctypes.c_uint32) for n in ("total_bytes", "off_a_f16", "off_a_bf16", "off_grid", "off_at_f16", "off_lut")]
 
-    for D, bits in ((64, 4), (256, 8), (96, 3)):
+    for D, bits in ((64, 4), (256, 8), (96, 3), (80, 4), (45, 2)):
         g = torch.Generator().manual_seed(D)
         Pi, _ = torch.linalg.qr(torch.randn(D, D, generator=g))
         cent = pkg.LloydMaxCodebook(D, bits).centroids
         blob = native.build_table(Pi, cent, bits)
         hd = Header.from_buffer_copy(blob[:ctypes.sizeof(Header)].tobytes())
+        logical, D = D, -(-D // 32) * 32          # the operand sets are those of the rotation extended by zeros to a multiple of 32
         operand = (D // 32) * (D // 16) * 1024
+        if logical != D:
+            assert (hd.head_dim, hd.bits, hd.total_bytes) == (logical, bits, blob.size) and hd.bytes_per_vec == -(-logical // (8 // bits))
+            a = blob[hd.off_a_bf16:hd.off_a_bf16 + operand].view(np.uint16).reshape(D // 32, D // 16, 64, 8)
+            pi = np.zeros((D, D), np.float32)
+            pi[:logical, :logical] = Pi.numpy()
+            for (t, s, l, i) in ((0, 0, 0, 0), (D // 32 - 1, D // 16 - 1, 63, 7), (1, 2, 37, 3), (D // 32 - 1, 0, 5, 1), (0, D // 16 - 1, 33, 6)):
+                m, hk = l % 32, l // 32
+                row = 32 * t + 16 * ((m // 4) % 2) + 4 * (m // 8) + m % 4
+                want = torch.tensor(pi[row, 16 * s + 8 * hk + i]).to(torch.bfloat16).view(torch.int16).item() & 0xffff
+                assert a[t, s, l, i] == want, (logical, t, s, l, i)
+            at = blob[hd.off_at_f16:hd.off_at_f16 + operand].view(np.float16).reshape(D // 32, D // 16, 64, 8)
+            for (t, s, l, i) in ((1, 1, 40, 5), (D // 32 - 1, D // 16 - 1, 63, 7)):
+                m, hk = l % 32, l // 32
+                col = 32 * t + 16 * ((m // 4) % 2) + 4 * (m // 8) + m % 4
+                assert at[t, s, l, i] == np.float16(pi[16 * s + 8 * hk + i, col])
+            assert native.lib().tq_table_check(blob.ctypes.data, blob.size, logical, bits) == 0
+            assert native.lib().tq_table_check(blob.ctypes.data, blob.size, D, bits) != 0
+            continue
         assert (hd.head_dim, hd.bits, hd.total_bytes) == (D, bits, blob.size)
         assert hd.off_a_bf16 - hd.off_a_f16 == 2 * operand and hd.off_at_f16 - hd.off_a_bf16 == 3 * operand
         assert hd.bytes_per_vec == D // (8 // bits) and hd.grid_cells * 8 <= 18432
@@ -506,7 +528,7 @@ def test_device_default_is_the_references(pkg):
 
 def test_host_side_of_the_abi_under_sanitizers(tmp_path):
     """csrc/tq_host.cpp (table builders, thresholds, host quantiser) compiled with AddressSanitizer and
-    UndefinedBehaviorSanitizer and driven by tests/native/host_sanitize.cpp over head dimensions 32 ... 256 and every
+    UndefinedBehaviorSanitizer and driven by tests/native/host_sanitize.cpp over head dimensions 8 ... 256 (multiples of 32 and others) and every
     width, with table buffers of exactly the size tq_table_bytes reports; the driver also checks the host quantiser
     against the nearest-centroid definition."""
     import shutil

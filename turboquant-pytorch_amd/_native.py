@@ -299,6 +299,12 @@ def dtype_code(dt: torch.dtype) -> int:
         raise TqError(f"unsupported element type {dt}; float32, float16 and bfloat16 are supported") from None
 
 
+def _vector_alignment(head_dim: int, elem_bytes: int) -> int:
+    """Bytes the vectors' address and strides must be a multiple of: 16, except for head dimensions that are not a
+    multiple of 32, which the kernels move element by element."""
+    return elem_bytes if head_dim % 32 else 16
+
+
 def vector_layout(t: torch.Tensor) -> Optional[Tuple[int, int, int, int]]:
     """(rows, tokens, row_stride, token_stride) in elements for a [B,H,S,D] tensor whose last
     dimension is dense, or None if its strides do not reduce to the two-level form."""
@@ -307,7 +313,8 @@ def vector_layout(t: torch.Tensor) -> Optional[Tuple[int, int, int, int]]:
     if D != 1 and sd != 1:
         return None
     esz = t.element_size()
-    if (t.data_ptr() % 16) or any((s * esz) % 16 for s in (sb, sh, ss)):
+    align = _vector_alignment(D, esz)
+    if (t.data_ptr() % align) or any((s * esz) % align for s in (sb, sh, ss)):
         return None
     n = B * H * S
     if n == 0:
@@ -338,7 +345,8 @@ def row_layout(t: torch.Tensor) -> Optional[Tuple[int, int, int, int]]:
     if D != 1 and sd != 1:
         return None
     esz = t.element_size()
-    if (t.data_ptr() % 16) or any((st * esz) % 16 for st in (sb, sh, ss)):
+    align = _vector_alignment(D, esz)
+    if (t.data_ptr() % align) or any((st * esz) % align for st in (sb, sh, ss)):
         return None
     if B != 1 and H != 1 and sb != H * sh:
         return None

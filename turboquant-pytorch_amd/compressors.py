@@ -72,7 +72,7 @@ class TurboQuantCompressorV2:
         self._qjl_tables = {}
         self._s_on = {}
         if self.head_dim != _native.HEAD_DIM:
-            # The residual kernels are built for 128-wide heads.  Other head dimensions (the multiples of 32 up to 256 that
+            # The residual kernels are built for 128-wide heads.  Other head dimensions (8 to 256, what
             # the MSE stage takes) get their codes and norms from the same kernels and the residual part (reconstruction,
             # projection by S, signs, norm) from float32 tensor operations on the device: the reference's own arithmetic.
             return
@@ -151,8 +151,10 @@ class TurboQuantCompressorV2:
         residual = x - k_mse
         signs = (residual @ self._s(dev).T) >= 0
         weights = torch.tensor([128, 64, 32, 16, 8, 4, 2, 1], device=dev, dtype=torch.int32)      # coordinate 8b + k in bit 7 - k
-        sign_bytes = (signs.reshape(-1, D // 8, 8).to(torch.int32) * weights).sum(-1).to(torch.uint8)
-        return {"idx_bytes": first["idx_bytes"], "vec_norms": first["vec_norms"], "sign_bytes": sign_bytes.reshape(B, H, S, D // 8),
+        if D % 8:       # the bits of the last byte a vector does not fill stay clear
+            signs = torch.nn.functional.pad(signs, (0, 8 - D % 8))
+        sign_bytes = (signs.reshape(-1, -(-D // 8), 8).to(torch.int32) * weights).sum(-1).to(torch.uint8)
+        return {"idx_bytes": first["idx_bytes"], "vec_norms": first["vec_norms"], "sign_bytes": sign_bytes.reshape(B, H, S, -(-D // 8)),
                 "residual_norm": torch.norm(residual, dim=-1).to(torch.float16).reshape(B, H, S), "shape": (B, H, S, D)}
 
     def empty_packed(self, B: int, H: int, S: int, device) -> dict:
@@ -161,7 +163,7 @@ class TurboQuantCompressorV2:
         G = -(-D // (8 // self.mse_bits))
         return {"idx_bytes": torch.empty((B, H, S, G), dtype=torch.uint8, device=device),
                 "vec_norms": torch.empty((B, H, S), dtype=torch.float16, device=device),
-                "sign_bytes": torch.empty((B, H, S, D // 8), dtype=torch.uint8, device=device),
+                "sign_bytes": torch.empty((B, H, S, -(-D // 8)), dtype=torch.uint8, device=device),
                 "residual_norm": torch.empty((B, H, S), dtype=torch.float16, device=device), "shape": (B, H, S, D)}
 
     def job(self, states: torch.Tensor, packed: dict) -> dict:
@@ -176,10 +178,10 @@ class TurboQuantCompressorV2:
         {-1,+1} [B,H,S,D], "residual_norm", "shape", expanded from the packed form."""
         B, H, S, D = compressed["shape"]
         k_mse = self._mse.decompress({"idx_bytes": compressed["idx_bytes"], "vec_norms": compressed["vec_norms"],
-                                      "shape": (B, H, S, D), "idx_pad": 0}).to(torch.float16)
+                                      "shape": (B, H, S, D), "idx_pad": -D % (8 // self.mse_bits)}).to(torch.float16)
         shifts = torch.arange(7, -1, -1, device=compressed["sign_bytes"].device, dtype=torch.uint8)
         bits = (compressed["sign_bytes"].unsqueeze(-1) >> shifts) & 1
-        signs = (bits.to(torch.int8) * 2 - 1).reshape(B, H, S, D)
+        signs = (bits.to(torch.int8) * 2 - 1).reshape(B, H, S, -1)[..., :D]
         return {"k_mse": k_mse, "qjl_signs": signs, "residual_norm": compressed["residual_norm"], "shape": (B, H, S, D)}
 
     @torch.no_grad()
@@ -253,8 +255,11 @@ class TurboQuantCompressorMSE:
         idx_bytes = compressed.get("idx_bytes")
         if idx_bytes is None:
             ipb = 8 // self.bits
-            codes = compressed["indices"].reshape(B * H * S, D // ipb, ipb).to(torch.int32)
+            codes = compressed["indices"].reshape(B * H * S, D).to(torch.int32)
+            if D % ipb:     # compressors_v3.py:64-68: zero codes up to a whole byte
+                codes = torch.nn.functional.pad(codes, (0, ipb - D % ipb))
+            codes = codes.reshape(B * H * S, -1, ipb)
             weights = torch.tensor([1 << (self.bits * i) for i in range(ipb - 1, -1, -1)], device=codes.device, dtype=torch.int32)
             idx_bytes = (codes * weights).sum(-1).to(torch.uint8).reshape(B, H, S, -1)
         return self._mse.decompress({"idx_bytes": idx_bytes, "vec_norms": compressed["vec_norms"].reshape(B, H, S),
-                                     "shape": (B, H, S, D), "idx_pad": 0})
+                                     "shape": (B, H, S, D), "idx_pad": -D % (8 // self.bits)})

@@ -1,6 +1,10 @@
-// compress and decompress for head dimensions other than 128: any multiple of 32 from 32 to 256, taken at run
-// time (upstream turboquant/compressors_v3.py:37-43 builds its rotation and codebook for whatever head_dim it
-// is given; :46-81 compress, :84-105 decompress).  Same arithmetic as the 128-wide kernels (split rotation on the
+// compress and decompress for head dimensions other than 128: 8 to 256, taken at run time (upstream
+// turboquant/compressors_v3.py:37-43 builds its rotation and codebook for whatever head_dim it is given; :46-81
+// compress, :84-105 decompress).  A dimension that is not a multiple of 32 is worked on as the next multiple (the
+// RAGGED instantiations): the operand sets in the table are those of the rotation extended by zeros, the elements a
+// vector does not have are staged as zeros, the coordinates it does not have get the code 0 (:64-68 pads the codes of
+// a vector with zeros to a whole byte) and are neither decoded nor stored on the way back; input, packed codes and
+// output are then moved element by element and byte by byte, since nothing about their alignment is known.  Same arithmetic as the 128-wide kernels (split rotation on the
 // matrix cores, fp32 accumulation, norm applied after the rotation, threshold-grid code search, MSB-first packing,
 // fp16 centroids on the way back), in a plain form: no register-resident rotation, no software pipeline.
 //
@@ -69,8 +73,9 @@ struct PackAny {
     static constexpr int NW = NB < 4 ? 1 : NB / 4;
 };
 
-template <int DTYPE, int BITS>
-__global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t d, uint32_t nt) {
+// d: the dimension of the operand sets (a multiple of 32); dl: the head dimension itself (RAGGED: dl < d)
+template <int DTYPE, int BITS, bool RAGGED>
+__global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t d, uint32_t dl, uint32_t nt) {
     using T = AnyIn<DTYPE>;
     using P = PackAny<BITS>;
     constexpr int ELEM = T::ELEM, NT = T::NT;      // NT: the most column tiles a group may have; nt <= NT: those it has
@@ -100,7 +105,7 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kern
     const uint32_t a_term = TQ_OPERAND_BYTES_FOR(d);
     tq_copy_to_lds(lds_grid, job.table + hd->off_grid, hd->grid_cells * 8u, tid, nthreads);
     const float grid_scale = hd->grid_scale, grid_bias = hd->grid_bias;
-    const uint32_t g_bytes = d / IPB;                // packed bytes per vector
+    const uint32_t g_bytes = (dl + IPB - 1u) / IPB;  // packed bytes per vector
 
     auto load_a = [&](uint32_t rb, uint32_t s, tq_u4 (&a)[T::ATERMS]) {
         const uint8_t *p = a_src + (((size_t)rb * steps + s) * 64u + lane) * 16u;
@@ -117,7 +122,22 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kern
             const uint32_t v = i / pieces, p = i - v * pieces;
             uint32_t gv = g * GV + v;
             gv = gv < job.n_vec ? gv : job.n_vec - 1u;
-            return tq_gload16(job.states + tq_vec_offset(job, gv) + p * 16u);
+            if constexpr (RAGGED) {      // element by element; what lies past the vector's end is zero
+                constexpr uint32_t EPP = 16 / ELEM;
+                const TQ_GLOBAL uint8_t *src = (const TQ_GLOBAL uint8_t *)job.states + tq_vec_offset(job, gv);
+                tq_u4 q = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (uint32_t k = 0; k < EPP; ++k) {
+                    const uint32_t e = p * EPP + k;
+                    if (e < dl) {
+                        if constexpr (ELEM == 2) q[k / 2] |= (uint32_t)*reinterpret_cast<const TQ_GLOBAL uint16_t *>(src + 2u * e) << (16 * (k & 1));
+                        else q[k] = *reinterpret_cast<const TQ_GLOBAL uint32_t *>(src + 4u * e);
+                    }
+                }
+                return q;
+            } else {
+                return tq_gload16(job.states + tq_vec_offset(job, gv) + p * 16u);
+            }
         };
         auto place = [&](uint32_t i, const tq_u4 q) {
             const uint32_t v = i / pieces, p = i - v * pieces;
@@ -219,7 +239,8 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kern
                     const uint32_t addr = __float_as_uint(fmaf(a, inv_cell, grid_bias)) & TQ_GRID_ADDR_MASK;
                     const tq_u2 cell = *reinterpret_cast<const tq_u2 *>(lds_grid + addr);
                     const float t = fmaf(a, inv, -__uint_as_float(cell[0]));
-                    const uint32_t code = cell[1] + (~__float_as_uint(t) >> 31);      // base + !(rho < threshold)
+                    uint32_t code = cell[1] + (~__float_as_uint(t) >> 31);            // base + !(rho < threshold)
+                    if constexpr (RAGGED) code = 32u * rb + 16u * hk + (uint32_t)r < dl ? code : 0u;
                     const int byte = r / IPB, k = r % IPB;                            // most significant code of a byte first
                     words[byte / 4] |= code << (8 * (byte % 4) + BITS * (IPB - 1 - k));
                 }
@@ -227,7 +248,12 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kern
                 if (v < job.n_vec) {
                     const uint32_t slot = tq_packed_slot(job, v);
                     uint8_t *dst = job.idx_bytes + (size_t)slot * g_bytes + (2u * rb + hk) * NB;
-                    if constexpr (NB == 2) {
+                    if constexpr (RAGGED) {
+#pragma unroll
+                        for (int b = 0; b < NB; ++b)
+                            if ((2u * rb + hk) * NB + (uint32_t)b < g_bytes)
+                                *((TQ_GLOBAL uint8_t *)dst + b) = (uint8_t)(words[b / 4] >> (8 * (b % 4)));
+                    } else if constexpr (NB == 2) {
                         tq_gstore2(reinterpret_cast<uint16_t *>(dst), (uint16_t)words[0]);
                     } else if constexpr (NB == 4) {
                         *reinterpret_cast<TQ_GLOBAL uint32_t *>((TQ_GLOBAL uint8_t *)dst) = words[0];
@@ -248,8 +274,8 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kern
     }
 }
 
-template <int DTYPE, int IPB>
-__global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t d, uint32_t nt) {
+template <int DTYPE, int IPB, bool RAGGED>
+__global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t d, uint32_t dl, uint32_t nt) {
     constexpr int ELEM = DTYPE == TQ_F32 ? 4 : 2;
     constexpr int NT = DEC_NT;
     const uint32_t GV = nt * 32u;
@@ -267,7 +293,8 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_ke
 
     const uint32_t row_halves = d + ROW_PAD;
     const uint32_t tiles = d / 32u, steps = d / 16u;
-    const uint32_t g_bytes = d / IPB, g_words = g_bytes / 4u;
+    const uint32_t g_words = d / IPB / 4u;               // staged words per vector (of the padded dimension)
+    const uint32_t g_bytes = (dl + IPB - 1u) / IPB;      // packed bytes per vector in memory
     uint8_t *lds_lut = lds;
     float *norms = reinterpret_cast<float *>(lds + 4096);
     uint16_t *ys = reinterpret_cast<uint16_t *>(norms + GV);
@@ -286,7 +313,16 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_ke
             uint32_t gv = g * GV + v;
             gv = gv < job.n_vec ? gv : job.n_vec - 1u;
             const uint32_t slot = tq_packed_slot(job, gv);
-            return *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)job.idx_bytes + (size_t)slot * g_bytes + 4u * w);
+            if constexpr (RAGGED) {      // byte by byte; past the vector's last byte: zero (never decoded)
+                const TQ_GLOBAL uint8_t *src = (const TQ_GLOBAL uint8_t *)job.idx_bytes + (size_t)slot * g_bytes;
+                uint32_t raw = 0u;
+#pragma unroll
+                for (uint32_t b = 0; b < 4u; ++b)
+                    if (4u * w + b < g_bytes) raw |= (uint32_t)src[4u * w + b] << (8u * b);
+                return raw;
+            } else {
+                return *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)job.idx_bytes + (size_t)slot * g_bytes + 4u * w);
+            }
         };
         auto place = [&](uint32_t i, uint32_t raw) {
             const uint32_t v = i / g_words, w = i - v * g_words;
@@ -298,6 +334,13 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_ke
                 else if constexpr (ENTRY == 4) *reinterpret_cast<uint32_t *>(dst + b * ENTRY) = *reinterpret_cast<const uint32_t *>(e);
                 else if constexpr (ENTRY == 8) *reinterpret_cast<tq_u2 *>(dst + b * ENTRY) = *reinterpret_cast<const tq_u2 *>(e);
                 else *reinterpret_cast<tq_u4 *>(dst + b * ENTRY) = *reinterpret_cast<const tq_u4 *>(e);
+                if constexpr (RAGGED) {      // coordinates the vector does not have contribute nothing
+                    const uint32_t c0 = (4u * w + (uint32_t)b) * IPB;
+                    uint16_t *y = reinterpret_cast<uint16_t *>(dst + b * ENTRY);
+#pragma unroll
+                    for (uint32_t k = 0; k < (uint32_t)IPB; ++k)
+                        if (c0 + k >= dl) y[k] = 0;
+                }
             }
         };
         const uint32_t total = GV * g_words;
@@ -349,7 +392,22 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_ke
                 if (v >= job.n_vec) continue;
                 const float nrm = norms[(share.ct0 + ct) * 32u + n];
                 uint8_t *dst = out_base + tq_vec_offset(job, v) + (32u * rb + 16u * hk) * ELEM;
-                if constexpr (ELEM == 2) {
+                if constexpr (RAGGED) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        if (32u * rb + 16u * hk + (uint32_t)r >= dl) break;
+                        const float x = acc[ct][r] * nrm;
+                        if constexpr (DTYPE == TQ_F32) {
+                            *reinterpret_cast<TQ_GLOBAL uint32_t *>((TQ_GLOBAL uint8_t *)dst + 4 * r) = __float_as_uint(x);
+                        } else if constexpr (DTYPE == TQ_F16) {
+                            const _Float16 h = (_Float16)x;
+                            *reinterpret_cast<TQ_GLOBAL uint16_t *>((TQ_GLOBAL uint8_t *)dst + 2 * r) = __builtin_bit_cast(uint16_t, h);
+                        } else {
+                            const __bf16 h = (__bf16)x;
+                            *reinterpret_cast<TQ_GLOBAL uint16_t *>((TQ_GLOBAL uint8_t *)dst + 2 * r) = __builtin_bit_cast(uint16_t, h);
+                        }
+                    }
+                } else if constexpr (ELEM == 2) {
 #pragma unroll
                     for (int c = 0; c < 2; ++c) {
                         tq_u4 o;
@@ -699,7 +757,7 @@ int device_cus(int &dev, int &cus) {
 // dynamic LDS; `raised[dev]` remembers the largest LDS size the kernel has been allowed on each device.
 template <typename K, typename L>
 int launch(K kernel, uint32_t (&raised)[MAX_DEVICES], L lds_for, uint32_t nt_max, const TqDevJob &job,
-           const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, hipStream_t stream) {
+           const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, uint32_t dl, hipStream_t stream) {
     // column tiles per group: as many as leave room for two blocks on a compute unit (the phases of a block do not
     // overlap one another; a second block fills the gaps), but at least half of the most
     uint32_t nt = nt_max;
@@ -720,7 +778,7 @@ int launch(K kernel, uint32_t (&raised)[MAX_DEVICES], L lds_for, uint32_t nt_max
     const uint32_t waves = MAX_WAVES;
     const int resident = lds <= 53u * 1024u ? 3 : lds <= 80u * 1024u ? 2 : 1;     // blocks per compute unit (160 KiB of LDS, 168 registers)
     const uint32_t bx = tq_blocks_per_job(groups, cus * resident, n_jobs);
-    hipLaunchKernelGGL(kernel, dim3(bx, (unsigned)n_jobs, 1), dim3(waves * TQ_WAVE, 1, 1), lds, stream, job, jobs_dev, d, nt);
+    hipLaunchKernelGGL(kernel, dim3(bx, (unsigned)n_jobs, 1), dim3(waves * TQ_WAVE, 1, 1), lds, stream, job, jobs_dev, d, dl, nt);
     return (int)hipGetLastError();
 }
 
@@ -754,9 +812,15 @@ int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uin
             return launch_d256(&tq_d256_compress_kernel<DTYPE, BITS>, raised256, lds, 512u, 1, job, jobs_dev, n_jobs, max_vec, s);
         }
     }
+    const uint32_t dp = TQ_PADDED_DIM(d);
+    if (dp != d) {
+        static uint32_t raised_ragged[MAX_DEVICES] = {};
+        return launch(&tq_anydim_compress_kernel<DTYPE, BITS, true>, raised_ragged, compress_lds_bytes<DTYPE>, AnyIn<DTYPE>::NT, job,
+                      jobs_dev, n_jobs, max_vec, dp, d, s);
+    }
     static uint32_t raised[MAX_DEVICES] = {};
-    return launch(&tq_anydim_compress_kernel<DTYPE, BITS>, raised, compress_lds_bytes<DTYPE>, AnyIn<DTYPE>::NT, job, jobs_dev,
-                  n_jobs, max_vec, d, s);
+    return launch(&tq_anydim_compress_kernel<DTYPE, BITS, false>, raised, compress_lds_bytes<DTYPE>, AnyIn<DTYPE>::NT, job, jobs_dev,
+                  n_jobs, max_vec, d, d, s);
 }
 template <int DTYPE>
 int compress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, hipStream_t s) {
@@ -780,8 +844,14 @@ int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, u
             return launch_d256(&tq_d256_decompress_kernel<DTYPE, IPB>, raised256, lds, 256u, 2, job, jobs_dev, n_jobs, max_vec, s);
         }
     }
+    const uint32_t dp = TQ_PADDED_DIM(d);
+    if (dp != d) {
+        static uint32_t raised_ragged[MAX_DEVICES] = {};
+        return launch(&tq_anydim_decompress_kernel<DTYPE, IPB, true>, raised_ragged, decompress_lds_bytes, DEC_NT, job, jobs_dev, n_jobs,
+                      max_vec, dp, d, s);
+    }
     static uint32_t raised[MAX_DEVICES] = {};
-    return launch(&tq_anydim_decompress_kernel<DTYPE, IPB>, raised, decompress_lds_bytes, DEC_NT, job, jobs_dev, n_jobs, max_vec, d, s);
+    return launch(&tq_anydim_decompress_kernel<DTYPE, IPB, false>, raised, decompress_lds_bytes, DEC_NT, job, jobs_dev, n_jobs, max_vec, d, d, s);
 }
 template <int DTYPE>
 int decompress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t d, hipStream_t s) {
@@ -797,7 +867,7 @@ int decompress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n
 }  // namespace
 
 bool tq_anydim_supported(int head_dim) {
-    return head_dim >= TQ_ANYDIM_MIN && head_dim <= TQ_ANYDIM_MAX && head_dim % 32 == 0;
+    return head_dim >= TQ_ANYDIM_MIN && head_dim <= TQ_ANYDIM_MAX;
 }
 
 int tq_anydim_compress(int dtype, int bits, int head_dim, const TqDevJob &single, const tq_job *jobs_dev, int n_jobs,

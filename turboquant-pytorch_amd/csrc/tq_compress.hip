@@ -762,9 +762,10 @@ int check_job(const void *states, int dtype, long long rows, long long tokens, l
     if (token_stride < head_dim && tokens > 1) return TQ_ERR_SIZE;
     if (rows > 1 && row_stride < 0) return TQ_ERR_SIZE;
     if (packed_row_stride != 0 && (packed_row_stride < tokens || packed_row_stride > (long long)0x7fffffff / rows)) return TQ_ERR_SIZE;
-    if (((uintptr_t)states & 15u) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & (tq_packed_alignment(head_dim, bits) - 1u)) || ((uintptr_t)vec_norms & 1u))
+    const uintptr_t va = tq_vector_alignment(head_dim, eb) - 1u;
+    if (((uintptr_t)states & va) || ((uintptr_t)table & 15u) || ((uintptr_t)idx_bytes & (tq_packed_alignment(head_dim, bits) - 1u)) || ((uintptr_t)vec_norms & 1u))
         return TQ_ERR_ALIGN;
-    if (((token_stride * eb) & 15) || (rows > 1 && ((row_stride * eb) & 15))) return TQ_ERR_ALIGN;
+    if (((uintptr_t)(token_stride * eb) & va) || (rows > 1 && ((uintptr_t)(row_stride * eb) & va))) return TQ_ERR_ALIGN;
     return TQ_OK;
 }
 

@@ -347,9 +347,16 @@ static inline bool tq_pairable(long long rows, long long tokens, long long token
 // 24-byte vectors starts on a multiple of 8).
 static inline uintptr_t tq_packed_alignment(int head_dim, int bits) {
     if (head_dim == TQ_HEAD_DIM) return 16;
+    if (head_dim % 32) return 1;        // moved byte by byte
     const uintptr_t g = (uintptr_t)((head_dim + (8 / bits) - 1) / (8 / bits));
     const uintptr_t low = g & (~g + 1);
     return low < 16 ? low : 16;
+}
+
+// Alignment of the vectors themselves (pointer and strides, in bytes): 16, except for head dimensions that are not a
+// multiple of 32, whose vectors are moved element by element.
+static inline uintptr_t tq_vector_alignment(int head_dim, int elem_bytes) {
+    return head_dim % 32 ? (uintptr_t)elem_bytes : 16;
 }
 
 // Blocks per job for a (blocks_per_job x n_jobs) grid of equal-cost blocks on `cus` compute units

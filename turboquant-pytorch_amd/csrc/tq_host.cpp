@@ -98,8 +98,8 @@ struct Layout {
     uint32_t lut_entry_bytes;
     uint32_t off_pair_a_f16, off_pair_a_bf16, off_pair_at_f16;     // head_dim 64: room for the operands of diag(Pi, Pi)
 };
-// head dimensions the kernels take: 128 (the tuned kernels) and the other multiples of 32 up to 256
-bool supported_head_dim(int d) { return d >= TQ_ANYDIM_MIN && d <= TQ_ANYDIM_MAX && d % 32 == 0; }
+// head dimensions the kernels take: 128 (the tuned kernels) and every other one from 8 to 256
+bool supported_head_dim(int d) { return d >= TQ_ANYDIM_MIN && d <= TQ_ANYDIM_MAX; }
 
 Layout layout_for(int head_dim, int bits) {
     const uint32_t levels = 1u << bits, ipb = 8u / (uint32_t)bits;
@@ -134,7 +134,7 @@ const char *tq_status_string(int status) {
         case TQ_OK: return "ok";
         case TQ_ERR_NULL: return "null pointer argument";
         case TQ_ERR_BITS: return "bits must be in 1..8";
-        case TQ_ERR_HEAD_DIM: return "unsupported head_dim (compress / decompress: multiples of 32 up to 256; the other kernels: 128)";
+        case TQ_ERR_HEAD_DIM: return "unsupported head_dim (compress / decompress: 8 to 256; the other kernels: 128)";
         case TQ_ERR_DTYPE: return "unknown element type";
         case TQ_ERR_SIZE: return "invalid size or stride";
         case TQ_ERR_CODEBOOK: return "centroids must be finite and strictly ascending";
@@ -236,8 +236,10 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     if (!ok) return TQ_ERR_CODEBOOK;  // levels too dense for the grid the kernels keep in LDS
     std::memcpy(blob + L.off_grid, grid.data(), (size_t)cells * sizeof(TqGridCell));
 
-    // ---- rotation operands ----
-    const int tiles = D / 32, steps = D / 16;
+    // ---- rotation operands (of the rotation extended by zeros to a multiple of 32) ----
+    const int DP = TQ_PADDED_DIM(D);
+    const int tiles = DP / 32, steps = DP / 16;
+    auto pi_at = [&](int row, int col) { return (row < D && col < D) ? Pi[row * D + col] : 0.0f; };
     auto operand_index = [steps](int t, int s, int l, int i) { return (((size_t)t * steps + s) * 64 + l) * 8 + i; };
     uint16_t *a_f16 = reinterpret_cast<uint16_t *>(blob + L.off_a_f16);
     uint16_t *a_bf16 = reinterpret_cast<uint16_t *>(blob + L.off_a_bf16);
@@ -256,7 +258,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
                     const size_t o = operand_index(t, s, l, i);
                     {   // compress: rotated[out] = sum_k x[k] * Pi[out][k],  k = 16s + 8hk + i
                         const int k = 16 * s + 8 * hk + i;
-                        const float p = Pi[out_c * D + k];
+                        const float p = pi_at(out_c, k);
                         const double ps = (double)p * pi_scale;
                         const uint16_t hi = to_f16((float)ps);
                         const uint16_t lo = to_f16((float)(ps - (double)from_f16(hi)));
@@ -272,7 +274,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
                     }
                     {   // decompress: x[out] = sum_j y[j] * Pi[j][out],  j = 64hk + 8s + i
                         const int j = tuned ? 64 * hk + 8 * s + i : 16 * s + 8 * hk + i;
-                        const float p = Pi[j * D + out_d];
+                        const float p = pi_at(j, out_d);
                         const uint16_t hi = to_f16(p);
                         at_f16[o] = hi;
                         at_f16[term + o] = to_f16((float)((double)p - (double)from_f16(hi)));
@@ -350,6 +352,7 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     hd.off_pair_a_f16 = paired ? L.off_pair_a_f16 : 0u;
     hd.off_pair_a_bf16 = paired ? L.off_pair_a_bf16 : 0u;
     hd.off_pair_at_f16 = paired ? L.off_pair_at_f16 : 0u;
+    hd.padded_dim = (uint32_t)DP;
     hd.off_centroids = L.off_centroids;
     hd.off_thresholds = L.off_thresholds;
     hd.lut_entry_bytes = L.lut_entry_bytes;

@@ -6,7 +6,7 @@
 #include <stdint.h>
 
 #define TQ_TABLE_MAGIC 0x54514d49u /* "TQMI" */
-#define TQ_TABLE_VERSION 7u
+#define TQ_TABLE_VERSION 8u
 #define TQ_HEAD_DIM 128
 
 // --- MFMA operand tiling (v_mfma_f32_32x32x16_{f16,bf16}) --------------------------------
@@ -29,13 +29,18 @@
 #define TQ_STEPS 8  /* 128 inputs  / 16 deep  */
 #define TQ_OPERAND_BYTES (TQ_TILES * TQ_STEPS * 64 * 16) /* one 128x128 16-bit operand set: 32 KiB */
 
-// Other head dimensions (multiples of 32 from TQ_ANYDIM_MIN to TQ_ANYDIM_MAX) go through one pair of kernels that
-// takes the dimension at run time.  Their tables hold d/32 row tiles x d/16 steps per operand set, compress AND
-// decompress operands in the compress tiling above (out = 32t + 16h + r, in = 16s + 8hk + i), and a quantiser grid
-// of up to TQ_GRID_LDS_BYTES / 8 cells whatever the width (those kernels keep a single, unshifted copy).
-#define TQ_ANYDIM_MIN 32
+// Other head dimensions (TQ_ANYDIM_MIN to TQ_ANYDIM_MAX) go through one pair of kernels that takes the dimension at run
+// time.  Their tables hold d/32 row tiles x d/16 steps per operand set, compress AND decompress operands in the compress
+// tiling above (out = 32t + 16h + r, in = 16s + 8hk + i), and a quantiser grid of up to TQ_GRID_LDS_BYTES / 8 cells
+// whatever the width (those kernels keep a single, unshifted copy).
+// A head dimension that is not a multiple of 32 is worked on as the next multiple: the operand sets are those of the
+// rotation extended by zero rows and columns, the kernels read the missing input elements as zeros, give the missing
+// coordinates the code 0 (upstream turboquant/compressors_v3.py:64-68 pads the codes of a vector with zeros up to a
+// whole byte) and neither decode nor store them on the way back.
+#define TQ_ANYDIM_MIN 8
 #define TQ_ANYDIM_MAX 256
-#define TQ_OPERAND_BYTES_FOR(d) (((d) / 32) * ((d) / 16) * 64 * 16)
+#define TQ_PADDED_DIM(d) ((((d) + 31) / 32) * 32)
+#define TQ_OPERAND_BYTES_FOR(d) ((TQ_PADDED_DIM(d) / 32) * (TQ_PADDED_DIM(d) / 16) * 64 * 16)
 
 // The fp16 split of Pi is stored multiplied by 2^TQ_F16_PI_SHIFT so that the low term stays
 // in the fp16 normal range; the kernels fold 2^-shift into the per-vector scale.
@@ -93,7 +98,8 @@ struct TqTableHeader {
     uint32_t off_pair_a_f16;  // compress operand of diag(Pi, Pi) * 2^shift as fp16 hi, lo     (2 x 32 KiB)
     uint32_t off_pair_a_bf16; // compress operand of diag(Pi, Pi) as bf16 hi, mid, lo          (3 x 32 KiB)
     uint32_t off_pair_at_f16; // decompress operand of diag(Pi, Pi)^T as fp16 hi, lo           (2 x 32 KiB)
-    uint32_t reserved[42];
+    uint32_t padded_dim;      // TQ_PADDED_DIM(head_dim): the dimension of the operand sets
+    uint32_t reserved[41];
 };
 static_assert(sizeof(TqTableHeader) == 256, "header is one 256-byte block");
 
