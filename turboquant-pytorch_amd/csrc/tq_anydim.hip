@@ -122,10 +122,13 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kern
             const uint32_t v = i / pieces, p = i - v * pieces;
             uint32_t gv = g * GV + v;
             gv = gv < job.n_vec ? gv : job.n_vec - 1u;
-            if constexpr (RAGGED) {      // element by element; what lies past the vector's end is zero
+            if constexpr (RAGGED) {      // what lies past the vector's end is zero
                 constexpr uint32_t EPP = 16 / ELEM;
                 const TQ_GLOBAL uint8_t *src = (const TQ_GLOBAL uint8_t *)job.states + tq_vec_offset(job, gv);
-                tq_u4 q = {0u, 0u, 0u, 0u};
+                if (p * EPP + EPP <= dl && (((uintptr_t)src + p * 16u) & 15u) == 0u)      // a whole piece at an aligned address
+                    return *reinterpret_cast<const TQ_GLOBAL tq_u4 *>(src + p * 16u);
+                if (p * EPP >= dl) return tq_u4{0u, 0u, 0u, 0u};
+                tq_u4 q = {0u, 0u, 0u, 0u};      // element by element
 #pragma unroll
                 for (uint32_t k = 0; k < EPP; ++k) {
                     const uint32_t e = p * EPP + k;
@@ -248,7 +251,9 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_compress_kern
                 if (v < job.n_vec) {
                     const uint32_t slot = tq_packed_slot(job, v);
                     uint8_t *dst = job.idx_bytes + (size_t)slot * g_bytes + (2u * rb + hk) * NB;
-                    if constexpr (RAGGED) {
+                    bool bytewise = false;
+                    if constexpr (RAGGED) bytewise = (2u * rb + hk) * NB + NB > g_bytes || ((uintptr_t)dst & (uintptr_t)(NB - 1));
+                    if (bytewise) {
 #pragma unroll
                         for (int b = 0; b < NB; ++b)
                             if ((2u * rb + hk) * NB + (uint32_t)b < g_bytes)
@@ -315,6 +320,8 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_ke
             const uint32_t slot = tq_packed_slot(job, gv);
             if constexpr (RAGGED) {      // byte by byte; past the vector's last byte: zero (never decoded)
                 const TQ_GLOBAL uint8_t *src = (const TQ_GLOBAL uint8_t *)job.idx_bytes + (size_t)slot * g_bytes;
+                if (4u * w + 4u <= g_bytes && (((uintptr_t)src + 4u * w) & 3u) == 0u)      // a whole word at an aligned address
+                    return *reinterpret_cast<const TQ_GLOBAL uint32_t *>(src + 4u * w);
                 uint32_t raw = 0u;
 #pragma unroll
                 for (uint32_t b = 0; b < 4u; ++b)
@@ -392,7 +399,9 @@ __global__ __launch_bounds__(MAX_WAVES *TQ_WAVE, 2) void tq_anydim_decompress_ke
                 if (v >= job.n_vec) continue;
                 const float nrm = norms[(share.ct0 + ct) * 32u + n];
                 uint8_t *dst = out_base + tq_vec_offset(job, v) + (32u * rb + 16u * hk) * ELEM;
-                if constexpr (RAGGED) {
+                bool elementwise = false;
+                if constexpr (RAGGED) elementwise = 32u * rb + 16u * hk + 16u > dl || ((uintptr_t)dst & 15u);
+                if (elementwise) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         if (32u * rb + 16u * hk + (uint32_t)r >= dl) break;
