@@ -20,8 +20,8 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(CSRC, "libtqamd.so")
-SOURCES = ("tq_host.cpp", "tq_compress.hip", "tq_decompress.hip", "tq_anydim.hip", "tq_attend.hip", "tq_qjl.hip")
-HEADERS = ("tq_table.h", "tq_device.h", "tq_anydim.h", os.path.join("..", "..", "include", "tqamd.h"))
+SOURCES = ("tq_host.cpp", "tq_compress.hip", "tq_decompress.hip", "tq_anydim.hip", "tq_wide.hip", "tq_attend.hip", "tq_qjl.hip")
+HEADERS = ("tq_table.h", "tq_device.h", "tq_anydim.h", "tq_wide.h", os.path.join("..", "..", "include", "tqamd.h"))
 GPU_ARCH = "gfx950"
 
 TQ_F32, TQ_F16, TQ_BF16 = 0, 1, 2

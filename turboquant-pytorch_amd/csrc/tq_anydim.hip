@@ -19,6 +19,7 @@
 #include <type_traits>
 
 #include "tq_anydim.h"
+#include "tq_wide.h"
 
 namespace {
 
@@ -883,6 +884,7 @@ int tq_anydim_compress(int dtype, int bits, int head_dim, const TqDevJob &single
                        uint32_t max_vec, hipStream_t stream) {
     if (!tq_anydim_supported(head_dim)) return TQ_ERR_HEAD_DIM;
     if (bits < 1 || bits > 8) return TQ_ERR_BITS;
+    if (tq_wide_supported(head_dim, dtype)) return tq_wide_compress(dtype, bits, head_dim, single, jobs_dev, n_jobs, max_vec, stream);
     const uint32_t d = (uint32_t)head_dim;
     switch (dtype) {
         case TQ_F32: return compress_bits<TQ_F32>(bits, single, jobs_dev, n_jobs, max_vec, d, stream);
@@ -896,6 +898,7 @@ int tq_anydim_decompress(int dtype, int bits, int head_dim, const TqDevJob &sing
                          uint32_t max_vec, hipStream_t stream) {
     if (!tq_anydim_supported(head_dim)) return TQ_ERR_HEAD_DIM;
     if (bits < 1 || bits > 8) return TQ_ERR_BITS;
+    if (tq_wide_supported(head_dim, dtype)) return tq_wide_decompress(dtype, bits, head_dim, single, jobs_dev, n_jobs, max_vec, stream);
     const uint32_t d = (uint32_t)head_dim;
     switch (dtype) {
         case TQ_F32: return decompress_bits<TQ_F32>(bits, single, jobs_dev, n_jobs, max_vec, d, stream);
