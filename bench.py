@@ -186,6 +186,59 @@ def cpu_baseline(pkg, widths, budget_s=20.0, head_dim=128):
     }
 
 
+def power_probe(torch, step, seconds):
+    """Socket power and clocks while the step runs back to back: `amd-smi metric -p -c` is called every half second from a
+    thread while this thread keeps the device busy (batches of steps with a synchronisation in between, so the queue stays
+    short).  Returns what amd-smi printed, reduced to the figures; untimed, and not part of any other number."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+    exe = shutil.which("amd-smi") or "/opt/rocm/bin/amd-smi"
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            try:
+                out = subprocess.run([exe, "metric", "-p", "-c"], capture_output=True, text=True, timeout=10).stdout
+            except Exception as e:      # the tool is missing or hangs: say so in the result
+                samples.append({"error": repr(e)})
+                return
+            power = re.search(r"SOCKET_POWER:\s*(\d+)", out)
+            gfx = [int(v) for v in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", out)]
+            mem = re.search(r"MEM_0:\s*\n\s*CLK:\s*(\d+)\s*MHz", out)
+            samples.append({"t": time.perf_counter(), "socket_W": int(power.group(1)) if power else None,
+                            "gfx_clk_MHz": gfx, "mem_clk_MHz": int(mem.group(1)) if mem else None, "raw_chars": len(out)})
+            stop.wait(0.5)
+
+    th = threading.Thread(target=sampler, daemon=True)
+    t0 = time.perf_counter()
+    th.start()
+    n = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+        n += 20
+    elapsed = time.perf_counter() - t0
+    stop.set()
+    th.join(timeout=15)
+    good = [x for x in samples if x.get("socket_W") is not None and x["t"] - t0 > 1.0]       # skip the first second
+    res = {"seconds": elapsed, "steps": n, "ms_per_step": elapsed * 1e3 / max(n, 1), "samples": len(good),
+           "how": "amd-smi metric -p -c every 0.5 s while the step runs back to back (samples of the first second left out)"}
+    if good:
+        res["socket_W"] = sorted(x["socket_W"] for x in good)[len(good) // 2]
+        clocks = sorted(c for x in good for c in x["gfx_clk_MHz"])
+        if clocks:
+            res["gfx_clk_MHz"] = {"min": clocks[0], "median": clocks[len(clocks) // 2], "max": clocks[-1]}
+        mems = [x["mem_clk_MHz"] for x in good if x["mem_clk_MHz"]]
+        if mems:
+            res["mem_clk_MHz"] = sorted(mems)[len(mems) // 2]
+    else:
+        res["note"] = "amd-smi gave no usable sample: " + json.dumps(samples[:2])
+    return res
+
+
 def run_v2(args, torch, pkg, w, dev):
     """TurboQuantCompressorV2 on synthetic keys: a step compresses the keys of every layer (one launch for all layers
     through the batched entry point: codes, norms, residual signs and residual norms from one pass over the input) and
@@ -357,6 +410,9 @@ def main():
                     help="time the memory-skeleton build of the two codec kernels (csrc/libtqamd_skeleton.so from "
                          "_native.build_skeleton(): loads, LDS traffic and stores only; the output is garbage)")
     ap.add_argument("--no-stream-rates", action="store_true", help="skip the plain-stream leg (copy / read / write rates of the part)")
+    ap.add_argument("--power-probe", type=float, default=0.0, metavar="SECONDS",
+                    help="after the timed region keep the step running for this long and sample socket power and clocks with amd-smi "
+                         "(reported as `power_probe`; untimed)")
     ap.add_argument("--launch-order", default="",
                     help="sequence of the step's launches, e.g. c2,c4,c8,d8,d4,d2 (default: compress by width, then decompress by width)")
     args = ap.parse_args()
@@ -578,6 +634,8 @@ def main():
         # the part's plain-stream rates beside the codec's: what a copy, a read and a write kernel reach on this box
         result["roofline"]["stream_GBps"] = stream_rates(torch, dev)
         result["roofline"]["step_frac_of_copy_rate"] = result["step_GBps"] / result["roofline"]["stream_GBps"]["copy"]
+    if args.power_probe > 0:
+        result["power_probe"] = power_probe(torch, step, args.power_probe)
     if not args.no_cpu_baseline and not args.skeleton:
         result["cpu_baseline"] = cpu_baseline(pkg, widths, args.cpu_seconds, head_dim=D)
     print(json.dumps(result))
