@@ -149,6 +149,32 @@ def test_thresholds_and_grid_equal_argmin(pkg, golden, oracle, bits):
     assert np.array_equal(pkg._native.quantize_host(table, r), ref)
 
 
+@pytest.mark.parametrize("D,bits", [(8, 8), (8, 6), (12, 7), (16, 8), (10, 5)])
+def test_codebooks_that_reach_beyond_the_unit_interval(pkg, oracle, D, bits):
+    """Very small head dimensions at many bits: the outer levels of N(0, 1/d) codebooks lie beyond +-1, where no coordinate
+    of a unit vector can fall.  The table builds (thresholds outside the grid's span are counted for every coordinate or
+    for none) and the search agrees with the nearest-centroid definition on everything a coordinate can be."""
+    cent = pkg.LloydMaxCodebook(D, bits).centroids.numpy()
+    g = torch.Generator().manual_seed(D)
+    Pi, _ = torch.linalg.qr(torch.randn(D, D, generator=g))
+    table = pkg._native.build_table(Pi, torch.from_numpy(cent), bits)
+    thr = pkg._native.decision_thresholds(cent)
+    rng = np.random.default_rng(D * bits)
+    near = []
+    for t in thr[np.abs(thr) <= 1.0]:
+        lo = hi = np.float32(t)
+        near.append(lo)
+        for _ in range(3):
+            lo = np.nextafter(lo, np.float32(-np.inf))
+            hi = np.nextafter(hi, np.float32(np.inf))
+            near += [lo, hi]
+    r = np.concatenate([rng.uniform(-1.0, 1.0, 200000).astype(np.float32), np.array(near + [1.0, -1.0, 0.0], np.float32)])
+    r = r[np.abs(r) <= 1.0]
+    ref = np.empty(r.size, np.uint8)
+    oracle._load().tqo_nearest(r, r.size, cent, cent.size, ref)
+    assert np.array_equal(pkg._native.quantize_host(table, r), ref)
+
+
 def test_table_rotation_split_reconstructs_pi(pkg, golden):
     """The 16-bit operand tiles in the table sum back to Pi: fp16 hi+lo to ~2^-21 relative,
     bf16 three terms exactly, and the tiling puts element (out, k) where the kernels read it."""

@@ -210,6 +210,11 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
     // Cell k covers the reals [edge(k), edge(k+1)), edge(k) = (k - cells/2 - 1/16) / scale (see
     // tq_table.h); unit-sphere coordinates satisfy |rho| <= 1 + rounding, the grid spans +-1.0625.
     const double range = 1.0625;
+    // Thresholds outside the span cannot be met by a coordinate of a unit vector (the codebooks of very small head
+    // dimensions at 6 to 8 bits reach beyond +-1): those below count for every coordinate, those above for none.
+    int t_first = 0, t_end = levels - 1;
+    while (t_first < t_end && (double)thr[t_first] < -range) ++t_first;
+    while (t_end > t_first && (double)thr[t_end - 1] > range) --t_end;
     float scale = 0.f, bias = 0.f;
     uint32_t cells = 0;
     std::vector<TqGridCell> grid;
@@ -222,13 +227,13 @@ int tq_table_build(const float *Pi, const float *centroids, int head_dim, int bi
         grid.assign(cells, TqGridCell{INFINITY, 0});
         auto edge = [&](uint32_t k) { return ((double)k - (double)(cells / 2) - 0.0625) / (double)scale; };
         ok = true;
-        int t = 0;  // thresholds are ascending; walk them alongside the cells
+        int t = t_first;  // thresholds are ascending; walk them alongside the cells
         for (uint32_t q = 0; q < cells && ok; ++q) {
             const double lo = q == 0 ? -INFINITY : edge(q), hi = q + 1 == cells ? INFINITY : edge(q + 1);
-            while (t < levels - 1 && (double)thr[t] < lo) ++t;   // below the cell: counted for all of it
+            while (t < t_end && (double)thr[t] < lo) ++t;   // below the cell: counted for all of it
             grid[q].base = (uint32_t)t;
             int inside = 0;
-            while (t + inside < levels - 1 && (double)thr[t + inside] < hi) ++inside;
+            while (t + inside < t_end && (double)thr[t + inside] < hi) ++inside;
             if (inside > 1) { ok = false; break; }
             if (inside == 1) grid[q].threshold = thr[t];
         }
