@@ -413,6 +413,8 @@ def main():
     ap.add_argument("--power-probe", type=float, default=0.0, metavar="SECONDS",
                     help="after the timed region keep the step running for this long and sample socket power and clocks with amd-smi "
                          "(reported as `power_probe`; untimed)")
+    ap.add_argument("--probe-launches", default="all", choices=("all", "compress", "decompress"),
+                    help="which launches of the step the power probe repeats (default: the whole step)")
     ap.add_argument("--launch-order", default="",
                     help="sequence of the step's launches, e.g. c2,c4,c8,d8,d4,d2 (default: compress by width, then decompress by width)")
     args = ap.parse_args()
@@ -635,7 +637,12 @@ def main():
         result["roofline"]["stream_GBps"] = stream_rates(torch, dev)
         result["roofline"]["step_frac_of_copy_rate"] = result["step_GBps"] / result["roofline"]["stream_GBps"]["copy"]
     if args.power_probe > 0:
-        result["power_probe"] = power_probe(torch, step, args.power_probe)
+        def probe_step():
+            for direction, b in launches:
+                if args.probe_launches in ("all", direction):
+                    (comp_lists[b].compress if direction == "compress" else deco_lists[b].decompress)()
+        result["power_probe"] = power_probe(torch, probe_step, args.power_probe)
+        result["power_probe"]["launches"] = args.probe_launches
     if not args.no_cpu_baseline and not args.skeleton:
         result["cpu_baseline"] = cpu_baseline(pkg, widths, args.cpu_seconds, head_dim=D)
     print(json.dumps(result))

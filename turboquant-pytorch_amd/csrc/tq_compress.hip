@@ -45,11 +45,13 @@ namespace {
 #define TQ_PRIO_SHIFT 3
 #endif
 // Measurement build (never the shipped library): the pipelined path keeps its loads, LDS traffic, barriers, norm
-// arithmetic and stores, and leaves out the matrix instructions and the code search.  What it writes is garbage; its
-// time is what the kernel's memory pattern costs on its own.
+// arithmetic and stores, and leaves out the matrix instructions and the code search (1), the matrix instructions only
+// (2) or the code search only (3).  What it writes is garbage; its time is what the rest of the kernel costs on its own.
 #ifndef TQ_SKELETON
 #define TQ_SKELETON 0
 #endif
+#define TQ_SKEL_NO_MFMA (TQ_SKELETON == 1 || TQ_SKELETON == 2)
+#define TQ_SKEL_NO_SEARCH (TQ_SKELETON == 1 || TQ_SKELETON == 3)
 template <int DTYPE> struct InTraits;
 template <> struct InTraits<TQ_F16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = TQ_C16_WAVES; };
 template <> struct InTraits<TQ_BF16> { static constexpr int ELEM = 2, TERMS = 2, MIN_WAVES = TQ_C16_WAVES; };
@@ -479,7 +481,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
                 const uint8_t *stage = lds_stage[SLOT];
                 auto operand = [&](int i) { return *reinterpret_cast<const tq_u4 *>(stage + op_off[i]); };
                 auto mfma = [&](int term, int i, tq_u4 bop) {
-#if TQ_SKELETON
+#if TQ_SKEL_NO_MFMA
                     if (term == 0) acc_new[i] = __uint_as_float(bop[0] ^ bop[1] ^ bop[2] ^ bop[3]);     // the operand read stays alive
 #else
                     acc_new = (DTYPE == TQ_F16) ? mfma_f16(areg[term][i], bop, acc_new) : mfma_bf16(areg[term][i], bop, acc_new);
@@ -500,17 +502,17 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
                     tq_u4 bop_next = bop;
                     tq_u2 n0 = c0, n1 = c1;
                     if (i + 1 < TQ_STEPS) bop_next = operand(i + 1);
-                    if constexpr (SEARCH && !TQ_SKELETON) {
+                    if constexpr (SEARCH && !TQ_SKEL_NO_SEARCH) {
                         if (i >= 1) { n0 = search_lookup(2 * i - 2, acc_old, sc_old); n1 = search_lookup(2 * i - 1, acc_old, sc_old); }
                     }
                     mfma(0, i, bop);
                     if (i < 2) share = sumsq8<DTYPE>(bop, share);
                     if constexpr (SEARCH) {
                         if (i == 0) sc_old = scale_from_shares(par ^ 1u);
-                        if (i >= 2 && !TQ_SKELETON) search_apply(z, 2 * i - 4, acc_old, sc_old, c0);
+                        if (i >= 2 && !TQ_SKEL_NO_SEARCH) search_apply(z, 2 * i - 4, acc_old, sc_old, c0);
                     }
                     mfma(1, i, bop);
-                    if constexpr (SEARCH && !TQ_SKELETON) {
+                    if constexpr (SEARCH && !TQ_SKEL_NO_SEARCH) {
                         if (i >= 2) search_apply(z, 2 * i - 3, acc_old, sc_old, c1);
                     }
                     if (i == 1) {
@@ -546,7 +548,7 @@ __global__ __launch_bounds__(CTHREADS, InTraits<DTYPE>::MIN_WAVES) void tq_compr
                     bop = bop_next; c0 = n0; c1 = n1;
                 }
                 if constexpr (SEARCH) {
-#if TQ_SKELETON
+#if TQ_SKEL_NO_SEARCH
 #pragma unroll
                     for (int w = 0; w < NW; ++w) words[w] = __float_as_uint(acc_old[w] * sc_old.inv);
 #else
