@@ -48,8 +48,8 @@ WORKLOADS = {
     # 64-wide vectors go through the 128-wide kernels two at a time, 256-wide ones through kernels of their own
     "d64-k4v2-64k": dict(layers=8, batch=1, heads=8, tokens=65536, dtype="bf16", key_bits=4, value_bits=2, protected=0, head_dim=64),
     "d256-k4v2-16k": dict(layers=8, batch=1, heads=8, tokens=16384, dtype="bf16", key_bits=4, value_bits=2, protected=0, head_dim=256),
-    # 96 (with 160, 192 and 224: the 256-wide kernels' structure with the dimension as a template argument), and 80, which goes
-    # through the kernels that take the dimension at run time (worked on as 96, in whole 16-byte pieces)
+    # 96 (with 160, 192 and 224: the 256-wide kernels' structure with the dimension as a template argument), and 80, which the
+    # same kernels work on as 96 (zero elements in, zero codes out, whole 16-byte pieces moved as such)
     "d96-k4v2-43k": dict(layers=8, batch=1, heads=8, tokens=43648, dtype="bf16", key_bits=4, value_bits=2, protected=0, head_dim=96),
     "d80-k4v2-52k": dict(layers=8, batch=1, heads=8, tokens=52416, dtype="bf16", key_bits=4, value_bits=2, protected=0, head_dim=80),
     # streaming decode: 64 sequences with 16384 compressed + 128 window tokens; a step is

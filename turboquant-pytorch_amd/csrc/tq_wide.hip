@@ -10,7 +10,11 @@
 // wave as B operands.  A row of such a tile is D*2 bytes, an odd multiple of 64: rows are rotated by their index
 // (piece p of row v sits at position (p + v) mod D/8), which spreads the eight rows a 16-byte LDS access touches over all
 // banks.  Same arithmetic, in the same order, as the run-time-dimension kernels: a vector gets the same bytes whichever
-// of the two compresses it (fp32 elements, and strides these kernels do not assume anything about, go there).
+// of the two compresses it (fp32 elements go there).  The RAGGED instantiations take a head dimension dl that is not a
+// multiple of 32 as the next multiple D, the way the run-time-dimension kernels do: the table holds the rotation extended
+// by zeros, elements a vector does not have are staged as zeros, coordinates it does not have get the code 0 and are
+// neither decoded nor stored; whole 16-byte pieces at aligned addresses take the wide loads and stores, the rest moves
+// element by element.
 #include <mutex>
 #include <type_traits>
 
@@ -39,8 +43,8 @@ __device__ __forceinline__ uint32_t rotated_piece(uint32_t p, uint32_t v) {
     return (p + v) % (uint32_t)Wide<D>::PIECES;
 }
 
-template <int DTYPE, int BITS, int D>
-__global__ __launch_bounds__(Wide<D>::THREADS, Wide<D>::COMPRESS_WAVES_PER_SIMD) void tq_wide_compress_kernel(TqDevJob job0, const tq_job *jobs) {
+template <int DTYPE, int BITS, int D, bool RAGGED>
+__global__ __launch_bounds__(Wide<D>::THREADS, Wide<D>::COMPRESS_WAVES_PER_SIMD) void tq_wide_compress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t dl) {
     static_assert(DTYPE == TQ_F16 || DTYPE == TQ_BF16, "16-bit inputs");
     using W = Wide<D>;
     constexpr int STEPS = W::STEPS, PIECES = W::PIECES, ROW = W::ROW, THREADS = W::THREADS;
@@ -75,7 +79,21 @@ __global__ __launch_bounds__(Wide<D>::THREADS, Wide<D>::COMPRESS_WAVES_PER_SIMD)
         for (int l = 0; l < 2; ++l) {
             uint32_t v = tl * 32u + ld_vec[l];
             v = v < job.n_vec ? v : job.n_vec - 1u;
-            pre[l] = tq_gload16(job.states + tq_vec_offset(job, v) + ld_piece[l] * 16u);
+            if constexpr (RAGGED) {
+                const TQ_GLOBAL uint8_t *src = (const TQ_GLOBAL uint8_t *)job.states + tq_vec_offset(job, v);
+                const uint32_t e0 = ld_piece[l] * 8u;
+                if (e0 + 8u <= dl && (((uintptr_t)src + 2u * e0) & 15u) == 0u) {      // a whole piece at an aligned address
+                    pre[l] = *reinterpret_cast<const TQ_GLOBAL tq_u4 *>(src + 2u * e0);
+                } else {                                                              // element by element; past the end: zero
+                    tq_u4 q = {0u, 0u, 0u, 0u};
+#pragma unroll
+                    for (uint32_t k = 0; k < 8u; ++k)
+                        if (e0 + k < dl) q[k / 2] |= (uint32_t)*reinterpret_cast<const TQ_GLOBAL uint16_t *>(src + 2u * (e0 + k)) << (16 * (k & 1));
+                    pre[l] = q;
+                }
+            } else {
+                pre[l] = tq_gload16(job.states + tq_vec_offset(job, v) + ld_piece[l] * 16u);
+            }
         }
     };
     issue_loads(blockIdx.x);
@@ -107,7 +125,7 @@ __global__ __launch_bounds__(Wide<D>::THREADS, Wide<D>::COMPRESS_WAVES_PER_SIMD)
     uint32_t op_off[STEPS];
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) op_off[s] = n * ROW + (rotated_piece<D>(2u * s + hk, n) << 4);
-    constexpr uint32_t g_bytes = D / IPB;
+    const uint32_t g_bytes = RAGGED ? (dl + IPB - 1u) / IPB : (uint32_t)(D / IPB);      // packed bytes per vector
 
     // iteration j: rotate tile j into acc_new, search tile j-1 from acc_old
     auto iteration = [&](auto rot_tag, auto search_tag, uint32_t j, tq_f16v &acc_new, const tq_f16v &acc_old) {
@@ -146,7 +164,8 @@ __global__ __launch_bounds__(Wide<D>::THREADS, Wide<D>::COMPRESS_WAVES_PER_SIMD)
                     const uint32_t addr = __float_as_uint(fmaf(a, inv_cell, grid_bias)) & TQ_GRID_ADDR_MASK;
                     const tq_u2 cell = *reinterpret_cast<const tq_u2 *>(lds_grid + addr);
                     const float t = fmaf(a, inv, -__uint_as_float(cell[0]));
-                    const uint32_t code = cell[1] + (~__float_as_uint(t) >> 31);          // base + !(rho < threshold)
+                    uint32_t code = cell[1] + (~__float_as_uint(t) >> 31);                // base + !(rho < threshold)
+                    if constexpr (RAGGED) code = 32u * wave + 16u * hk + (uint32_t)c < dl ? code : 0u;
                     const int byte = c / IPB, k = c % IPB;                                // most significant code of a byte first
                     words[byte / 4] |= code << (8 * (byte % 4) + BITS * (IPB - 1 - k));
                 }
@@ -158,7 +177,14 @@ __global__ __launch_bounds__(Wide<D>::THREADS, Wide<D>::COMPRESS_WAVES_PER_SIMD)
             if (v < job.n_vec) {
                 const uint32_t slot = tq_packed_slot(job, v);
                 uint8_t *dst = job.idx_bytes + (size_t)slot * g_bytes + (2u * wave + hk) * NB;
-                if constexpr (NB == 2) tq_gstore2(reinterpret_cast<uint16_t *>(dst), (uint16_t)words[0]);
+                bool bytewise = false;
+                if constexpr (RAGGED) bytewise = (2u * wave + hk) * NB + NB > g_bytes || ((uintptr_t)dst & (uintptr_t)(NB - 1));
+                if (bytewise) {
+#pragma unroll
+                    for (int b = 0; b < NB; ++b)
+                        if ((2u * wave + hk) * NB + (uint32_t)b < g_bytes)
+                            *((TQ_GLOBAL uint8_t *)dst + b) = (uint8_t)(words[b / 4] >> (8 * (b % 4)));
+                } else if constexpr (NB == 2) tq_gstore2(reinterpret_cast<uint16_t *>(dst), (uint16_t)words[0]);
                 else if constexpr (NB == 4) *reinterpret_cast<TQ_GLOBAL uint32_t *>((TQ_GLOBAL uint8_t *)dst) = words[0];
                 else if constexpr (NB == 8) { const tq_u2 o = {words[0], words[1]}; tq_gstore8(dst, o); }
                 else { const tq_u4 o = {words[0], words[1], words[2], words[3]}; tq_gstore16(dst, o); }
@@ -201,8 +227,8 @@ __global__ __launch_bounds__(Wide<D>::THREADS, Wide<D>::COMPRESS_WAVES_PER_SIMD)
 // one tile ahead (every thread the bytes of 16 codes), turned into fp16 centroids through the byte -> centroids table and
 // parked in a double-buffered LDS tile that all waves read as B operands; the scaled, rounded results go through a
 // second LDS tile so that the stores are D*2 contiguous bytes per vector.
-template <int DTYPE, int IPB, int D>
-__global__ __launch_bounds__(Wide<D>::THREADS) void tq_wide_decompress_kernel(TqDevJob job0, const tq_job *jobs) {
+template <int DTYPE, int IPB, int D, bool RAGGED>
+__global__ __launch_bounds__(Wide<D>::THREADS) void tq_wide_decompress_kernel(TqDevJob job0, const tq_job *jobs, uint32_t dl) {
     static_assert(DTYPE == TQ_F16 || DTYPE == TQ_BF16, "16-bit outputs");
     using W = Wide<D>;
     constexpr int STEPS = W::STEPS, PIECES = W::PIECES, ROW = W::ROW, THREADS = W::THREADS, WAVES = W::WAVES;
@@ -223,7 +249,7 @@ __global__ __launch_bounds__(Wide<D>::THREADS) void tq_wide_decompress_kernel(Tq
     const uint32_t n_tiles = (job.n_vec + 31u) / 32u;
     if (blockIdx.x >= n_tiles) return;
     const TqTableHeader *hd = reinterpret_cast<const TqTableHeader *>(job.table);
-    constexpr uint32_t g_bytes = D / IPB;
+    const uint32_t g_bytes = RAGGED ? (dl + IPB - 1u) / IPB : (uint32_t)(D / IPB);      // packed bytes per vector in memory
 
     // a thread's share of a tile: codes [16 c, 16 c + 16) of vector dv, c = tid % (2 WAVES)
     const uint32_t dv = tid / (2u * WAVES), chunk = tid % (2u * WAVES);
@@ -234,7 +260,15 @@ __global__ __launch_bounds__(Wide<D>::THREADS) void tq_wide_decompress_kernel(Tq
         v = v < job.n_vec ? v : job.n_vec - 1u;
         const uint32_t slot = tq_packed_slot(job, v);
         const uint8_t *src = job.idx_bytes + (size_t)slot * g_bytes + chunk * RAW;
-        if constexpr (RAW == 2) raw[0] = tq_gload2(reinterpret_cast<const uint16_t *>(src));
+        bool bytewise = false;
+        if constexpr (RAGGED) bytewise = chunk * RAW + RAW > g_bytes || ((uintptr_t)src & (uintptr_t)(RAW - 1));
+        if (bytewise) {     // byte by byte; past the vector's last byte: zero (never decoded)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) raw[q] = 0u;
+#pragma unroll
+            for (int b = 0; b < RAW; ++b)
+                if (chunk * RAW + (uint32_t)b < g_bytes) raw[b / 4] |= (uint32_t)*((const TQ_GLOBAL uint8_t *)src + b) << (8 * (b % 4));
+        } else if constexpr (RAW == 2) raw[0] = tq_gload2(reinterpret_cast<const uint16_t *>(src));
         else if constexpr (RAW == 4) raw[0] = *reinterpret_cast<const TQ_GLOBAL uint32_t *>((const TQ_GLOBAL uint8_t *)src);
         else if constexpr (RAW == 8) { const tq_u2 t = tq_gload8(src); raw[0] = t[0]; raw[1] = t[1]; }
         else { const tq_u4 t = tq_gload16(src); raw[0] = t[0]; raw[1] = t[1]; raw[2] = t[2]; raw[3] = t[3]; }
@@ -271,6 +305,11 @@ __global__ __launch_bounds__(Wide<D>::THREADS) void tq_wide_decompress_kernel(Tq
                 const tq_u4 c = *reinterpret_cast<const tq_u4 *>(e);
                 h[4 * byte] = c[0]; h[4 * byte + 1] = c[1]; h[4 * byte + 2] = c[2]; h[4 * byte + 3] = c[3];
             }
+        }
+        if constexpr (RAGGED) {     // coordinates the vector does not have contribute nothing
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                if (16u * chunk + (uint32_t)k >= dl) h[k / 2] &= (k & 1) ? 0x0000ffffu : 0xffff0000u;
         }
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
@@ -329,7 +368,19 @@ __global__ __launch_bounds__(Wide<D>::THREADS) void tq_wide_decompress_kernel(Tq
         for (int k = 0; k < 2; ++k) {
             const tq_u4 val = *reinterpret_cast<const tq_u4 *>(lds_out + st_off[k]);
             const uint32_t v = tl * 32u + st_vec[k];
-            if (v < job.n_vec) tq_gstore16_stream(out_base + tq_vec_offset(job, v) + st_piece[k] * 16u, val);
+            if (v >= job.n_vec) continue;
+            uint8_t *dst = out_base + tq_vec_offset(job, v) + st_piece[k] * 16u;
+            if constexpr (RAGGED) {
+                const uint32_t e0 = st_piece[k] * 8u;
+                if (e0 >= dl) continue;
+                if (e0 + 8u > dl || ((uintptr_t)dst & 15u)) {       // element by element
+#pragma unroll
+                    for (uint32_t e = 0; e < 8u; ++e)
+                        if (e0 + e < dl) *reinterpret_cast<TQ_GLOBAL uint16_t *>((TQ_GLOBAL uint8_t *)dst + 2u * e) = (uint16_t)(val[e / 2] >> (16 * (e & 1)));
+                    continue;
+                }
+            }
+            tq_gstore16_stream(dst, val);
         }
         if (j + 1u < m) decode((j + 1u) & 1u);
     }
@@ -344,7 +395,7 @@ std::mutex host_state_mutex;
 // runtime says fit (remembered per device in `slots`).
 template <typename K>
 int launch(K kernel, int (&slots)[MAX_DEVICES], uint32_t lds, uint32_t threads, const TqDevJob &job, const tq_job *jobs_dev,
-           int n_jobs, uint32_t max_vec, hipStream_t stream) {
+           int n_jobs, uint32_t max_vec, uint32_t dl, hipStream_t stream) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
@@ -366,60 +417,70 @@ int launch(K kernel, int (&slots)[MAX_DEVICES], uint32_t lds, uint32_t threads, 
     }
     const uint32_t tiles = (max_vec + 31u) / 32u;
     const uint32_t bx = tq_blocks_per_job(tiles, resident, n_jobs);
-    hipLaunchKernelGGL(kernel, dim3(bx, (unsigned)n_jobs, 1), dim3(threads, 1, 1), lds, stream, job, jobs_dev);
+    hipLaunchKernelGGL(kernel, dim3(bx, (unsigned)n_jobs, 1), dim3(threads, 1, 1), lds, stream, job, jobs_dev, dl);
     return (int)hipGetLastError();
 }
 
 template <int DTYPE, int BITS, int D>
-int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, hipStream_t s) {
+int launch_compress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t dl, hipStream_t s) {
+    if (dl != (uint32_t)D) {
+        static int slots_ragged[MAX_DEVICES] = {};
+        return launch(&tq_wide_compress_kernel<DTYPE, BITS, D, true>, slots_ragged, Wide<D>::COMPRESS_LDS, Wide<D>::THREADS, job, jobs_dev, n_jobs, max_vec, dl, s);
+    }
     static int slots[MAX_DEVICES] = {};
-    return launch(&tq_wide_compress_kernel<DTYPE, BITS, D>, slots, Wide<D>::COMPRESS_LDS, Wide<D>::THREADS, job, jobs_dev, n_jobs, max_vec, s);
+    return launch(&tq_wide_compress_kernel<DTYPE, BITS, D, false>, slots, Wide<D>::COMPRESS_LDS, Wide<D>::THREADS, job, jobs_dev, n_jobs, max_vec, dl, s);
 }
 template <int DTYPE, int D>
-int compress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, hipStream_t s) {
+int compress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t dl, hipStream_t s) {
     switch (bits) {
-        case 1: return launch_compress<DTYPE, 1, D>(job, jobs_dev, n_jobs, max_vec, s);
-        case 2: return launch_compress<DTYPE, 2, D>(job, jobs_dev, n_jobs, max_vec, s);
-        case 3: return launch_compress<DTYPE, 3, D>(job, jobs_dev, n_jobs, max_vec, s);
-        case 4: return launch_compress<DTYPE, 4, D>(job, jobs_dev, n_jobs, max_vec, s);
+        case 1: return launch_compress<DTYPE, 1, D>(job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 2: return launch_compress<DTYPE, 2, D>(job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 3: return launch_compress<DTYPE, 3, D>(job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 4: return launch_compress<DTYPE, 4, D>(job, jobs_dev, n_jobs, max_vec, dl, s);
         case 5: case 6: case 7: case 8:  // one code per byte: identical packing
-            return launch_compress<DTYPE, 8, D>(job, jobs_dev, n_jobs, max_vec, s);
+            return launch_compress<DTYPE, 8, D>(job, jobs_dev, n_jobs, max_vec, dl, s);
         default: return TQ_ERR_BITS;
     }
 }
 template <int DTYPE>
 int compress_dim(int head_dim, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, hipStream_t s) {
-    switch (head_dim) {
-        case 96: return compress_bits<DTYPE, 96>(bits, job, jobs_dev, n_jobs, max_vec, s);
-        case 160: return compress_bits<DTYPE, 160>(bits, job, jobs_dev, n_jobs, max_vec, s);
-        case 192: return compress_bits<DTYPE, 192>(bits, job, jobs_dev, n_jobs, max_vec, s);
-        case 224: return compress_bits<DTYPE, 224>(bits, job, jobs_dev, n_jobs, max_vec, s);
+    const uint32_t dl = (uint32_t)head_dim;
+    switch (TQ_PADDED_DIM(head_dim)) {
+        case 96: return compress_bits<DTYPE, 96>(bits, job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 160: return compress_bits<DTYPE, 160>(bits, job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 192: return compress_bits<DTYPE, 192>(bits, job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 224: return compress_bits<DTYPE, 224>(bits, job, jobs_dev, n_jobs, max_vec, dl, s);
         default: return TQ_ERR_HEAD_DIM;
     }
 }
 
 template <int DTYPE, int IPB, int D>
-int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, hipStream_t s) {
+int launch_decompress(const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t dl, hipStream_t s) {
+    if (dl != (uint32_t)D) {
+        static int slots_ragged[MAX_DEVICES] = {};
+        return launch(&tq_wide_decompress_kernel<DTYPE, IPB, D, true>, slots_ragged, Wide<D>::DECOMPRESS_LDS, Wide<D>::THREADS, job, jobs_dev, n_jobs, max_vec, dl, s);
+    }
     static int slots[MAX_DEVICES] = {};
-    return launch(&tq_wide_decompress_kernel<DTYPE, IPB, D>, slots, Wide<D>::DECOMPRESS_LDS, Wide<D>::THREADS, job, jobs_dev, n_jobs, max_vec, s);
+    return launch(&tq_wide_decompress_kernel<DTYPE, IPB, D, false>, slots, Wide<D>::DECOMPRESS_LDS, Wide<D>::THREADS, job, jobs_dev, n_jobs, max_vec, dl, s);
 }
 template <int DTYPE, int D>
-int decompress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, hipStream_t s) {
+int decompress_bits(int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, uint32_t dl, hipStream_t s) {
     switch (8 / bits) {
-        case 8: return launch_decompress<DTYPE, 8, D>(job, jobs_dev, n_jobs, max_vec, s);
-        case 4: return launch_decompress<DTYPE, 4, D>(job, jobs_dev, n_jobs, max_vec, s);
-        case 2: return launch_decompress<DTYPE, 2, D>(job, jobs_dev, n_jobs, max_vec, s);
-        case 1: return launch_decompress<DTYPE, 1, D>(job, jobs_dev, n_jobs, max_vec, s);
+        case 8: return launch_decompress<DTYPE, 8, D>(job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 4: return launch_decompress<DTYPE, 4, D>(job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 2: return launch_decompress<DTYPE, 2, D>(job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 1: return launch_decompress<DTYPE, 1, D>(job, jobs_dev, n_jobs, max_vec, dl, s);
         default: return TQ_ERR_BITS;
     }
 }
 template <int DTYPE>
 int decompress_dim(int head_dim, int bits, const TqDevJob &job, const tq_job *jobs_dev, int n_jobs, uint32_t max_vec, hipStream_t s) {
-    switch (head_dim) {
-        case 96: return decompress_bits<DTYPE, 96>(bits, job, jobs_dev, n_jobs, max_vec, s);
-        case 160: return decompress_bits<DTYPE, 160>(bits, job, jobs_dev, n_jobs, max_vec, s);
-        case 192: return decompress_bits<DTYPE, 192>(bits, job, jobs_dev, n_jobs, max_vec, s);
-        case 224: return decompress_bits<DTYPE, 224>(bits, job, jobs_dev, n_jobs, max_vec, s);
+    const uint32_t dl = (uint32_t)head_dim;
+    switch (TQ_PADDED_DIM(head_dim)) {
+        case 96: return decompress_bits<DTYPE, 96>(bits, job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 160: return decompress_bits<DTYPE, 160>(bits, job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 192: return decompress_bits<DTYPE, 192>(bits, job, jobs_dev, n_jobs, max_vec, dl, s);
+        case 224: return decompress_bits<DTYPE, 224>(bits, job, jobs_dev, n_jobs, max_vec, dl, s);
         default: return TQ_ERR_HEAD_DIM;
     }
 }
@@ -427,7 +488,8 @@ int decompress_dim(int head_dim, int bits, const TqDevJob &job, const tq_job *jo
 }  // namespace
 
 bool tq_wide_supported(int head_dim, int dtype) {
-    return (dtype == TQ_F16 || dtype == TQ_BF16) && (head_dim == 96 || head_dim == 160 || head_dim == 192 || head_dim == 224);
+    const int padded = TQ_PADDED_DIM(head_dim);      // 65 ... 96, 129 ... 224
+    return (dtype == TQ_F16 || dtype == TQ_BF16) && head_dim >= 8 && (padded == 96 || padded == 160 || padded == 192 || padded == 224);
 }
 
 int tq_wide_compress(int dtype, int bits, int head_dim, const TqDevJob &single, const tq_job *jobs_dev, int n_jobs,
