@@ -188,11 +188,13 @@ def test_edge_inputs(pkg, oracle):
     assert torch.equal(one["idx_bytes"], out["idx_bytes"][:, :, 1:2])
 
 
-def test_strided_store_and_batched_jobs(pkg, oracle):
+@pytest.mark.parametrize("D", [256, 96, 192, 32])
+def test_strided_store_and_batched_jobs(pkg, oracle, D):
     """Token-axis slices of a preallocated [B,H,capacity,..] store, and a job list of several tensors in one launch,
-    give the bytes of plain calls."""
+    give the bytes of plain calls (256: the kernels of that width; 96, 192: the kernels templated on the dimension; 32:
+    the run-time-dimension kernels)."""
     native = pkg._native
-    D, bits = 256, 2
+    bits = 2
     comp = pkg.MSECompressor(D, bits, seed=3, device=DEV)
     B, H, cap = 2, 2, 300
     x = outlier_kv((B, H, 140, D), seed=5, dtype=torch.bfloat16).to(DEV)
