@@ -686,14 +686,19 @@ __global__ __launch_bounds__(256, 2) void tq_d256_decompress_kernel(TqDevJob job
                 h[4 * byte] = c[0]; h[4 * byte + 1] = c[1]; h[4 * byte + 2] = c[2]; h[4 * byte + 3] = c[3];
             }
         }
+        // piece p = 4 chunk + q of a row sits at position ((q << 3) | chunk) ^ (row & 31): the eight threads that decode one
+        // row write eight different bank groups at a time (with the pieces in place they would hit two), and the eight
+        // rows an operand read touches still differ in the low three bits
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const tq_u4 o = {h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3]};
-            *reinterpret_cast<tq_u4 *>(lds_y[b] + dv * (D * 2) + (((4u * chunk + q) ^ (dv & 31u)) << 4)) = o;
+            *reinterpret_cast<tq_u4 *>(lds_y[b] + dv * (D * 2) + (((((uint32_t)q << 3) | chunk) ^ (dv & 31u)) << 4)) = o;
         }
         if (chunk == 0u) lds_norm[b][dv] = (float)__builtin_bit_cast(_Float16, norm_bits);
     };
-    const uint32_t op_base = n * (D * 2) + ((hk ^ (n & 31u)) << 4);     // B operand of step s: at op_base ^ (32 s)
+    // B operand of step s: piece 2 s + hk = 4 (s >> 1) + (2 (s & 1) + hk), i.e. position ((2 (s & 1) + hk) << 3 | s >> 1) ^ (n & 31)
+    const uint32_t op_base = n * (D * 2) + (((hk << 3) ^ (n & 31u)) << 4);
+    auto op_step = [](int s) { return (uint32_t)((((2 * (s & 1)) << 3) | (s >> 1)) << 4); };
 
     const uint32_t m = (n_tiles - blockIdx.x + gridDim.x - 1u) / gridDim.x;
     decode(0u);
@@ -705,7 +710,7 @@ __global__ __launch_bounds__(256, 2) void tq_d256_decompress_kernel(TqDevJob job
         tq_f16v acc[2] = {tq_zero16(), tq_zero16()};
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
-            const tq_u4 b = *reinterpret_cast<const tq_u4 *>(ys + (op_base ^ (32u * s)));
+            const tq_u4 b = *reinterpret_cast<const tq_u4 *>(ys + (op_base ^ op_step(s)));
             acc[0] = mfma_f16(areg[0][s], b, acc[0]);
             acc[1] = mfma_f16(areg[1][s], b, acc[1]);
         }

@@ -285,8 +285,11 @@ __global__ __launch_bounds__(Wide<D>::THREADS) void tq_wide_decompress_kernel(Tq
     tq_copy_to_lds(lds_lut, job.table + hd->off_lut, 256u * ENTRY, tid, (uint32_t)THREADS);
     __syncthreads();
 
-    // the prefetched bytes -> 16 fp16 centroids = pieces 2 chunk, 2 chunk + 1 of row dv of buffer b
-    const uint32_t y_off[2] = {dv * ROW + (rotated_piece<D>(2u * chunk, dv) << 4), dv * ROW + (rotated_piece<D>(2u * chunk + 1u, dv) << 4)};
+    // the prefetched bytes -> 16 fp16 centroids = pieces 2 chunk, 2 chunk + 1 of row dv of buffer b.  In this tile the even
+    // pieces of a row come first and the odd ones after them (piece 2 c + q at index q * PIECES/2 + c, then rotated by the
+    // row like everywhere else): the threads that decode a row write neighbouring bank groups at a time instead of every
+    // second one.
+    const uint32_t y_off[2] = {dv * ROW + (rotated_piece<D>(chunk, dv) << 4), dv * ROW + (rotated_piece<D>(PIECES / 2 + chunk, dv) << 4)};
     auto decode = [&](uint32_t b) {
         uint32_t h[8];          // 16 halves
 #pragma unroll
@@ -318,9 +321,9 @@ __global__ __launch_bounds__(Wide<D>::THREADS) void tq_wide_decompress_kernel(Tq
         }
         if (chunk == 0u) lds_norm[b][dv] = (float)__builtin_bit_cast(_Float16, norm_bits);
     };
-    uint32_t op_off[STEPS];     // B operand of step s: piece 2 s + hk of row n
+    uint32_t op_off[STEPS];     // B operand of step s: piece 2 s + hk of row n, at index hk * PIECES/2 + s
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) op_off[s] = n * ROW + (rotated_piece<D>(2u * s + hk, n) << 4);
+    for (int s = 0; s < STEPS; ++s) op_off[s] = n * ROW + (rotated_piece<D>(hk * (PIECES / 2) + s, n) << 4);
     // lane (n, hk) ends up with elements 32 w + 16 hk + r of vector n: pieces 4 w + 2 hk + c of its output row
     const uint32_t out_off[2] = {n * ROW + (rotated_piece<D>(4u * wave + 2u * hk, n) << 4), n * ROW + (rotated_piece<D>(4u * wave + 2u * hk + 1u, n) << 4)};
     // the stores of a tile: piece i = k * THREADS + tid is piece i % PIECES of vector i / PIECES
